@@ -1,0 +1,234 @@
+/*
+ * dgs_hip.h -- C ABI of libdgs_hip.so: the gfx950 kernels behind the
+ * torch.classes.dgs_classes.ChunkTensor / torch.ops.dgs_ops operator surface.
+ *
+ * Conventions
+ *   - every entry point returns a dgs_status (0 = ok); nothing aborts or throws;
+ *     dgs_last_error() gives a thread-local message for the last failure;
+ *   - all pointers named dev_* / *_dev / out_* are device-accessible addresses
+ *     (HBM, or pinned host memory mapped into the device address space);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); every
+ *     kernel is enqueued there and nothing synchronises unless the name says so;
+ *   - entry points that need temporary device memory take a caller-owned
+ *     workspace whose size the matching *_workspace_bytes() call reports; the
+ *     kernels themselves never allocate;
+ *   - ids are int32 or int64 (`id_bytes` 4 or 8), selected at run time.
+ *
+ * Each declaration cites the reference interface (file:line under the upstream
+ * source tree) whose behaviour it reproduces.
+ */
+#ifndef DGS_HIP_H_
+#define DGS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int dgs_status;
+enum {
+  DGS_OK = 0,
+  DGS_ERR_INVALID = 1,      /* bad argument (null pointer, negative size, width not 4/8 ...) */
+  DGS_ERR_HIP = 2,          /* a HIP runtime call failed */
+  DGS_ERR_WORKSPACE = 3,    /* workspace too small or misaligned */
+  DGS_ERR_UNSUPPORTED = 4,  /* valid request outside what the kernels cover */
+  DGS_ERR_RANGE = 5         /* data-dependent failure reported by a kernel (see each call) */
+};
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* dgs_last_error(void);
+/* Static name of a status code. */
+const char* dgs_status_name(dgs_status s);
+/* ABI version of this header (bumped on incompatible change). */
+int dgs_abi_version(void);
+
+/* ------------------------------------------------------------------------ */
+/* Two-tier positional store (ChunkTensor)                                   */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Device-side view of a store, passed to kernels BY VALUE.
+ * Element i lives at dev[i] when i < threshold, else at host[i - threshold].
+ * Replaces the device-resident accessor struct chunk_tensor_wrapper<T>
+ * (src/chunk_tensor.h:10-59) at world size 1.  A plain device array is the
+ * view {dev = ptr, host = NULL, threshold = total = n}.
+ */
+typedef struct dgs_view {
+  const void* dev;    /* HBM slice: elements [0, threshold)                  */
+  const void* host;   /* device-visible address of the pinned host slice     */
+  int64_t threshold;  /* elements held in HBM                                */
+  int64_t total;      /* elements in the whole store                         */
+  int32_t elem_bytes; /* 1, 2, 4 or 8                                        */
+  int32_t reserved_;
+} dgs_view;
+
+typedef struct dgs_store dgs_store; /* opaque, owns both slices */
+
+/*
+ * Split arithmetic of ChunkTensor::ChunkTensor (src/chunk_tensor.cc:37-73) at
+ * world size 1: device elements = capacity_bytes / elem_bytes clamped to
+ * total_elems; host elements = the rest.  Pure host arithmetic, no GPU needed.
+ */
+dgs_status dgs_store_split(int64_t total_elems, int32_t elem_bytes,
+                           int64_t capacity_bytes, int64_t* device_elems,
+                           int64_t* host_elems);
+
+/*
+ * Allocates the HBM slice (filled with 0xFF bytes, src/chunk_tensor.cc:100-109)
+ * and the pinned, device-mapped host slice (hipHostMalloc; replaces SysV shm +
+ * cudaHostRegister, src/chunk_tensor.cc:76-96) on the current device.
+ */
+dgs_status dgs_store_create(int64_t total_elems, int32_t elem_bytes,
+                            int64_t capacity_bytes, dgs_store** out);
+/* ChunkTensor::_Free (src/chunk_tensor.cc:235-263). NULL is accepted. */
+dgs_status dgs_store_destroy(dgs_store* s);
+/*
+ * ChunkTensor::LoadFromTensor (src/chunk_tensor.cc:173-200): copies
+ * total_elems elements from pageable or pinned HOST memory `src` into the two
+ * slices.  Blocking.
+ */
+dgs_status dgs_store_load(dgs_store* s, const void* src, int64_t n_elems);
+/* Fills *v with the by-value kernel view of the store. */
+dgs_status dgs_store_view(const dgs_store* s, dgs_view* v);
+/*
+ * Raw slices for GetSubDeviceTensor / GetHostTensor (src/chunk_tensor.cc:151-171).
+ * host_cpu_ptr is the CPU address of the pinned slice.
+ */
+dgs_status dgs_store_slices(const dgs_store* s, void** dev_ptr,
+                            int64_t* device_elems, void** host_cpu_ptr,
+                            int64_t* host_elems);
+/*
+ * Bytes of HBM currently held by stores: CUDAContext::GetCurrAllocated
+ * (src/cuda_context.h:13-15, src/cuda_context.cc:5-6).
+ */
+int64_t dgs_current_allocated(void);
+
+/* ------------------------------------------------------------------------ */
+/* Row gather                                                                */
+/* ------------------------------------------------------------------------ */
+
+enum {
+  DGS_TIER_ANY = 0,   /* _CAPI_index:       per-element device/host resolution */
+  DGS_TIER_DEVICE = 1,/* _CAPI_local_index: every row read from the HBM slice  */
+  DGS_TIER_HOST = 2   /* _CAPI_host_index:  every row read from the host slice */
+};
+
+/*
+ * out[i, 0:row_elems] = X[index[i], 0:row_elems] for i in [0, n), X the
+ * row-major [total/row_elems, row_elems] matrix behind `v`.
+ * Replaces IndexFromChunkTensorCUDA / LocalIndex... / HostIndex...
+ * (src/cuda/index_with_chunk_tensor.cu:9-53, :110-128/:170-194, :150-168/:223-247).
+ * A row that straddles the device/host boundary is resolved per element, like
+ * chunk_tensor_wrapper::At (src/chunk_tensor.h:33-42).  `out` holds
+ * n * row_elems elements.  index values are not range-checked.
+ */
+dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
+                           int32_t index_bytes, int64_t n, void* out,
+                           int32_t tier, void* stream);
+
+/*
+ * Stable partition of an index list into (device-resident rows, host-resident
+ * rows): row r is "host" iff r >= threshold / row_elems
+ * (src/cuda/index_with_chunk_tensor.cu:55-108; the "remote" class is empty at
+ * world size 1).  out_local / out_host each hold up to n ids; counts_dev[0..1]
+ * (int64, device) receive the two lengths.
+ */
+size_t dgs_split_index_workspace_bytes(int64_t n);
+dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
+                           int32_t index_bytes, int64_t n, void* out_local,
+                           void* out_host, int64_t* counts_dev, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Row-wise uniform neighbour sampling over CSC                              */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Random-number contract ("dgs-philox-1"), shared bit for bit with the CPU
+ * oracle: draw number j of row r is the Philox4x32-10 block with
+ *   key     = (rng_seed & 0xffffffff, rng_seed >> 32)
+ *   counter = (j, rng_stream, r & 0xffffffff, r >> 32)
+ * reduced to [0, n) by Lemire's multiply-shift with rejection over the block's
+ * four words in order (the fourth word is accepted unconditionally).
+ *   - without replacement, deg > k: Floyd's subset algorithm; step i (0-based)
+ *     draws t in [0, deg-k+i] and keeps t unless an earlier step kept it, in
+ *     which case it keeps deg-k+i; output slot i holds that position;
+ *   - without replacement, deg <= k: the whole row in CSC order;
+ *   - with replacement, deg > 0: slot i holds draw i reduced to [0, deg).
+ */
+
+/*
+ * One hop.  For every seed row (in order) emits its picks contiguously:
+ *   out_rows[e] = seed id, out_cols[e] = picked neighbour id.
+ * Replaces RowWiseSamplingUniformWithChunkTensorCUDA and
+ * RowWiseSamplingUniformCUDA (src/cuda/rowwise_sampling_with_chunk_tensor.cu:113-194,
+ * src/cuda/rowwise_sampling.cu:13-187).
+ *   seeds    : device, n_seeds ids of width id_bytes (also the width of
+ *              out_rows / out_cols and of `indices`)
+ *   indptr   : view of N+1 offsets, elem_bytes 4 or 8
+ *   indices  : view of E ids, elem_bytes == id_bytes
+ *   out_rows, out_cols : device, capacity n_seeds * num_picks ids each
+ *   nnz_dev  : device int64[2]; [0] receives the number of emitted edges,
+ *              [1] a non-zero flag when some row had degree >= 2^32
+ *              (its output is unspecified; report DGS_ERR_RANGE to the user)
+ * Nothing is read back: the caller copies nnz_dev when it needs the length.
+ */
+size_t dgs_sample_workspace_bytes(int64_t n_seeds);
+dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes,
+                                int64_t n_seeds, dgs_view indptr,
+                                dgs_view indices, int64_t num_picks,
+                                int32_t replace, uint64_t rng_seed,
+                                uint32_t rng_stream, void* out_rows,
+                                void* out_cols, int64_t* nnz_dev,
+                                void* workspace, size_t workspace_bytes,
+                                void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Unique + relabel                                                          */
+/* ------------------------------------------------------------------------ */
+
+#define DGS_MAX_SEGMENTS 8
+/* A logical concatenation of up to DGS_MAX_SEGMENTS device arrays of ids. */
+typedef struct dgs_segments {
+  const void* ptr[DGS_MAX_SEGMENTS];
+  int64_t len[DGS_MAX_SEGMENTS];
+  int32_t count;
+  int32_t reserved_;
+} dgs_segments;
+
+/*
+ * unique  = distinct ids of cat(mapping) in first-occurrence order;
+ * out[t][i] = position of requiring[t][i] in unique, or -1 when absent.
+ * Replaces TensorRelabelCUDA / Unique / Relabel / RelabelHashmap
+ * (src/cuda/tensor_reindex.cu:11-205).
+ *   unique_out     : device, capacity sum(mapping.len) ids
+ *   num_unique_dev : device int64[1]
+ *   out            : device arrays, out.len must equal requiring.len
+ * ids must be >= 0 (-1 is the empty-slot marker, as in the reference).
+ * sum(mapping.len) must be < 2^31.
+ */
+size_t dgs_unique_relabel_workspace_bytes(int64_t n_mapping, int32_t id_bytes);
+dgs_status dgs_unique_relabel(dgs_segments mapping, dgs_segments requiring,
+                              int32_t id_bytes, void* unique_out,
+                              int64_t* num_unique_dev, dgs_segments out,
+                              void* workspace, size_t workspace_bytes,
+                              void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Small utilities                                                           */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Copies n_bytes from device memory to `host_dst` on `stream` and waits for the
+ * stream: the blocking length read the reference does after each scan
+ * (src/cuda/rowwise_sampling_with_chunk_tensor.cu:154-156, src/cuda/tensor_reindex.cu:129).
+ */
+dgs_status dgs_read_back(void* host_dst, const void* dev_src, size_t n_bytes,
+                         void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DGS_HIP_H_ */
