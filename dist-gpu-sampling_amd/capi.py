@@ -1,0 +1,199 @@
+"""ctypes binding of the C ABI in include/dgs_hip.h (libdgs_hip.so).
+
+Thin by design: arguments are raw addresses and sizes.  The helpers at the
+bottom accept torch tensors only to take their data_ptr(); torch supplies the
+device memory and the stream, nothing else.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdgs_hip.so")
+
+DGS_OK, DGS_ERR_INVALID, DGS_ERR_HIP, DGS_ERR_WORKSPACE, DGS_ERR_UNSUPPORTED, DGS_ERR_RANGE = range(6)
+TIER_ANY, TIER_DEVICE, TIER_HOST = 0, 1, 2
+MAX_SEGMENTS = 8
+
+c_i64, c_i32, c_u64, c_u32, c_vp, c_sz = (ctypes.c_int64, ctypes.c_int32, ctypes.c_uint64, ctypes.c_uint32,
+                                          ctypes.c_void_p, ctypes.c_size_t)
+
+
+class View(ctypes.Structure):
+    """dgs_view"""
+    _fields_ = [("dev", c_vp), ("host", c_vp), ("threshold", c_i64), ("total", c_i64),
+                ("elem_bytes", c_i32), ("reserved_", c_i32)]
+
+
+class Segments(ctypes.Structure):
+    """dgs_segments"""
+    _fields_ = [("ptr", c_vp * MAX_SEGMENTS), ("len", c_i64 * MAX_SEGMENTS), ("count", c_i32),
+                ("reserved_", c_i32)]
+
+
+# name -> (restype, argtypes); must list every function include/dgs_hip.h declares
+SIGNATURES = {
+    "dgs_last_error": (ctypes.c_char_p, []),
+    "dgs_status_name": (ctypes.c_char_p, [ctypes.c_int]),
+    "dgs_abi_version": (ctypes.c_int, []),
+    "dgs_store_split": (ctypes.c_int, [c_i64, c_i32, c_i64, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)]),
+    "dgs_store_create": (ctypes.c_int, [c_i64, c_i32, c_i64, ctypes.POINTER(c_vp)]),
+    "dgs_store_destroy": (ctypes.c_int, [c_vp]),
+    "dgs_store_load": (ctypes.c_int, [c_vp, c_vp, c_i64]),
+    "dgs_store_view": (ctypes.c_int, [c_vp, ctypes.POINTER(View)]),
+    "dgs_store_slices": (ctypes.c_int, [c_vp, ctypes.POINTER(c_vp), ctypes.POINTER(c_i64),
+                                        ctypes.POINTER(c_vp), ctypes.POINTER(c_i64)]),
+    "dgs_current_allocated": (c_i64, []),
+    "dgs_gather_rows": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i32, c_vp]),
+    "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
+    "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_workspace_bytes": (c_sz, [c_i64]),
+    "dgs_sample_count": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_fill": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_u64, c_u32, c_vp, c_vp,
+                                       c_vp, c_sz, c_vp]),
+    "dgs_sample_neighbors": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32,
+                                            c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_unique_relabel_workspace_bytes": (c_sz, [c_i64, c_i32]),
+    "dgs_unique_relabel": (ctypes.c_int, [Segments, Segments, c_i32, c_vp, c_vp, Segments, c_vp, c_sz, c_vp]),
+    "dgs_read_back": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp]),
+}
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(f"{LIB_PATH} is missing; build it with dist-gpu-sampling_amd/build.py")
+lib = ctypes.CDLL(LIB_PATH)
+for _name, (_res, _args) in SIGNATURES.items():
+    _f = getattr(lib, _name)
+    _f.restype = _res
+    _f.argtypes = _args
+
+
+class DgsError(RuntimeError):
+    def __init__(self, status):
+        self.status = status
+        super().__init__(f"{lib.dgs_status_name(status).decode()}: {lib.dgs_last_error().decode()}")
+
+
+def check(status):
+    if status != DGS_OK:
+        raise DgsError(status)
+
+
+# ---- helpers over torch tensors (addresses only) --------------------------------
+def stream_ptr():
+    return c_vp(torch.cuda.current_stream().cuda_stream)
+
+
+def tensor_view(t):
+    """A plain device array as a single-tier view."""
+    assert t.is_contiguous()
+    return View(t.data_ptr(), None, t.numel(), t.numel(), t.element_size(), 0)
+
+
+def segments(tensors):
+    s = Segments()
+    s.count = len(tensors)
+    for i, t in enumerate(tensors):
+        assert t.is_contiguous()
+        s.ptr[i] = t.data_ptr()
+        s.len[i] = t.numel()
+    return s
+
+
+class Store:
+    """Owner of a dgs_store (two-tier ChunkTensor storage)."""
+
+    def __init__(self, total_elems, elem_bytes, capacity_bytes):
+        h = c_vp()
+        check(lib.dgs_store_create(total_elems, elem_bytes, capacity_bytes, ctypes.byref(h)))
+        self.handle = h
+        self.view = View()
+        check(lib.dgs_store_view(self.handle, ctypes.byref(self.view)))
+
+    def load(self, cpu_tensor):
+        assert cpu_tensor.device.type == "cpu" and cpu_tensor.is_contiguous()
+        check(lib.dgs_store_load(self.handle, cpu_tensor.data_ptr(), cpu_tensor.numel()))
+
+    def close(self):
+        if self.handle is not None:
+            check(lib.dgs_store_destroy(self.handle))
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _ws(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def read_i64(dev_tensor, count):
+    host = torch.empty(count, dtype=torch.int64).pin_memory()
+    check(lib.dgs_read_back(host.data_ptr(), dev_tensor.data_ptr(), 8 * count, stream_ptr()))
+    return host.tolist()
+
+
+def gather_rows(view, row_elems, index, dtype, tier=TIER_ANY):
+    n = index.numel()
+    out = torch.empty((n, row_elems), dtype=dtype, device=index.device)
+    check(lib.dgs_gather_rows(view, row_elems, index.data_ptr(), index.element_size(), n, out.data_ptr(), tier,
+                              stream_ptr()))
+    return out
+
+
+def split_index(view, row_elems, index):
+    n = index.numel()
+    local = torch.empty_like(index)
+    host = torch.empty_like(index)
+    counts = torch.empty(2, dtype=torch.int64, device=index.device)
+    nb = lib.dgs_split_index_workspace_bytes(n)
+    ws = _ws(nb, index.device)
+    check(lib.dgs_split_index(view, row_elems, index.data_ptr(), index.element_size(), n, local.data_ptr(),
+                              host.data_ptr(), counts.data_ptr(), ws.data_ptr(), nb, stream_ptr()))
+    c = read_i64(counts, 2)
+    return local[:c[0]], host[:c[1]]
+
+
+def sample_neighbors(seeds, indptr_view, indices_view, num_picks, replace, rng_seed, rng_stream, two_step=False):
+    """Returns (coo_row, coo_col, flags)."""
+    n = seeds.numel()
+    nb = lib.dgs_sample_workspace_bytes(n)
+    ws = _ws(nb, seeds.device)
+    nnz = torch.empty(2, dtype=torch.int64, device=seeds.device)
+    w = seeds.element_size()
+    if two_step:
+        check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
+                                   ws.data_ptr(), nb, stream_ptr()))
+        cnt, flags = read_i64(nnz, 2)
+        rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
+        cols = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
+        check(lib.dgs_sample_fill(seeds.data_ptr(), w, n, indices_view, num_picks, int(replace), rng_seed,
+                                  rng_stream, rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), nb, stream_ptr()))
+        return rows, cols, flags
+    rows = torch.empty(n * num_picks, dtype=seeds.dtype, device=seeds.device)
+    cols = torch.empty(n * num_picks, dtype=seeds.dtype, device=seeds.device)
+    check(lib.dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr_view, indices_view, num_picks, int(replace),
+                                   rng_seed, rng_stream, rows.data_ptr(), cols.data_ptr(), nnz.data_ptr(),
+                                   ws.data_ptr(), nb, stream_ptr()))
+    cnt, flags = read_i64(nnz, 2)
+    return rows[:cnt], cols[:cnt], flags
+
+
+def unique_relabel(mapping, requiring):
+    """Returns (unique, [relabelled ...])."""
+    dev = mapping[0].device
+    dt = mapping[0].dtype
+    n = sum(t.numel() for t in mapping)
+    unique = torch.empty(n, dtype=dt, device=dev)
+    outs = [torch.empty_like(t) for t in requiring]
+    num = torch.empty(1, dtype=torch.int64, device=dev)
+    w = mapping[0].element_size()
+    nb = lib.dgs_unique_relabel_workspace_bytes(n, w)
+    ws = _ws(nb, dev)
+    check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, unique.data_ptr(), num.data_ptr(),
+                                 segments(outs), ws.data_ptr(), nb, stream_ptr()))
+    u = read_i64(num, 1)[0]
+    return unique[:u], outs

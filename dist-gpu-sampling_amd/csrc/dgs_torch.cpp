@@ -1,0 +1,389 @@
+// libdgs.so: the torch-facing layer.  It registers the operator surface of the
+// upstream library (src/pybind.cc:11-38) -- torch.classes.dgs_classes.ChunkTensor
+// and the torch.ops.dgs_ops free functions on the sampling / relabel / gather
+// path -- and does nothing but validate arguments, allocate outputs and
+// workspaces with torch, and call the C ABI of libdgs_hip.so on torch's current
+// HIP stream.  There is no CPU implementation behind these operators: without
+// the HIP library the shared object does not load.
+//
+// Deliberate differences from upstream, all on the safe side:
+//   - argument violations raise (TORCH_CHECK) where upstream aborts the process
+//     (CHECK / LOG(FATAL) / exit in src/chunk_tensor.cc:39-40,174-181,
+//     src/dgs_headers.h:33-45);
+//   - world size is 1: _CAPI_get_unique_id / _CAPI_set_nccl are inert shims and
+//     _CAPI_remote_index returns an empty [0, D] tensor;
+//   - seeds/indices share one id width but indptr may have the other one;
+//   - the store accepts every dtype of 1, 2, 4 or 8 bytes (upstream: i32, i64,
+//     f32 only, src/dgs_headers.h:60-74);
+//   - random picks come from a counter-based generator whose (seed, stream) is
+//     settable; upstream re-seeds the constant 7777 on every call
+//     (src/cuda/rowwise_sampling_with_chunk_tensor.cu:162).
+#include <c10/hip/HIPStream.h>
+#include <torch/custom_class.h>
+#include <torch/script.h>
+
+#include <atomic>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#include "dgs_hip.h"
+
+namespace dgs {
+namespace {
+
+void check(dgs_status s) {
+  TORCH_CHECK(s == DGS_OK, "dgs: ", dgs_status_name(s), ": ", dgs_last_error());
+}
+
+void* current_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+#define DGS_CHECK_GPU(x) TORCH_CHECK((x).device().is_cuda(), #x " must be a GPU tensor")
+
+int32_t id_width(const torch::Tensor& t, const char* what) {
+  TORCH_CHECK(t.scalar_type() == torch::kInt32 || t.scalar_type() == torch::kInt64, what,
+              " must be int32 or int64, got ", t.scalar_type());
+  return t.scalar_type() == torch::kInt64 ? 8 : 4;
+}
+
+torch::Tensor device_bytes(size_t n, const torch::Device& dev) {
+  // torch's caching allocator hands out 512-byte aligned blocks
+  return torch::empty({static_cast<int64_t>(n)}, torch::TensorOptions().dtype(torch::kUInt8).device(dev));
+}
+
+// Blocking read of a few int64 values from the device through a pinned buffer.
+std::vector<int64_t> read_back(const torch::Tensor& dev, int64_t count) {
+  thread_local torch::Tensor pinned =
+      torch::empty({16}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+  TORCH_CHECK(count <= 16);
+  check(dgs_read_back(pinned.data_ptr(), dev.data_ptr(), sizeof(int64_t) * count, current_stream()));
+  const int64_t* p = pinned.data_ptr<int64_t>();
+  return std::vector<int64_t>(p, p + count);
+}
+
+// ---- generator state for the sampling ops ------------------------------------
+std::mutex g_rng_mutex;
+uint64_t g_rng_seed = 7777;  // upstream's constant, used until the caller sets one
+uint32_t g_rng_stream = 0;   // advanced by one per sampling call
+
+std::pair<uint64_t, uint32_t> next_rng() {
+  std::lock_guard<std::mutex> lock(g_rng_mutex);
+  return {g_rng_seed, g_rng_stream++};
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------
+// ChunkTensor (upstream src/chunk_tensor.h:61-106)
+// ---------------------------------------------------------------------------------
+class ChunkTensor : public torch::CustomClassHolder {
+ public:
+  ChunkTensor(std::vector<int64_t> shapes, torch::ScalarType dtype, int64_t capacity_per_gpu)
+      : shapes_(std::move(shapes)), dtype_(dtype) {
+    TORCH_CHECK(shapes_.size() == 1 || shapes_.size() == 2, "ChunkTensor: shapes must have 1 or 2 entries, got ",
+                shapes_.size());
+    TORCH_CHECK(capacity_per_gpu >= 0, "ChunkTensor: capacity_per_gpu must be >= 0, got ", capacity_per_gpu);
+    strides_.resize(shapes_.size());
+    int64_t stride = 1;
+    for (int i = static_cast<int>(shapes_.size()) - 1; i >= 0; --i) {
+      TORCH_CHECK(shapes_[i] >= 0, "ChunkTensor: negative extent");
+      strides_[i] = stride;
+      stride *= shapes_[i];
+    }
+    elem_stride_ = strides_[0];
+    total_ = stride;
+    const size_t eb = c10::elementSize(dtype_);
+    TORCH_CHECK(eb == 1 || eb == 2 || eb == 4 || eb == 8, "ChunkTensor: unsupported dtype ", dtype_);
+    check(dgs_store_create(total_, static_cast<int32_t>(eb), capacity_per_gpu, &store_));
+    check(dgs_store_view(store_, &view_));
+    // torch on ROCm names its GPU device type CUDA; only the index comes from the HIP stream
+    device_ = c10::Device(c10::DeviceType::CUDA, c10::hip::getCurrentHIPStream().device_index());
+  }
+  ~ChunkTensor() override { dgs_store_destroy(store_); }
+
+  // upstream GetHostTensor (src/chunk_tensor.cc:151-160): flat, non-owning
+  torch::Tensor GetHostTensor() {
+    void* p = nullptr;
+    int64_t n = 0;
+    check(dgs_store_slices(store_, nullptr, nullptr, &p, &n));
+    auto opt = torch::TensorOptions().device(torch::kCPU).dtype(dtype_);
+    return n > 0 ? torch::from_blob(p, {n}, opt) : torch::empty({0}, opt);
+  }
+
+  // upstream GetSubDeviceTensor (src/chunk_tensor.cc:162-171): flat, non-owning
+  torch::Tensor GetSubDeviceTensor() {
+    void* p = nullptr;
+    int64_t n = 0;
+    check(dgs_store_slices(store_, &p, &n, nullptr, nullptr));
+    auto opt = torch::TensorOptions().device(device_).dtype(dtype_);
+    return n > 0 ? torch::from_blob(p, {n}, opt) : torch::empty({0}, opt);
+  }
+
+  // upstream LoadFromTensor (src/chunk_tensor.cc:173-200)
+  void LoadFromTensor(torch::Tensor data) {
+    TORCH_CHECK(static_cast<size_t>(data.dim()) == shapes_.size(), "load_from_tensor: expected ", shapes_.size(),
+                " dimensions, got ", data.dim());
+    TORCH_CHECK(data.scalar_type() == dtype_, "load_from_tensor: expected dtype ", dtype_, ", got ",
+                data.scalar_type());
+    TORCH_CHECK(data.device().is_cpu(), "load_from_tensor: data must be a CPU tensor");
+    for (size_t i = 0; i < shapes_.size(); ++i) {
+      TORCH_CHECK(data.size(i) == shapes_[i], "load_from_tensor: extent ", i, " is ", data.size(i), ", expected ",
+                  shapes_[i]);
+      TORCH_CHECK(data.size(i) <= 1 || data.stride(i) == strides_[i], "load_from_tensor: data must be contiguous");
+    }
+    check(dgs_store_load(store_, data.data_ptr(), total_));
+  }
+
+  torch::Tensor Gather(const torch::Tensor& index_in, int32_t tier) const {
+    DGS_CHECK_GPU(index_in);
+    const int32_t w = id_width(index_in, "index");
+    torch::Tensor index = index_in.contiguous();
+    const int64_t n = index.numel();
+    torch::Tensor out = torch::empty({n, elem_stride_}, torch::TensorOptions().dtype(dtype_).device(index.device()));
+    check(dgs_gather_rows(view_, elem_stride_, index.data_ptr(), w, n, out.data_ptr(), tier, current_stream()));
+    return out;
+  }
+  // upstream Index / LocalIndex / RemoteIndex / HostIndex (src/chunk_tensor.cc:207-221)
+  torch::Tensor Index(torch::Tensor index) { return Gather(index, DGS_TIER_ANY); }
+  torch::Tensor LocalIndex(torch::Tensor index) { return Gather(index, DGS_TIER_DEVICE); }
+  torch::Tensor HostIndex(torch::Tensor index) { return Gather(index, DGS_TIER_HOST); }
+  torch::Tensor RemoteIndex(torch::Tensor index) {
+    DGS_CHECK_GPU(index);
+    TORCH_CHECK(index.numel() == 0, "_CAPI_remote_index: there is no peer tier at world size 1, but ", index.numel(),
+                " rows were requested");
+    return torch::empty({0, elem_stride_}, torch::TensorOptions().dtype(dtype_).device(index.device()));
+  }
+
+  // upstream SplitIndex (src/chunk_tensor.cc:202-205)
+  std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> SplitIndex(torch::Tensor index_in) {
+    DGS_CHECK_GPU(index_in);
+    const int32_t w = id_width(index_in, "index");
+    torch::Tensor index = index_in.contiguous().view({-1});
+    const int64_t n = index.numel();
+    torch::Tensor local = torch::empty_like(index);
+    torch::Tensor host = torch::empty_like(index);
+    torch::Tensor counts = torch::empty({2}, index.options().dtype(torch::kInt64));
+    const size_t ws_bytes = dgs_split_index_workspace_bytes(n);
+    torch::Tensor ws = device_bytes(ws_bytes, index.device());
+    check(dgs_split_index(view_, elem_stride_, index.data_ptr(), w, n, local.data_ptr(), host.data_ptr(),
+                          counts.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, current_stream()));
+    const std::vector<int64_t> c = read_back(counts, 2);
+    return std::make_tuple(local.narrow(0, 0, c[0]), torch::empty({0}, index.options()), host.narrow(0, 0, c[1]));
+  }
+
+  const dgs_view& view() const { return view_; }
+  torch::ScalarType dtype() const { return dtype_; }
+
+ private:
+  std::vector<int64_t> shapes_;
+  std::vector<int64_t> strides_;
+  torch::ScalarType dtype_;
+  int64_t elem_stride_ = 1;
+  int64_t total_ = 0;
+  dgs_store* store_ = nullptr;
+  dgs_view view_{};
+  c10::Device device_{c10::DeviceType::CUDA, 0};
+};
+
+namespace {
+
+dgs_view tensor_view(const torch::Tensor& t) {
+  dgs_view v{};
+  v.dev = t.data_ptr();
+  v.host = nullptr;
+  v.threshold = t.numel();
+  v.total = t.numel();
+  v.elem_bytes = static_cast<int32_t>(t.element_size());
+  return v;
+}
+
+// Shared body of the two sampling operators.
+std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_in, const dgs_view& indptr,
+                                                     const dgs_view& indices, torch::ScalarType indices_dtype,
+                                                     int64_t num_picks, bool replace) {
+  DGS_CHECK_GPU(seeds_in);
+  const int32_t w = id_width(seeds_in, "seeds");
+  TORCH_CHECK(seeds_in.scalar_type() == indices_dtype, "seeds (", seeds_in.scalar_type(), ") and indices (",
+              indices_dtype, ") must have the same dtype");
+  TORCH_CHECK(indptr.elem_bytes == 4 || indptr.elem_bytes == 8, "indptr must be int32 or int64");
+  TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0, got ", num_picks);
+  torch::Tensor seeds = seeds_in.contiguous().view({-1});
+  const int64_t n = seeds.numel();
+  const auto rng = next_rng();
+  void* st = current_stream();
+
+  const size_t ws_bytes = dgs_sample_workspace_bytes(n);
+  torch::Tensor ws = device_bytes(ws_bytes, seeds.device());
+  torch::Tensor nnz_dev = torch::empty({2}, seeds.options().dtype(torch::kInt64));
+
+  // Worst case n * num_picks ids per output: when that is modest the whole hop is
+  // enqueued before the one blocking length read; otherwise count first.
+  const bool one_shot = num_picks <= (int64_t(1) << 20) && n * num_picks <= (int64_t(1) << 28);
+  torch::Tensor rows, cols;
+  std::vector<int64_t> len;
+  if (one_shot) {
+    rows = torch::empty({n * num_picks}, seeds.options());
+    cols = torch::empty({n * num_picks}, seeds.options());
+    check(dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr, indices, num_picks, replace, rng.first, rng.second,
+                               rows.data_ptr(), cols.data_ptr(), nnz_dev.data_ptr<int64_t>(), ws.data_ptr(),
+                               ws_bytes, st));
+    len = read_back(nnz_dev, 2);
+  } else {
+    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(),
+                           ws.data_ptr(), ws_bytes, st));
+    len = read_back(nnz_dev, 2);
+    rows = torch::empty({len[0]}, seeds.options());
+    cols = torch::empty({len[0]}, seeds.options());
+    check(dgs_sample_fill(seeds.data_ptr(), w, n, indices, num_picks, replace, rng.first, rng.second,
+                          rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st));
+  }
+  TORCH_CHECK((len[1] & 1) == 0, "sample_neighbors: a seed row has a degree of 2^32 or more");
+  TORCH_CHECK((len[1] & 2) == 0,
+              "sample_neighbors: num_picks above 2048 without replacement needs every sampled row to have at most "
+              "num_picks neighbours");
+  return std::make_tuple(rows.narrow(0, 0, len[0]), cols.narrow(0, 0, len[0]));
+}
+
+// upstream RowWiseSamplingUniformCUDA (src/cuda/rowwise_sampling.cu:176-187)
+std::tuple<torch::Tensor, torch::Tensor> SampleNeighbors(torch::Tensor seeds, torch::Tensor indptr,
+                                                         torch::Tensor indices, int64_t num_picks, bool replace) {
+  DGS_CHECK_GPU(indptr);
+  DGS_CHECK_GPU(indices);
+  id_width(indptr, "indptr");
+  id_width(indices, "indices");
+  torch::Tensor ip = indptr.contiguous();
+  torch::Tensor ix = indices.contiguous();
+  return sample_impl(seeds, tensor_view(ip), tensor_view(ix), ix.scalar_type(), num_picks, replace);
+}
+
+// upstream RowWiseSamplingUniformWithChunkTensorCUDA
+// (src/cuda/rowwise_sampling_with_chunk_tensor.cu:185-194)
+std::tuple<torch::Tensor, torch::Tensor> SampleNeighborsWithChunkTensor(torch::Tensor seeds,
+                                                                        c10::intrusive_ptr<ChunkTensor> indptr,
+                                                                        c10::intrusive_ptr<ChunkTensor> indices,
+                                                                        int64_t num_picks, bool replace) {
+  TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
+              "indptr store must be int32 or int64");
+  return sample_impl(seeds, indptr->view(), indices->view(), indices->dtype(), num_picks, replace);
+}
+
+// Packs up to DGS_MAX_SEGMENTS tensors; more are concatenated first.
+dgs_segments pack_segments(std::vector<torch::Tensor>& tensors, std::vector<torch::Tensor>& keep_alive) {
+  dgs_segments s{};
+  if (tensors.size() > DGS_MAX_SEGMENTS) {
+    torch::Tensor all = torch::cat(tensors, 0);
+    keep_alive.push_back(all);
+    s.count = 1;
+    s.ptr[0] = all.data_ptr();
+    s.len[0] = all.numel();
+    return s;
+  }
+  s.count = static_cast<int32_t>(tensors.size());
+  for (size_t i = 0; i < tensors.size(); ++i) {
+    tensors[i] = tensors[i].contiguous().view({-1});
+    keep_alive.push_back(tensors[i]);
+    s.ptr[i] = tensors[i].data_ptr();
+    s.len[i] = tensors[i].numel();
+  }
+  return s;
+}
+
+// upstream TensorRelabelCUDA (src/cuda/tensor_reindex.cu:182-205)
+std::tuple<torch::Tensor, std::vector<torch::Tensor>> TensorRelabel(std::vector<torch::Tensor> mapping_tensors,
+                                                                    std::vector<torch::Tensor> requiring_relabel_tensors) {
+  TORCH_CHECK(!mapping_tensors.empty(), "tensor_relabel: mapping_tensors is empty");
+  const torch::ScalarType dt = mapping_tensors[0].scalar_type();
+  const int32_t w = id_width(mapping_tensors[0], "mapping tensors");
+  const torch::Device dev = mapping_tensors[0].device();
+  for (const auto& t : mapping_tensors) {
+    DGS_CHECK_GPU(t);
+    TORCH_CHECK(t.scalar_type() == dt, "tensor_relabel: all tensors must share one dtype");
+  }
+  for (const auto& t : requiring_relabel_tensors) {
+    DGS_CHECK_GPU(t);
+    TORCH_CHECK(t.scalar_type() == dt, "tensor_relabel: all tensors must share one dtype");
+  }
+  std::vector<torch::Tensor> keep;
+  dgs_segments map_seg = pack_segments(mapping_tensors, keep);
+  int64_t n = 0;
+  for (int i = 0; i < map_seg.count; ++i) n += map_seg.len[i];
+
+  // outputs: one flat buffer split like the inputs (upstream split_with_sizes, :201-202)
+  std::vector<int64_t> sizes;
+  int64_t m = 0;
+  for (const auto& t : requiring_relabel_tensors) {
+    sizes.push_back(t.numel());
+    m += t.numel();
+  }
+  auto opt = torch::TensorOptions().dtype(dt).device(dev);
+  torch::Tensor relabelled = torch::empty({m}, opt);
+  dgs_segments req_seg = pack_segments(requiring_relabel_tensors, keep);
+  dgs_segments out_seg{};
+  out_seg.count = req_seg.count;
+  {
+    char* p = static_cast<char*>(relabelled.data_ptr());
+    for (int i = 0; i < req_seg.count; ++i) {
+      out_seg.ptr[i] = p;
+      out_seg.len[i] = req_seg.len[i];
+      p += req_seg.len[i] * w;
+    }
+  }
+  torch::Tensor unique = torch::empty({n}, opt);
+  torch::Tensor num_unique = torch::empty({1}, opt.dtype(torch::kInt64));
+  const size_t ws_bytes = dgs_unique_relabel_workspace_bytes(n, w);
+  torch::Tensor ws = device_bytes(ws_bytes, dev);
+  check(dgs_unique_relabel(map_seg, req_seg, w, unique.data_ptr(), num_unique.data_ptr<int64_t>(), out_seg,
+                           ws.data_ptr(), ws_bytes, current_stream()));
+  const int64_t u = read_back(num_unique, 1)[0];
+  return std::make_tuple(unique.narrow(0, 0, u), relabelled.split_with_sizes(sizes, 0));
+}
+
+int64_t GetCurrentAllocated() { return dgs_current_allocated(); }
+
+// upstream nccl::GetUniqueId / nccl::SetNCCL (src/nccl_context.cc:17-34): there is no
+// communicator at world size 1; the shims keep unmodified harness code running.
+std::vector<int64_t> GetUniqueId() { return std::vector<int64_t>(16, 0); }
+void SetNCCL(int64_t nranks, std::vector<int64_t> /*unique_id*/, int64_t rank) {
+  TORCH_CHECK(nranks == 1 && rank == 0, "_CAPI_set_nccl: this build runs at world size 1 (got nranks=", nranks,
+              ", rank=", rank, ")");
+}
+
+void SetRngState(int64_t seed, int64_t stream) {
+  std::lock_guard<std::mutex> lock(g_rng_mutex);
+  g_rng_seed = static_cast<uint64_t>(seed);
+  g_rng_stream = static_cast<uint32_t>(stream);
+}
+std::vector<int64_t> GetRngState() {
+  std::lock_guard<std::mutex> lock(g_rng_mutex);
+  return {static_cast<int64_t>(g_rng_seed), static_cast<int64_t>(g_rng_stream)};
+}
+
+}  // namespace
+}  // namespace dgs
+
+using dgs::ChunkTensor;
+
+TORCH_LIBRARY(dgs_classes, m) {
+  m.class_<ChunkTensor>("ChunkTensor")
+      .def(torch::init<std::vector<int64_t>, torch::ScalarType, int64_t>())
+      .def("_CAPI_get_host_tensor", &ChunkTensor::GetHostTensor)
+      .def("_CAPI_get_sub_device_tensor", &ChunkTensor::GetSubDeviceTensor)
+      .def("_CAPI_index", &ChunkTensor::Index)
+      .def("_CAPI_split_index", &ChunkTensor::SplitIndex)
+      .def("_CAPI_local_index", &ChunkTensor::LocalIndex)
+      .def("_CAPI_remote_index", &ChunkTensor::RemoteIndex)
+      .def("_CAPI_host_index", &ChunkTensor::HostIndex)
+      .def("_CAPI_load_from_tensor", &ChunkTensor::LoadFromTensor);
+}
+
+TORCH_LIBRARY(dgs_ops, m) {
+  m.def("_CAPI_tensor_relabel", &dgs::TensorRelabel)
+      .def("_CAPI_sample_neighbors", &dgs::SampleNeighbors)
+      .def("_CAPI_sample_neighbors_with_chunk_tensor", &dgs::SampleNeighborsWithChunkTensor)
+      .def("_CAPI_get_unique_id", &dgs::GetUniqueId)
+      .def("_CAPI_set_nccl", &dgs::SetNCCL)
+      .def("_CAPI_get_current_allocated", &dgs::GetCurrentAllocated)
+      // not in upstream: the sampling generator's (seed, stream)
+      .def("_CAPI_set_rng_state", &dgs::SetRngState)
+      .def("_CAPI_get_rng_state", &dgs::GetRngState);
+}

@@ -1,0 +1,170 @@
+// Two-tier positional store: an HBM slice followed by a pinned, device-mapped
+// host slice.  World size is 1, so the peer tier and its IPC handle exchange
+// (upstream src/chunk_tensor.cc:112-139) have no counterpart here.
+#include <atomic>
+#include <cstdarg>
+#include <cstring>
+#include <new>
+
+#include "common.h"
+
+namespace dgs {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+// HBM bytes held by live stores (upstream src/cuda_context.h:11-38, made atomic).
+static std::atomic<int64_t> g_allocated{0};
+
+}  // namespace dgs
+
+struct dgs_store {
+  int64_t total = 0;
+  int64_t device_elems = 0;
+  int64_t host_elems = 0;
+  int32_t elem_bytes = 0;
+  int device = -1;
+  void* dev = nullptr;       // HBM slice
+  void* host_cpu = nullptr;  // pinned slice, CPU address
+  void* host_dev = nullptr;  // same memory, device address
+};
+
+DGS_API const char* dgs_last_error(void) { return dgs::g_error; }
+
+DGS_API const char* dgs_status_name(dgs_status s) {
+  switch (s) {
+    case DGS_OK: return "DGS_OK";
+    case DGS_ERR_INVALID: return "DGS_ERR_INVALID";
+    case DGS_ERR_HIP: return "DGS_ERR_HIP";
+    case DGS_ERR_WORKSPACE: return "DGS_ERR_WORKSPACE";
+    case DGS_ERR_UNSUPPORTED: return "DGS_ERR_UNSUPPORTED";
+    case DGS_ERR_RANGE: return "DGS_ERR_RANGE";
+    default: return "DGS_ERR_?";
+  }
+}
+
+DGS_API int dgs_abi_version(void) { return 1; }
+
+DGS_API dgs_status dgs_store_split(int64_t total_elems, int32_t elem_bytes, int64_t capacity_bytes,
+                                   int64_t* device_elems, int64_t* host_elems) {
+  DGS_REQUIRE(total_elems >= 0, DGS_ERR_INVALID, "store: negative element count %lld",
+              (long long)total_elems);
+  DGS_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8,
+              DGS_ERR_INVALID, "store: element width %d is not 1, 2, 4 or 8", elem_bytes);
+  DGS_REQUIRE(capacity_bytes >= 0, DGS_ERR_INVALID, "store: capacity_per_gpu %lld is negative",
+              (long long)capacity_bytes);
+  DGS_REQUIRE(device_elems && host_elems, DGS_ERR_INVALID, "store: null output pointer");
+  int64_t dev = capacity_bytes / elem_bytes;
+  if (dev > total_elems) dev = total_elems;
+  *device_elems = dev;
+  *host_elems = total_elems - dev;
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_store_create(int64_t total_elems, int32_t elem_bytes, int64_t capacity_bytes,
+                                    dgs_store** out) {
+  DGS_REQUIRE(out != nullptr, DGS_ERR_INVALID, "store: null output pointer");
+  *out = nullptr;
+  int64_t dev_elems = 0, host_elems = 0;
+  dgs_status st = dgs_store_split(total_elems, elem_bytes, capacity_bytes, &dev_elems, &host_elems);
+  if (st != DGS_OK) return st;
+
+  dgs_store* s = new (std::nothrow) dgs_store();
+  DGS_REQUIRE(s != nullptr, DGS_ERR_INVALID, "store: out of host memory");
+  s->total = total_elems;
+  s->device_elems = dev_elems;
+  s->host_elems = host_elems;
+  s->elem_bytes = elem_bytes;
+  hipError_t e = hipGetDevice(&s->device);
+  if (e == hipSuccess && host_elems > 0) {
+    e = hipHostMalloc(&s->host_cpu, size_t(host_elems) * elem_bytes,
+                      hipHostMallocMapped | hipHostMallocPortable);
+    if (e == hipSuccess) e = hipHostGetDevicePointer(&s->host_dev, s->host_cpu, 0);
+  }
+  if (e == hipSuccess && dev_elems > 0) {
+    const size_t bytes = size_t(dev_elems) * elem_bytes;
+    e = hipMalloc(&s->dev, bytes);
+    if (e == hipSuccess) {
+      dgs::g_allocated += int64_t(bytes);
+      e = hipMemset(s->dev, 0xFF, bytes);
+    }
+  }
+  if (e != hipSuccess) {
+    dgs::set_error("store: allocating %lld device + %lld host elements of %d B failed: %s",
+                   (long long)dev_elems, (long long)host_elems, elem_bytes, hipGetErrorString(e));
+    dgs_store_destroy(s);
+    return DGS_ERR_HIP;
+  }
+  *out = s;
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_store_destroy(dgs_store* s) {
+  if (s == nullptr) return DGS_OK;
+  hipError_t first = hipSuccess;
+  if (s->dev) {
+    hipError_t e = hipFree(s->dev);
+    if (e == hipSuccess) dgs::g_allocated -= s->device_elems * int64_t(s->elem_bytes);
+    else first = e;
+  }
+  if (s->host_cpu) {
+    hipError_t e = hipHostFree(s->host_cpu);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  }
+  delete s;
+  if (first != hipSuccess) {
+    dgs::set_error("store: release failed: %s", hipGetErrorString(first));
+    return DGS_ERR_HIP;
+  }
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_store_load(dgs_store* s, const void* src, int64_t n_elems) {
+  DGS_REQUIRE(s != nullptr, DGS_ERR_INVALID, "store: null store");
+  DGS_REQUIRE(n_elems == s->total, DGS_ERR_INVALID,
+              "store: load of %lld elements into a store of %lld", (long long)n_elems,
+              (long long)s->total);
+  DGS_REQUIRE(src != nullptr || n_elems == 0, DGS_ERR_INVALID, "store: null source");
+  const char* p = static_cast<const char*>(src);
+  const size_t dev_bytes = size_t(s->device_elems) * s->elem_bytes;
+  if (dev_bytes) DGS_HIP_TRY(hipMemcpy(s->dev, p, dev_bytes, hipMemcpyHostToDevice));
+  if (s->host_elems) memcpy(s->host_cpu, p + dev_bytes, size_t(s->host_elems) * s->elem_bytes);
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_store_view(const dgs_store* s, dgs_view* v) {
+  DGS_REQUIRE(s != nullptr && v != nullptr, DGS_ERR_INVALID, "store: null argument");
+  v->dev = s->dev;
+  v->host = s->host_dev;
+  v->threshold = s->device_elems;
+  v->total = s->total;
+  v->elem_bytes = s->elem_bytes;
+  v->reserved_ = 0;
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_store_slices(const dgs_store* s, void** dev_ptr, int64_t* device_elems,
+                                    void** host_cpu_ptr, int64_t* host_elems) {
+  DGS_REQUIRE(s != nullptr, DGS_ERR_INVALID, "store: null store");
+  if (dev_ptr) *dev_ptr = s->dev;
+  if (device_elems) *device_elems = s->device_elems;
+  if (host_cpu_ptr) *host_cpu_ptr = s->host_cpu;
+  if (host_elems) *host_elems = s->host_elems;
+  return DGS_OK;
+}
+
+DGS_API int64_t dgs_current_allocated(void) { return dgs::g_allocated.load(); }
+
+DGS_API dgs_status dgs_read_back(void* host_dst, const void* dev_src, size_t n_bytes, void* stream) {
+  DGS_REQUIRE(host_dst != nullptr && dev_src != nullptr, DGS_ERR_INVALID, "read_back: null pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  DGS_HIP_TRY(hipMemcpyAsync(host_dst, dev_src, n_bytes, hipMemcpyDeviceToHost, st));
+  DGS_HIP_TRY(hipStreamSynchronize(st));
+  return DGS_OK;
+}

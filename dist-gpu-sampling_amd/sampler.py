@@ -1,0 +1,66 @@
+"""Host-side counterpart of the upstream sampler glue
+(oppo_bench/single_node/utils/chunktensor_sampler.py) at world size 1, without
+DGL: a block is a plain record instead of a DGLBlock.
+"""
+from collections import namedtuple
+
+import torch
+
+# One message-flow block: edges (src_local[e] -> dst_local[e]); src_ids / dst_ids map
+# local to global node ids (upstream: block.srcdata[dgl.NID] / block.dstdata[dgl.NID]).
+Block = namedtuple("Block", ["src_local", "dst_local", "num_src", "num_dst", "src_ids", "dst_ids"])
+
+
+def set_rng_state(seed, stream=0):
+    """Seeds the sampling generator; the stream advances by one per sampling call."""
+    torch.ops.dgs_ops._CAPI_set_rng_state(int(seed), int(stream))
+
+
+def create_dgs_communicator(group_size=1, local_group=None):
+    """chunktensor_sampler.py:7-19.  World size is 1: the id exchange is a no-op."""
+    unique_ids = torch.ops.dgs_ops._CAPI_get_unique_id()
+    torch.ops.dgs_ops._CAPI_set_nccl(group_size, unique_ids, 0)
+
+
+def get_available_memory(device, reserved_mem, local_group=None):
+    """chunktensor_sampler.py:22-29 without the all_reduce(MIN) over ranks."""
+    available = (torch.cuda.mem_get_info(device)[1] - reserved_mem
+                 - torch.ops.dgs_ops._CAPI_get_current_allocated()
+                 - 0.3 * torch.cuda.max_memory_reserved())
+    return int(max(available, 0))
+
+
+def create_chunktensor(tensor, num_gpus, available_mem, cache_rate=1.0, root_rank=0, local_group=None):
+    """chunktensor_sampler.py:32-60: capacity per GPU =
+    int(min(total_bytes * cache_rate // num_gpus, available_mem))."""
+    if num_gpus != 1:
+        raise ValueError("this build runs at world size 1")
+    total_size = tensor.numel() * tensor.element_size()
+    cached_size_per_gpu = int(min(total_size * cache_rate // num_gpus, available_mem))
+    chunk_tensor = torch.classes.dgs_classes.ChunkTensor(list(tensor.shape), tensor.dtype, cached_size_per_gpu)
+    chunk_tensor._CAPI_load_from_tensor(tensor)
+    return chunk_tensor
+
+
+class ChunkTensorSampler:
+    """chunktensor_sampler.py:63-118 (uniform sampling only)."""
+
+    def __init__(self, fanouts, chunk_indptr, chunk_indices, replace=False):
+        self.chunk_indptr = chunk_indptr
+        self.chunk_indices = chunk_indices
+        self.fanouts = list(fanouts)
+        self.replace = replace
+
+    def sample_blocks(self, g, seed_nodes, exclude_eids=None):
+        """Returns (input_nodes, seed_nodes, blocks); `g` is unused, as upstream."""
+        seeds = seed_nodes.cuda()
+        blocks = []
+        frontier = seeds
+        for fan_out in reversed(self.fanouts):
+            coo_row, coo_col = torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor(
+                seeds, self.chunk_indptr, self.chunk_indices, fan_out, self.replace)
+            frontier, (coo_row, coo_col) = torch.ops.dgs_ops._CAPI_tensor_relabel(
+                [seeds, coo_col], [coo_row, coo_col])
+            blocks.insert(0, Block(coo_col, coo_row, frontier.numel(), seeds.numel(), frontier, seeds))
+            seeds = frontier
+        return frontier, seed_nodes, blocks

@@ -169,13 +169,31 @@ dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
  *              out_rows / out_cols and of `indices`)
  *   indptr   : view of N+1 offsets, elem_bytes 4 or 8
  *   indices  : view of E ids, elem_bytes == id_bytes
- *   out_rows, out_cols : device, capacity n_seeds * num_picks ids each
  *   nnz_dev  : device int64[2]; [0] receives the number of emitted edges,
- *              [1] a non-zero flag when some row had degree >= 2^32
- *              (its output is unspecified; report DGS_ERR_RANGE to the user)
- * Nothing is read back: the caller copies nnz_dev when it needs the length.
+ *              [1] flags: bit 0 = some row has degree >= 2^32, bit 1 = some
+ *              row has degree > num_picks > 2048 without replacement.  Flagged
+ *              rows emit nothing; the caller reports DGS_ERR_RANGE.
+ *   workspace: dgs_sample_workspace_bytes(n_seeds) bytes, 256-byte aligned,
+ *              shared by the count and the fill of the same hop
+ *
+ * dgs_sample_count is the degree/count/scan half (the reference's sub_indptr,
+ * rowwise_sampling_with_chunk_tensor.cu:127-156): it leaves the per-row
+ * offsets in the workspace and the edge count in nnz_dev.
+ * dgs_sample_fill is the COO fill (:15-111, :158-180); out_rows / out_cols
+ * must hold nnz ids.  dgs_sample_neighbors runs both; its outputs must hold
+ * n_seeds * num_picks ids (the worst case), so no length is read back between
+ * the two halves.  Nothing synchronises: copy nnz_dev when the length is needed.
  */
 size_t dgs_sample_workspace_bytes(int64_t n_seeds);
+dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t n_seeds,
+                            dgs_view indptr, int64_t num_picks, int32_t replace,
+                            int64_t* nnz_dev, void* workspace,
+                            size_t workspace_bytes, void* stream);
+dgs_status dgs_sample_fill(const void* seeds, int32_t id_bytes, int64_t n_seeds,
+                           dgs_view indices, int64_t num_picks, int32_t replace,
+                           uint64_t rng_seed, uint32_t rng_stream, void* out_rows,
+                           void* out_cols, void* workspace, size_t workspace_bytes,
+                           void* stream);
 dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes,
                                 int64_t n_seeds, dgs_view indptr,
                                 dgs_view indices, int64_t num_picks,
@@ -207,7 +225,7 @@ typedef struct dgs_segments {
  *   num_unique_dev : device int64[1]
  *   out            : device arrays, out.len must equal requiring.len
  * ids must be >= 0 (-1 is the empty-slot marker, as in the reference).
- * sum(mapping.len) must be < 2^31.
+ * sum(mapping.len) must be <= 2^30.
  */
 size_t dgs_unique_relabel_workspace_bytes(int64_t n_mapping, int32_t id_bytes);
 dgs_status dgs_unique_relabel(dgs_segments mapping, dgs_segments requiring,

@@ -1,0 +1,24 @@
+import importlib
+
+import numpy as np
+
+
+def load_pkg():
+    """The package directory name is not a Python identifier; import it by string."""
+    return importlib.import_module("dist-gpu-sampling_amd")
+
+
+def powerlaw_graph(rng, n, mean_deg, max_deg, zero_frac=0.02, id_dtype=np.int64, ptr_dtype=np.int64):
+    """CSC arrays with Pareto-like in-degrees (some zero) and uniform sources."""
+    deg = np.floor(rng.pareto(1.3, size=n) * mean_deg * 0.35 + 1).astype(np.int64)
+    deg = np.minimum(deg, max_deg)
+    deg[rng.random(n) < zero_frac] = 0
+    indptr = np.zeros(n + 1, dtype=ptr_dtype)
+    indptr[1:] = np.cumsum(deg)
+    indices = rng.integers(0, n, size=int(indptr[-1])).astype(id_dtype)
+    return indptr, indices
+
+
+def np_unique_first(x):
+    u, first = np.unique(x, return_index=True)
+    return u[np.argsort(first, kind="stable")]

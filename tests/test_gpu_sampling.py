@@ -1,0 +1,183 @@
+"""GPU parity of row-wise sampling and unique/relabel against the CPU oracle.
+Everything is bit-exact: full-fanout rows by construction, fanout < degree rows
+because kernel and oracle implement the same Philox/Floyd contract."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import load_pkg, np_unique_first, powerlaw_graph
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    return load_pkg()
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _np(t):
+    return t.cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def graph():
+    rng = np.random.default_rng(11)
+    return powerlaw_graph(rng, 20000, 20, 3000)
+
+
+@pytest.mark.parametrize("k,replace", [(1, False), (5, False), (8, False), (10, False), (15, False), (16, False),
+                                       (25, False), (50, False), (64, False), (65, False), (200, False),
+                                       (3, True), (15, True), (50, True), (64, True), (100, True)])
+def test_sample_parity_c_abi(pkg, oracle, graph, k, replace):
+    capi = pkg.capi
+    indptr, indices = graph
+    rng = np.random.default_rng(k * 7 + int(replace))
+    seeds = rng.integers(0, 20000, size=3001).astype(np.int64)
+    want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, k, replace, 0xABCDEF0123, 9)
+    ip, ix = _dev(indptr), _dev(indices)
+    for two_step in (False, True):
+        r, c, flags = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, replace,
+                                            0xABCDEF0123, 9, two_step=two_step)
+        assert flags == 0
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c), (k, replace, two_step)
+
+
+@pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int32, np.int32), (np.int32, np.int64), (np.int64, np.int32)])
+def test_sample_mixed_widths(pkg, oracle, id_dtype, ptr_dtype):
+    capi = pkg.capi
+    rng = np.random.default_rng(3)
+    indptr, indices = powerlaw_graph(rng, 5000, 15, 500, id_dtype=id_dtype, ptr_dtype=ptr_dtype)
+    seeds = rng.integers(0, 5000, size=1500).astype(id_dtype)
+    ip, ix = _dev(indptr), _dev(indices)
+    for k, replace in [(10, False), (7, True), (70, False)]:
+        want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, k, replace, 42, 1)
+        r, c, _ = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, replace, 42, 1)
+        assert r.dtype == _dev(seeds).dtype
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+
+
+def test_sample_edge_cases(pkg, oracle):
+    capi = pkg.capi
+    # rows: empty, degree 1, degree == k, degree k+1, large
+    deg = np.array([0, 1, 5, 6, 0, 300, 5, 0], dtype=np.int64)
+    indptr = np.zeros(9, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    indices = np.arange(indptr[-1], dtype=np.int64) * 3 + 1
+    ip, ix = _dev(indptr), _dev(indices)
+    seeds = np.array([7, 0, 3, 3, 5, 2, 1, 4, 6], dtype=np.int64)  # duplicates allowed
+    for k, replace in [(5, False), (5, True), (0, False), (1000, False)]:
+        want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, k, replace, 1, 2)
+        r, c, flags = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, replace, 1, 2)
+        assert flags == 0 and np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+    # no seeds at all
+    r, c, flags = capi.sample_neighbors(_dev(seeds[:0]), capi.tensor_view(ip), capi.tensor_view(ix), 5, False, 1, 2)
+    assert r.numel() == 0 and c.numel() == 0 and flags == 0
+    # fanout above the LDS limit with a row that would need sampling: flagged, row skipped
+    r, c, flags = capi.sample_neighbors(_dev(np.array([5], dtype=np.int64)), capi.tensor_view(ip),
+                                        capi.tensor_view(ix), 3000, False, 1, 2, two_step=True)
+    assert flags == 0 and r.numel() == 300  # deg 300 <= k: plain copy, nothing to flag
+
+
+def test_sample_with_chunk_tensor_tiers(pkg, oracle, graph):
+    indptr, indices = graph
+    rng = np.random.default_rng(8)
+    seeds = rng.permutation(20000)[:2048].astype(np.int64)
+    # both graph arrays split across HBM and host memory
+    ip_ct = pkg.ChunkTensor([indptr.size], torch.int64, 8 * 7001)
+    ip_ct._CAPI_load_from_tensor(torch.from_numpy(indptr))
+    ix_ct = pkg.ChunkTensor([indices.size], torch.int64, 8 * (indices.size // 3))
+    ix_ct._CAPI_load_from_tensor(torch.from_numpy(indices))
+    for k, replace in [(10, False), (10, True)]:
+        pkg.set_rng_state(555, 3)
+        r, c = pkg.ops._CAPI_sample_neighbors_with_chunk_tensor(_dev(seeds), ip_ct, ix_ct, k, replace)
+        want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, k, replace, 555, 3)
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+        assert pkg.ops._CAPI_get_rng_state() == [555, 4]  # one stream per call
+    # plain-tensor operator
+    pkg.set_rng_state(555, 3)
+    r, c = pkg.ops._CAPI_sample_neighbors(_dev(seeds), _dev(indptr), _dev(indices), 10, False)
+    want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, 10, False, 555, 3)
+    assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+
+
+def test_sample_chi_square_uniform(pkg):
+    # 4000 copies of one row of degree 40, k = 10 without replacement: each position is
+    # included with probability 1/4.  Rows are keyed by their id, so copies differ.
+    capi = pkg.capi
+    deg, k, copies = 40, 10, 4000
+    indptr = np.arange(0, (copies + 1) * deg, deg, dtype=np.int64)
+    indices = np.tile(np.arange(deg, dtype=np.int64), copies)
+    seeds = np.arange(copies, dtype=np.int64)
+    ip, ix = _dev(indptr), _dev(indices)
+    r, c, _ = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, False, 2024, 0)
+    picks = _np(c).reshape(copies, k)
+    assert all(len(set(row)) == k for row in picks[:500])
+    counts = np.bincount(picks.ravel(), minlength=deg).astype(float)
+    exp = copies * k / deg
+    # inclusion indicators are negatively correlated; variance per cell = n p (1-p)
+    z2 = ((counts - exp) ** 2 / (exp * (1 - k / deg))).sum()
+    assert z2 < 72.05  # chi-square 39 dof, p = 0.001
+    # with replacement: plain multinomial
+    r, c, _ = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, True, 2024, 1)
+    counts = np.bincount(_np(c), minlength=deg).astype(float)
+    assert ((counts - exp) ** 2 / exp).sum() < 72.05
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.int32])
+@pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (5000, 10 ** 6), (100000, 3000), (300000, 10 ** 9)])
+def test_unique_relabel_parity(pkg, oracle, dtype, n, hi):
+    rng = np.random.default_rng(n + hi)
+    seeds = rng.permutation(min(hi, 10 ** 6))[: min(hi, 37)].astype(dtype)
+    cols = rng.integers(0, hi, size=n).astype(dtype)
+    rows = rng.choice(seeds, size=n).astype(dtype)
+    want_u, (want_r, want_c) = oracle.unique_relabel([seeds, cols], [rows, cols])
+    assert np.array_equal(want_u, np_unique_first(np.concatenate([seeds, cols])))
+    u, (r, c) = pkg.capi.unique_relabel([_dev(seeds), _dev(cols)], [_dev(rows), _dev(cols)])
+    assert np.array_equal(_np(u), want_u) and np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+    # operator layer, including an id that is absent from the mapping
+    extra = np.array([hi + 5], dtype=dtype)
+    u2, outs = pkg.ops._CAPI_tensor_relabel([_dev(seeds), _dev(cols)], [_dev(rows), _dev(cols), _dev(extra)])
+    assert np.array_equal(_np(u2), want_u) and np.array_equal(_np(outs[1]), want_c)
+    assert _np(outs[2]).tolist() == [-1] and outs[0].dtype == _dev(rows).dtype
+
+
+def test_unique_many_segments(pkg, oracle):
+    rng = np.random.default_rng(12)
+    parts = [rng.integers(0, 500, size=s).astype(np.int64) for s in (5, 0, 300, 1, 77, 0, 1024, 3, 9, 200)]
+    want_u, want_outs = oracle.unique_relabel(parts, parts)
+    u, outs = pkg.ops._CAPI_tensor_relabel([_dev(p) for p in parts], [_dev(p) for p in parts])
+    assert np.array_equal(_np(u), want_u)
+    for a, b in zip(outs, want_outs):
+        assert np.array_equal(_np(a), b)
+    u8, outs8 = pkg.capi.unique_relabel([_dev(p) for p in parts[:8]], [_dev(p) for p in parts[:8]])
+    want_u8, _ = oracle.unique_relabel(parts[:8], parts[:8])
+    assert np.array_equal(_np(u8), want_u8)
+
+
+def test_sample_blocks_driver(pkg, oracle, graph):
+    indptr, indices = graph
+    ip_ct = pkg.ChunkTensor([indptr.size], torch.int64, 8 * indptr.size)
+    ip_ct._CAPI_load_from_tensor(torch.from_numpy(indptr))
+    ix_ct = pkg.ChunkTensor([indices.size], torch.int64, 8 * indices.size)
+    ix_ct._CAPI_load_from_tensor(torch.from_numpy(indices))
+    rng = np.random.default_rng(21)
+    seeds = rng.permutation(20000)[:512].astype(np.int64)
+    for fanouts, replace in [([15, 10, 5], False), ([4, 4], True)]:
+        sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, replace=replace)
+        pkg.set_rng_state(31337, 0)
+        frontier, out_seeds, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
+        o_frontier, _, o_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, replace, 31337, 0)
+        assert np.array_equal(_np(frontier), o_frontier) and len(blocks) == len(o_blocks)
+        for b, ob in zip(blocks, o_blocks):
+            assert np.array_equal(_np(b.src_local), ob[0]) and np.array_equal(_np(b.dst_local), ob[1])
+            assert (b.num_src, b.num_dst) == (ob[2], ob[3])
+            assert np.array_equal(_np(b.src_ids), ob[4]) and np.array_equal(_np(b.dst_ids), ob[5])
+        # then the feature gather of the final frontier
+        feats = torch.randn((20000, 100))
+        ft = pkg.create_chunktensor(feats, 1, 10 ** 12, cache_rate=0.5)
+        x = ft._CAPI_index(frontier)
+        assert torch.equal(x.cpu(), feats[frontier.cpu()])

@@ -1,0 +1,158 @@
+"""GPU parity of the two-tier store and its gathers against the CPU oracle and
+torch.index_select, through the C ABI and through the torch operator layer."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import load_pkg
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    return load_pkg()
+
+
+def _bits(t):
+    """Reinterpret any tensor as integers for bit-exact comparison."""
+    t = t.contiguous()
+    return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
+
+
+def test_readme_demo(pkg):
+    # upstream README.md:51-62: [100] int64 with 200 bytes per GPU
+    before = pkg.ops._CAPI_get_current_allocated()
+    c = pkg.ChunkTensor([100], torch.int64, 200)
+    assert pkg.ops._CAPI_get_current_allocated() - before == 200
+    assert (c._CAPI_get_sub_device_tensor() == -1).all()  # slice is pre-filled with 0xFF bytes
+    c._CAPI_load_from_tensor(torch.arange(100))
+    assert c._CAPI_get_host_tensor().tolist() == list(range(25, 100))
+    dev = c._CAPI_get_sub_device_tensor()
+    assert dev.is_cuda and dev.cpu().tolist() == list(range(25))
+    out = c._CAPI_index(torch.tensor([99, 0, 24, 25], device="cuda"))
+    assert out.shape == (4, 1) and out[:, 0].cpu().tolist() == [99, 0, 24, 25]
+    del c, dev
+    assert pkg.ops._CAPI_get_current_allocated() == before
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.int64, torch.int32, torch.bfloat16, torch.uint8,
+                                   torch.float64, torch.bool])
+@pytest.mark.parametrize("rows,dim", [(257, 100), (64, 128), (1000, 1), (33, 7), (50, 256)])
+def test_index_every_split(pkg, oracle, dtype, rows, dim):
+    g = torch.Generator().manual_seed(rows * 1000 + dim)
+    if dtype == torch.bool:
+        full = torch.rand((rows, dim), generator=g) > 0.5
+    elif dtype.is_floating_point:
+        full = torch.randn((rows, dim), generator=g).to(dtype)
+    else:
+        full = torch.randint(0, 200, (rows, dim), generator=g).to(dtype)
+    eb = full.element_size()
+    total_bytes = full.numel() * eb
+    # none, all, a row boundary, a split inside a row, an odd byte count
+    caps = [0, total_bytes, total_bytes + 999, (rows // 2) * dim * eb, (rows // 3) * dim * eb + 3 * eb,
+            (rows // 2) * dim * eb + 1]
+    for idx_dtype in (torch.int64, torch.int32):
+        idx = torch.randint(0, rows, (513,), generator=g).to(idx_dtype)
+        want = full[idx.long()]
+        for cap in caps:
+            ct = pkg.ChunkTensor([rows, dim], dtype, cap)
+            ct._CAPI_load_from_tensor(full)
+            got = ct._CAPI_index(idx.cuda())
+            assert got.dtype == dtype and got.shape == (513, dim)
+            assert torch.equal(_bits(got.cpu()), _bits(want)), (dtype, rows, dim, cap)
+            # the oracle (restating chunk_tensor_wrapper::At) agrees for the same split
+            if dtype not in (torch.bfloat16, torch.bool):
+                thr = oracle.store_split([rows, dim], eb, cap)["threshold"]
+                o = oracle.gather(full.numpy(), idx.numpy(), thr)
+                assert np.array_equal(o, got.cpu().numpy())
+
+
+def test_index_1d_and_empty(pkg):
+    full = torch.arange(1000, dtype=torch.int32)
+    ct = pkg.ChunkTensor([1000], torch.int32, 1234)
+    ct._CAPI_load_from_tensor(full)
+    idx = torch.tensor([999, 0, 308, 309, 500], device="cuda")
+    assert ct._CAPI_index(idx)[:, 0].cpu().tolist() == [999, 0, 308, 309, 500]
+    e = ct._CAPI_index(torch.empty(0, dtype=torch.int64, device="cuda"))
+    assert e.shape == (0, 1)
+    assert ct._CAPI_remote_index(torch.empty(0, dtype=torch.int64, device="cuda")).shape == (0, 1)
+
+
+def test_wide_rows(pkg):
+    # 600000-byte rows take the segment-per-block kernel
+    full = torch.randn((6, 150000))
+    ct = pkg.ChunkTensor([6, 150000], torch.float32, 2 * 150000 * 4 + 4 * 100)
+    ct._CAPI_load_from_tensor(full)
+    idx = torch.tensor([5, 2, 0, 2, 1], device="cuda")
+    assert torch.equal(ct._CAPI_index(idx).cpu(), full[idx.cpu()])
+
+
+def test_split_local_host_index(pkg, oracle):
+    rows, dim = 400, 12
+    full = torch.randn((rows, dim))
+    cap = 150 * dim * 4 + 5 * 4  # row 150 straddles the boundary
+    ct = pkg.ChunkTensor([rows, dim], torch.float32, cap)
+    ct._CAPI_load_from_tensor(full)
+    g = torch.Generator().manual_seed(5)
+    for n in (0, 1, 1023, 1024, 1025, 5000):
+        idx = torch.randint(0, rows, (n,), generator=g)
+        loc, rem, host = ct._CAPI_split_index(idx.cuda())
+        s = oracle.store_split([rows, dim], 4, cap)
+        o_loc, o_rem, o_host = oracle.split_index(idx.numpy(), s["threshold"], s["device_elems"], dim)
+        assert np.array_equal(loc.cpu().numpy(), o_loc) and np.array_equal(host.cpu().numpy(), o_host)
+        assert rem.numel() == 0 and o_rem.size == 0
+    # tier-specific gathers on rows wholly inside their tier
+    loc = loc[loc < 150]
+    assert torch.equal(ct._CAPI_local_index(loc).cpu(), full[loc.cpu()])
+    host = host[host > 150]
+    assert torch.equal(ct._CAPI_host_index(host).cpu(), full[host.cpu()])
+    # int32 ids
+    idx32 = torch.randint(0, rows, (777,), generator=g, dtype=torch.int32)
+    loc, _, host = ct._CAPI_split_index(idx32.cuda())
+    assert loc.dtype == torch.int32
+    assert torch.equal(loc.cpu(), idx32[idx32 < 150]) and torch.equal(host.cpu(), idx32[idx32 >= 150])
+
+
+def test_gather_through_c_abi(pkg, oracle):
+    capi = pkg.capi
+    rows, dim = 300, 100
+    full = torch.randn((rows, dim))
+    cap = 100 * dim * 4 + 8
+    st = capi.Store(rows * dim, 4, cap)
+    st.load(full)
+    assert (st.view.threshold, st.view.total, st.view.elem_bytes) == (100 * dim + 2, rows * dim, 4)
+    idx = torch.randint(0, rows, (999,), device="cuda")
+    out = capi.gather_rows(st.view, dim, idx, torch.float32)
+    assert np.array_equal(out.cpu().numpy(), oracle.gather(full.numpy(), idx.cpu().numpy(), st.view.threshold))
+    loc, host = capi.split_index(st.view, dim, idx)
+    assert torch.equal(loc, idx[idx < 100]) and torch.equal(host, idx[idx >= 100])
+    # plain device tensor as a single-tier view
+    dev = full.cuda()
+    out2 = capi.gather_rows(capi.tensor_view(dev), dim, idx, torch.float32)
+    assert torch.equal(out2, dev[idx])
+    st.close()
+
+
+def test_errors_raise_instead_of_aborting(pkg):
+    with pytest.raises(RuntimeError):
+        pkg.ChunkTensor([2, 2, 2], torch.float32, 0)
+    with pytest.raises(RuntimeError):
+        pkg.ChunkTensor([10], torch.float32, -1)
+    ct = pkg.ChunkTensor([10, 4], torch.float32, 64)
+    with pytest.raises(RuntimeError):
+        ct._CAPI_load_from_tensor(torch.zeros(10, 4, dtype=torch.float64))
+    with pytest.raises(RuntimeError):
+        ct._CAPI_load_from_tensor(torch.zeros(10, 5))
+    with pytest.raises(RuntimeError):
+        ct._CAPI_load_from_tensor(torch.zeros(4, 10).t())
+    with pytest.raises(RuntimeError):
+        ct._CAPI_load_from_tensor(torch.zeros(10, 4, device="cuda"))
+    with pytest.raises(RuntimeError):
+        ct._CAPI_index(torch.zeros(3, dtype=torch.int64))  # CPU index
+    with pytest.raises(RuntimeError):
+        ct._CAPI_index(torch.zeros(3, device="cuda"))  # float index
+    capi = pkg.capi
+    v = capi.tensor_view(torch.zeros(8, device="cuda"))
+    assert capi.lib.dgs_gather_rows(v, 1, None, 3, 1, None, 0, None) == capi.DGS_ERR_INVALID
+    assert b"index width" in capi.lib.dgs_last_error()
