@@ -135,6 +135,9 @@ def main():
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget-s", type=float, default=15.0)
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a known-size kernel to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings against)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures ONE GPU (world size 1); --gpus N with N > 1 is not supported")
@@ -175,6 +178,12 @@ def main():
     for i in range(args.warmup):
         step(batches[i])
     torch.cuda.synchronize()
+    if args.calibrate_copy_mib > 0:
+        src = torch.empty(args.calibrate_copy_mib << 18, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads and writes calibrate_copy_mib MiB each
+        torch.cuda.synchronize()
+        del src, dst
 
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
     stats = []

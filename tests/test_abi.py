@@ -1,0 +1,100 @@
+"""CPU-side checks of the boundary: the C ABI library loads, exports every symbol
+the header declares, and its host-only entry points behave; the operator layer
+registers the upstream names.  No GPU work is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from helpers import load_pkg
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "dgs_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dgs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    pkg = load_pkg()
+    names = _declared_functions()
+    assert len(names) >= 18
+    lib = ctypes.CDLL(pkg.HIP_LIB)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/dgs_hip.h but not exported"
+    # the ctypes binding covers exactly the declared functions
+    assert sorted(pkg.capi.SIGNATURES) == names
+
+
+def test_struct_layouts_match_the_header():
+    pkg = load_pkg()
+    assert ctypes.sizeof(pkg.capi.View) == 40      # 2 pointers + 2 int64 + 2 int32
+    assert ctypes.sizeof(pkg.capi.Segments) == 8 * 8 + 8 * 8 + 8
+    assert pkg.capi.lib.dgs_abi_version() == 1
+
+
+def test_store_split_matches_oracle(oracle):
+    pkg = load_pkg()
+    lib = pkg.capi.lib
+    d, h = ctypes.c_int64(), ctypes.c_int64()
+    for total, eb, cap in [(100, 8, 200), (100, 8, 0), (100, 8, 10 ** 6), (70, 4, 101), (0, 4, 16), (7, 1, 3),
+                           (10 ** 12, 2, 10 ** 11 + 1)]:
+        assert lib.dgs_store_split(total, eb, cap, ctypes.byref(d), ctypes.byref(h)) == 0
+        o = oracle.store_split([total], eb, cap)
+        assert (d.value, h.value) == (o["threshold"], o["host_elems"])
+    assert lib.dgs_store_split(100, 8, -1, ctypes.byref(d), ctypes.byref(h)) == pkg.capi.DGS_ERR_INVALID
+    assert b"capacity_per_gpu" in lib.dgs_last_error()
+    assert lib.dgs_store_split(100, 3, 8, ctypes.byref(d), ctypes.byref(h)) == pkg.capi.DGS_ERR_INVALID
+    assert lib.dgs_status_name(5) == b"DGS_ERR_RANGE"
+
+
+def test_workspace_queries_are_monotone():
+    lib = load_pkg().capi.lib
+    prev = 0
+    for n in (0, 1, 255, 256, 257, 10 ** 4, 10 ** 6):
+        cur = lib.dgs_sample_workspace_bytes(n)
+        assert cur >= prev and cur >= 12 * n
+        prev = cur
+    assert lib.dgs_unique_relabel_workspace_bytes(1000, 8) >= 2048 * 12 + 4000
+    assert lib.dgs_unique_relabel_workspace_bytes(10 ** 6, 4) < lib.dgs_unique_relabel_workspace_bytes(10 ** 6, 8)
+    assert lib.dgs_split_index_workspace_bytes(0) > 0
+
+
+def test_operator_surface_is_registered():
+    import torch
+    load_pkg()
+    for name in ("_CAPI_tensor_relabel", "_CAPI_sample_neighbors", "_CAPI_sample_neighbors_with_chunk_tensor",
+                 "_CAPI_get_current_allocated", "_CAPI_get_unique_id", "_CAPI_set_nccl"):
+        assert hasattr(torch.ops.dgs_ops, name)
+    cls = torch.classes.dgs_classes.ChunkTensor
+    assert cls is not None
+    schema = str(torch.ops.dgs_ops._CAPI_sample_neighbors.default._schema)
+    assert "Tensor seeds" in schema or "Tensor _0" in schema
+    assert torch.ops.dgs_ops._CAPI_get_current_allocated() == 0
+    assert len(torch.ops.dgs_ops._CAPI_get_unique_id()) == 16
+    torch.ops.dgs_ops._CAPI_set_nccl(1, [0] * 16, 0)
+    with pytest.raises(RuntimeError):
+        torch.ops.dgs_ops._CAPI_set_nccl(2, [0] * 16, 1)
+
+
+def test_no_gpu_means_a_loud_error_not_a_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    pkg = load_pkg()
+    with pytest.raises(RuntimeError, match="DGS_ERR_HIP"):
+        pkg.ChunkTensor([10], torch.float32, 16)
+
+
+def test_sampler_cache_size_formula():
+    # chunktensor_sampler.py:40-42: int(min(total_bytes * cache_rate // num_gpus, available_mem))
+    import inspect
+    pkg = load_pkg()
+    src = inspect.getsource(pkg.create_chunktensor)
+    assert "total_size * cache_rate // num_gpus" in src
+    with pytest.raises(ValueError):
+        import torch
+        pkg.create_chunktensor(torch.zeros(4), 2, 100)
