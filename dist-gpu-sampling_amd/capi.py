@@ -26,6 +26,11 @@ class View(ctypes.Structure):
                 ("elem_bytes", c_i32), ("reserved_", c_i32)]
 
 
+class BlockOut(ctypes.Structure):
+    """dgs_block_out"""
+    _fields_ = [("src_local", c_vp), ("dst_local", c_vp)]
+
+
 class Segments(ctypes.Structure):
     """dgs_segments"""
     _fields_ = [("ptr", c_vp * MAX_SEGMENTS), ("len", c_i64 * MAX_SEGMENTS), ("count", c_i32),
@@ -46,6 +51,7 @@ SIGNATURES = {
                                         ctypes.POINTER(c_vp), ctypes.POINTER(c_i64)]),
     "dgs_current_allocated": (c_i64, []),
     "dgs_gather_rows": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i32, c_vp]),
+    "dgs_gather_rows_dyn": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_i32, c_vp]),
     "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
     "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_workspace_bytes": (c_sz, [c_i64]),
@@ -56,6 +62,13 @@ SIGNATURES = {
                                             c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_unique_relabel_workspace_bytes": (c_sz, [c_i64, c_i32]),
     "dgs_unique_relabel": (ctypes.c_int, [Segments, Segments, c_i32, c_vp, c_vp, Segments, c_vp, c_sz, c_vp]),
+    "dgs_sample_blocks_plan": (ctypes.c_int, [c_i64, ctypes.POINTER(c_i64), c_i32, ctypes.POINTER(c_i64),
+                                              ctypes.POINTER(c_i64)]),
+    "dgs_sample_blocks_workspace_bytes": (c_sz, [c_i64, ctypes.POINTER(c_i64), c_i32, c_i32]),
+    "dgs_node_table_bytes": (c_sz, [c_i64]),
+    "dgs_sample_blocks": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, ctypes.POINTER(c_i64), c_i32, c_i32,
+                                         c_u64, c_u32, c_vp, c_u32, c_vp, ctypes.POINTER(BlockOut), c_vp, c_vp,
+                                         c_sz, c_vp]),
     "dgs_read_back": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp]),
 }
 
@@ -197,3 +210,42 @@ def unique_relabel(mapping, requiring):
                                  segments(outs), ws.data_ptr(), nb, stream_ptr()))
     u = read_i64(num, 1)[0]
     return unique[:u], outs
+
+
+def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_seed, first_stream,
+                  feature_view=None, feature_row_elems=None, feature_dtype=None, node_table=None, epoch=0):
+    """All hops in one call.  Returns [(frontier, src_local, dst_local) per hop], the gathered
+    rows of the last frontier when a feature view is given, and the per-hop error flags.
+    `node_table` is an int64 device tensor of dgs_node_table_bytes(n_nodes) bytes filled with -1."""
+    hops = len(hop_fanouts)
+    n = seeds.numel()
+    fan = (c_i64 * hops)(*hop_fanouts)
+    smax = (c_i64 * (hops + 1))()
+    emax = (c_i64 * hops)()
+    check(lib.dgs_sample_blocks_plan(n, fan, hops, smax, emax))
+    w = seeds.element_size()
+    frontier = torch.empty(smax[hops], dtype=seeds.dtype, device=seeds.device)
+    bufs = []
+    outs = (BlockOut * hops)()
+    for h in range(hops):
+        s = torch.empty(emax[h], dtype=seeds.dtype, device=seeds.device)
+        d = torch.empty(emax[h], dtype=seeds.dtype, device=seeds.device)
+        bufs.append((s, d))
+        outs[h] = BlockOut(s.data_ptr(), d.data_ptr())
+    sizes = torch.empty(3 * hops + 1, dtype=torch.int64, device=seeds.device)
+    nb = lib.dgs_sample_blocks_workspace_bytes(n, fan, hops, w)
+    ws = _ws(nb, seeds.device)
+    check(lib.dgs_sample_blocks(seeds.data_ptr(), w, n, indptr_view, indices_view, fan, hops, int(replace),
+                                rng_seed, first_stream, node_table.data_ptr() if node_table is not None else None,
+                                epoch, frontier.data_ptr(), outs, sizes.data_ptr(), ws.data_ptr(), nb,
+                                stream_ptr()))
+    x = None
+    if feature_view is not None:
+        x = torch.empty((smax[hops], feature_row_elems), dtype=feature_dtype, device=seeds.device)
+        check(lib.dgs_gather_rows_dyn(feature_view, feature_row_elems, frontier.data_ptr(), w, smax[hops],
+                                      sizes.data_ptr() + 8 * hops, x.data_ptr(), TIER_ANY, stream_ptr()))
+    sz = read_i64(sizes, 3 * hops + 1)
+    result = [(frontier[:sz[h + 1]], s[:sz[hops + 1 + h]], d[:sz[hops + 1 + h]]) for h, (s, d) in enumerate(bufs)]
+    if x is not None:
+        x = x[:sz[hops]]
+    return result, x, sz[2 * hops + 1:]

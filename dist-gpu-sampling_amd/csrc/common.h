@@ -97,26 +97,49 @@ __device__ __forceinline__ T block_exclusive_scan(T v, T* total, T* lds) {
   return wave_off + incl - v;
 }
 
-// One block: out[t] = exclusive prefix of in[0..t) for t < count, *sum = total.
-// Used for the per-tile totals of the multi-block scans (count is small).
-template <typename T>
-__device__ __forceinline__ void single_block_scan_1024(const T* __restrict__ in, T* __restrict__ out,
-                                                       int64_t count, T* sum) {
-  __shared__ T lds[1024 / kWave];
-  __shared__ T carry;
+// One block of NT threads: out[t] = exclusive prefix of in[0..t) for t < count, *sum = total
+// (valid in thread 0).  Used for the per-tile totals of the multi-block scans (count is small).
+template <int NT, typename TIn, typename TOut>
+__device__ __forceinline__ void single_block_scan(const TIn* __restrict__ in, TOut* __restrict__ out,
+                                                  int64_t count, TOut* sum) {
+  __shared__ TOut lds[NT / kWave];
+  __shared__ TOut carry;
   if (threadIdx.x == 0) carry = 0;
   __syncthreads();
-  for (int64_t t0 = 0; t0 < count; t0 += 1024) {
+  for (int64_t t0 = 0; t0 < count; t0 += NT) {
     const int64_t t = t0 + threadIdx.x;
-    const T v = t < count ? in[t] : T(0);
-    T total;
-    const T ex = block_exclusive_scan<1024, T>(v, &total, lds);
+    const TOut v = t < count ? TOut(in[t]) : TOut(0);
+    TOut total;
+    const TOut ex = block_exclusive_scan<NT, TOut>(v, &total, lds);
     if (t < count) out[t] = carry + ex;
     __syncthreads();
     if (threadIdx.x == 0) carry += total;
     __syncthreads();
   }
   if (threadIdx.x == 0) *sum = carry;
+}
+
+template <typename T>
+__device__ __forceinline__ void single_block_scan_1024(const T* __restrict__ in, T* __restrict__ out,
+                                                       int64_t count, T* sum) {
+  single_block_scan<1024, T, T>(in, out, count, sum);
+}
+
+// "Last block done" election without spinning: every block calls this once after its
+// global writes; exactly one block (the last to arrive) gets true and may then read what
+// all the others wrote.  The counter must be 0 on entry and is left at 0.
+__device__ __forceinline__ bool last_block_arrives(int* counter) {
+  __shared__ bool is_last;
+  __threadfence();  // release this block's writes at device scope
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int ticket = atomicAdd(counter, 1);
+    is_last = ticket == int(gridDim.x) - 1;
+    if (is_last) *counter = 0;
+  }
+  __syncthreads();
+  if (is_last) __threadfence();  // acquire the other blocks' writes
+  return is_last;
 }
 
 // Philox4x32-10 block for the "dgs-philox-1" contract.

@@ -54,8 +54,8 @@ torch::Tensor device_bytes(size_t n, const torch::Device& dev) {
 // Blocking read of a few int64 values from the device through a pinned buffer.
 std::vector<int64_t> read_back(const torch::Tensor& dev, int64_t count) {
   thread_local torch::Tensor pinned =
-      torch::empty({16}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-  TORCH_CHECK(count <= 16);
+      torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+  TORCH_CHECK(count <= 32);
   check(dgs_read_back(pinned.data_ptr(), dev.data_ptr(), sizeof(int64_t) * count, current_stream()));
   const int64_t* p = pinned.data_ptr<int64_t>();
   return std::vector<int64_t>(p, p + count);
@@ -66,9 +66,12 @@ std::mutex g_rng_mutex;
 uint64_t g_rng_seed = 7777;  // upstream's constant, used until the caller sets one
 uint32_t g_rng_stream = 0;   // advanced by one per sampling call
 
-std::pair<uint64_t, uint32_t> next_rng() {
+// Reserves `calls` consecutive streams and returns (seed, first stream).
+std::pair<uint64_t, uint32_t> next_rng(uint32_t calls = 1) {
   std::lock_guard<std::mutex> lock(g_rng_mutex);
-  return {g_rng_seed, g_rng_stream++};
+  const uint32_t first = g_rng_stream;
+  g_rng_stream += calls;
+  return {g_rng_seed, first};
 }
 
 }  // namespace
@@ -171,8 +174,24 @@ class ChunkTensor : public torch::CustomClassHolder {
     return std::make_tuple(local.narrow(0, 0, c[0]), torch::empty({0}, index.options()), host.narrow(0, 0, c[1]));
   }
 
+  // Persistent direct-address table for sample_blocks when this store is a graph's indptr
+  // (one entry per node).  Created on first use; returns (pointer, epoch for this call).
+  std::pair<void*, uint32_t> node_table() {
+    const int64_t n_nodes = total_ - 1;
+    const size_t bytes = dgs_node_table_bytes(n_nodes);
+    if (bytes == 0 || bytes > (size_t(8) << 30)) return {nullptr, 0u};
+    std::lock_guard<std::mutex> lock(node_table_mutex_);
+    if (!node_table_.defined() || node_epoch_ >= 0xffffff00u) {
+      node_table_ = torch::full({static_cast<int64_t>(bytes / 8)}, int64_t(-1),
+                                torch::TensorOptions().dtype(torch::kInt64).device(device_));
+      node_epoch_ = 0;
+    }
+    return {node_table_.data_ptr(), ++node_epoch_};
+  }
+
   const dgs_view& view() const { return view_; }
   torch::ScalarType dtype() const { return dtype_; }
+  int64_t elem_stride() const { return elem_stride_; }
 
  private:
   std::vector<int64_t> shapes_;
@@ -183,6 +202,9 @@ class ChunkTensor : public torch::CustomClassHolder {
   dgs_store* store_ = nullptr;
   dgs_view view_{};
   c10::Device device_{c10::DeviceType::CUDA, 0};
+  torch::Tensor node_table_;
+  uint32_t node_epoch_ = 0;
+  std::mutex node_table_mutex_;
 };
 
 namespace {
@@ -338,6 +360,79 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> TensorRelabel(std::vector<
   return std::make_tuple(unique.narrow(0, 0, u), relabelled.split_with_sizes(sizes, 0));
 }
 
+// All hops of the sampler loop (chunktensor_sampler.py:93-118) in one call with a single
+// blocking length read at the end.  `fanouts` is in hop order (the reversed model
+// fanouts).  Returns per hop, nearest the seeds first: frontier (= the hop's source ids,
+// seeds first), src_local, dst_local -- and, when `features` is given, the gathered
+// feature rows of the last frontier, enqueued before the lengths are known.
+std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor>
+sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<ChunkTensor>& indptr,
+                   const c10::intrusive_ptr<ChunkTensor>& indices, const std::vector<int64_t>& fanouts,
+                   bool replace, const c10::intrusive_ptr<ChunkTensor>& features) {
+  DGS_CHECK_GPU(seeds_in);
+  const int32_t w = id_width(seeds_in, "seeds");
+  TORCH_CHECK(seeds_in.scalar_type() == indices->dtype(), "seeds (", seeds_in.scalar_type(), ") and indices (",
+              indices->dtype(), ") must have the same dtype");
+  TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
+              "indptr store must be int32 or int64");
+  const int32_t hops = static_cast<int32_t>(fanouts.size());
+  TORCH_CHECK(hops >= 1 && hops <= DGS_MAX_HOPS, "sample_blocks: between 1 and ", DGS_MAX_HOPS, " fanouts");
+  torch::Tensor seeds = seeds_in.contiguous().view({-1});
+  const int64_t n = seeds.numel();
+  std::vector<int64_t> seeds_max(hops + 1), edges_max(hops);
+  check(dgs_sample_blocks_plan(n, fanouts.data(), hops, seeds_max.data(), edges_max.data()));
+
+  const auto opt = seeds.options();
+  std::vector<torch::Tensor> frontier(hops), src(hops), dst(hops);
+  std::vector<dgs_block_out> outs(hops);
+  torch::Tensor all = torch::empty({seeds_max[hops]}, opt);  // every hop's frontier is a prefix of it
+  for (int h = 0; h < hops; ++h) {
+    src[h] = torch::empty({edges_max[h]}, opt);
+    dst[h] = torch::empty({edges_max[h]}, opt);
+    outs[h] = dgs_block_out{src[h].data_ptr(), dst[h].data_ptr()};
+  }
+  const int n_sizes = 3 * hops + 1;
+  torch::Tensor sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
+  const size_t ws_bytes = dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
+  torch::Tensor ws = device_bytes(ws_bytes, seeds.device());
+  const auto rng = next_rng(static_cast<uint32_t>(hops));
+  const auto table = indptr->node_table();
+  void* st = current_stream();
+  check(dgs_sample_blocks(seeds.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops, replace,
+                          rng.first, rng.second, table.first, table.second, all.data_ptr(), outs.data(),
+                          sizes_dev.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
+  torch::Tensor x;
+  if (features) {
+    x = torch::empty({seeds_max[hops], features->elem_stride()}, opt.dtype(features->dtype()));
+    check(dgs_gather_rows_dyn(features->view(), features->elem_stride(), all.data_ptr(), w, seeds_max[hops],
+                              sizes_dev.data_ptr<int64_t>() + hops, x.data_ptr(), DGS_TIER_ANY, st));
+  }
+  const std::vector<int64_t> sz = read_back(sizes_dev, n_sizes);
+  for (int h = 0; h < hops; ++h) {
+    TORCH_CHECK(sz[2 * hops + 1 + h] == 0, "sample_blocks: a seed row of hop ", h, " has a degree of 2^32 or more");
+    frontier[h] = all.narrow(0, 0, sz[h + 1]);
+    src[h] = src[h].narrow(0, 0, sz[hops + 1 + h]);
+    dst[h] = dst[h].narrow(0, 0, sz[hops + 1 + h]);
+  }
+  if (features) x = x.narrow(0, 0, sz[hops]);
+  return std::make_tuple(frontier, src, dst, x);
+}
+
+std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>> SampleBlocks(
+    torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr, c10::intrusive_ptr<ChunkTensor> indices,
+    std::vector<int64_t> fanouts, bool replace) {
+  auto r = sample_blocks_impl(seeds, indptr, indices, fanouts, replace, c10::intrusive_ptr<ChunkTensor>());
+  return std::make_tuple(std::get<0>(r), std::get<1>(r), std::get<2>(r));
+}
+
+std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor>
+SampleBlocksAndIndex(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr,
+                     c10::intrusive_ptr<ChunkTensor> indices, std::vector<int64_t> fanouts, bool replace,
+                     c10::intrusive_ptr<ChunkTensor> features) {
+  TORCH_CHECK(features, "sample_blocks_and_index: features store is null");
+  return sample_blocks_impl(seeds, indptr, indices, fanouts, replace, features);
+}
+
 int64_t GetCurrentAllocated() { return dgs_current_allocated(); }
 
 // upstream nccl::GetUniqueId / nccl::SetNCCL (src/nccl_context.cc:17-34): there is no
@@ -383,6 +478,9 @@ TORCH_LIBRARY(dgs_ops, m) {
       .def("_CAPI_get_unique_id", &dgs::GetUniqueId)
       .def("_CAPI_set_nccl", &dgs::SetNCCL)
       .def("_CAPI_get_current_allocated", &dgs::GetCurrentAllocated)
+      // not in upstream: the whole sampler loop (and optionally the feature gather) in one call
+      .def("_CAPI_sample_blocks", &dgs::SampleBlocks)
+      .def("_CAPI_sample_blocks_and_index", &dgs::SampleBlocksAndIndex)
       // not in upstream: the sampling generator's (seed, stream)
       .def("_CAPI_set_rng_state", &dgs::SetRngState)
       .def("_CAPI_get_rng_state", &dgs::GetRngState);

@@ -43,9 +43,11 @@ template <int VEC, int TIER, typename IndexT>
 __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, uint32_t cpr, uint32_t magic, const IndexT* __restrict__ index,
-    int64_t total_chunks, char* __restrict__ out) {
+    int64_t total_chunks, const int64_t* __restrict__ n_rows_dev, char* __restrict__ out) {
   using C = typename Chunk<VEC>::type;
   const int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock;
+  if (n_rows_dev) total_chunks = *n_rows_dev * cpr;  // row count decided on the device
+  if (c0 >= total_chunks) return;
   const int64_t row0 = c0 / cpr;
   const uint32_t rem0 = uint32_t(c0 - row0 * cpr);
 
@@ -77,9 +79,10 @@ template <int VEC, int TIER, typename IndexT>
 __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, int64_t cpr, int64_t blocks_per_row, const IndexT* __restrict__ index,
-    char* __restrict__ out) {
+    const int64_t* __restrict__ n_rows_dev, char* __restrict__ out) {
   using C = typename Chunk<VEC>::type;
   const int64_t row = int64_t(blockIdx.x) / blocks_per_row;
+  if (n_rows_dev && row >= *n_rows_dev) return;
   const int64_t seg = int64_t(blockIdx.x) - row * blocks_per_row;
   const int64_t src_row = int64_t(index[row]);
 #pragma unroll
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
 
 template <int VEC, int TIER, typename IndexT>
 dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index, int64_t n,
-                         void* out, hipStream_t st) {
+                         const int64_t* n_dev, void* out, hipStream_t st) {
   const int64_t cpr = row_bytes / VEC;
   const int64_t thr_bytes = v.threshold * v.elem_bytes;
   const char* dev = static_cast<const char*>(v.dev);
@@ -108,7 +111,7 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
     const uint32_t magic = cpr > 1 ? uint32_t((uint64_t(1) << 32) / uint64_t(cpr)) + 1u : 0u;
     hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT>), dim3(uint32_t(blocks)),
                        dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
-                       magic, static_cast<const IndexT*>(index), total_chunks,
+                       magic, static_cast<const IndexT*>(index), total_chunks, n_dev,
                        static_cast<char*>(out));
   } else {
     const int64_t bpr = (cpr + kChunksPerBlock - 1) / kChunksPerBlock;
@@ -116,7 +119,7 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
                 (long long)n, (long long)row_bytes);
     hipLaunchKernelGGL((gather_wide_kernel<VEC, TIER, IndexT>), dim3(uint32_t(n * bpr)),
                        dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, cpr, bpr,
-                       static_cast<const IndexT*>(index), static_cast<char*>(out));
+                       static_cast<const IndexT*>(index), n_dev, static_cast<char*>(out));
   }
   DGS_LAUNCH_CHECK();
   return DGS_OK;
@@ -124,20 +127,20 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
 
 template <int VEC, int TIER>
 dgs_status dispatch_index(const dgs_view& v, int64_t row_bytes, const void* index,
-                          int32_t index_bytes, int64_t n, void* out, hipStream_t st) {
-  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, out, st)
-                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, out, st);
+                          int32_t index_bytes, int64_t n, const int64_t* n_dev, void* out, hipStream_t st) {
+  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, out, st)
+                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, out, st);
 }
 
 template <int TIER>
 dgs_status dispatch_vec(int vec, const dgs_view& v, int64_t row_bytes, const void* index,
-                        int32_t index_bytes, int64_t n, void* out, hipStream_t st) {
+                        int32_t index_bytes, int64_t n, const int64_t* n_dev, void* out, hipStream_t st) {
   switch (vec) {
-    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, out, st);
-    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, out, st);
-    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, out, st);
-    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, out, st);
-    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, out, st);
+    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
   }
 }
 
@@ -236,9 +239,9 @@ __global__ __launch_bounds__(kSplitThreads) void split_scatter_kernel(
 }  // namespace
 }  // namespace dgs
 
-DGS_API dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
-                                   int32_t index_bytes, int64_t n, void* out, int32_t tier,
-                                   void* stream) {
+namespace {
+dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_t index_bytes, int64_t n,
+                        const int64_t* n_dev, void* out, int32_t tier, void* stream) {
   using namespace dgs;
   DGS_REQUIRE(width_ok(index_bytes), DGS_ERR_INVALID, "gather: index width %d is not 4 or 8", index_bytes);
   DGS_REQUIRE(n >= 0 && row_elems > 0, DGS_ERR_INVALID, "gather: n=%lld row_elems=%lld", (long long)n,
@@ -258,10 +261,24 @@ DGS_API dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* in
   const int vec = pick_vec(v, row_bytes, out, tier);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (tier) {
-    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, out, st);
-    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, out, st);
-    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, out, st);
+    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, out, st);
   }
+}
+}  // namespace
+
+DGS_API dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
+                                   int32_t index_bytes, int64_t n, void* out, int32_t tier,
+                                   void* stream) {
+  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, out, tier, stream);
+}
+
+DGS_API dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
+                                       int32_t index_bytes, int64_t n_max, const int64_t* n_rows_dev,
+                                       void* out, int32_t tier, void* stream) {
+  DGS_REQUIRE(n_rows_dev != nullptr, DGS_ERR_INVALID, "gather_dyn: null n_rows_dev");
+  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, out, tier, stream);
 }
 
 DGS_API size_t dgs_split_index_workspace_bytes(int64_t n) {

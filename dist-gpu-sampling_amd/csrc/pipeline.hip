@@ -1,0 +1,563 @@
+// Multi-hop sampling + relabel as one stream of kernels with no host round trip and no
+// synchronisation between blocks inside a kernel.
+//
+// The per-hop operators (sample.hip, unique.hip) each read a length back to the host so
+// that they can return exactly-sized arrays.  Here every buffer has its worst-case size
+// (hop h has at most S_h = S_{h-1} (1 + k_{h-1}) seeds), lengths stay in device memory,
+// grids are sized for the worst case and surplus blocks retire at once.
+//
+// Two facts make the chain short:
+//   * ranks are decided by the ORDER of mapping positions only, so a hop may use the
+//     padded positions S + i*k + l (row i, pick l) instead of the packed ones: no
+//     count/scan has to run before the picks are inserted;
+//   * the frontier of hop h is the seed list of hop h+1 and its ids already sit in the
+//     table with value = rank = position, so ONE table serves all hops, seeds are never
+//     re-inserted, only the picked ids of a hop are flagged and compacted, and the
+//     frontier is a single array that grows hop by hop.
+//
+// Critical path per hop (3 launches): fill -> flag -> compact.
+//   fill     G lanes per seed row (G = 8..64): indptr pair, picks by the dgs-philox-1
+//            contract, picked id inserted at its padded position; keeps slot + row count.
+//   flag     a position is a first occurrence iff the table holds that position; counts
+//            per 1024-position tile.
+//   compact  every block sums the tile counts before its own (the list is short), ranks
+//            its first occurrences, appends them to the frontier, stores the rank in the
+//            table.
+// Off the critical path, riding as surplus blocks of the next launches: per-row pick
+// counts are scanned per 256-row tile (with flag), and the packed edge list
+// (src_local, dst_local) is written once ranks exist (with the next hop's fill, or a
+// final launch).
+#include <cstdlib>
+
+#include "common.h"
+#include "table.h"
+
+namespace dgs {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kRowTile = 256;                  // seed rows per offsets tile
+constexpr int kPosItems = 4;
+constexpr int kPosTile = kBlock * kPosItems;   // padded positions per flag/compact block
+constexpr uint32_t kFirstBit = 0x80000000u;
+constexpr uint32_t kInvalidSlot = 0xffffffffu; // padded position that holds no pick
+constexpr uint32_t kBadRow = 0xffffffffu;      // row_cnt marker: degree >= 2^32
+constexpr int kMaxPicks = 64;
+constexpr int64_t kMaxPositions = int64_t(1) << 30;
+constexpr int64_t kInlineTiles = 2048;         // above this a separate scan launch is used
+
+struct Hop {
+  const void* seeds;        // seed ids: caller's seeds (hop 0) or the frontier array
+  const int64_t* n_seeds;   // device scalar (ignored when n_seeds_host >= 0)
+  int64_t n_seeds_host;     // hop 0: the caller's count; later hops: -1
+  int64_t* n_seeds_out;     // hop 0: where to publish n_seeds on the device
+  int64_t* n_unique;        // device scalar: frontier size after this hop
+  int64_t* nnz;             // device scalar: edges of this hop
+  int64_t* flags;           // device scalar: non-zero on a bad row
+  uint32_t* row_cnt;        // [s_max] picks of every row (kBadRow on error)
+  uint32_t* row_off;        // [s_max] exclusive offset of the row inside its 256-row tile
+  int* tile_sum;            // [row tiles]
+  int* tile_flag;           // [row tiles]
+  int64_t* tile_off;        // [row tiles] only when row tiles > kInlineTiles
+  uint32_t* slot;           // [seed part + s_max * k] table slot of every padded position
+  int* pos_cnt;             // [position tiles] first occurrences per tile
+  int64_t* pos_off;         // [position tiles] only when position tiles > kInlineTiles
+  void* frontier;           // growing array of distinct ids
+  void* src_local;          // out [nnz]
+  void* dst_local;          // out [nnz]
+  int64_t s_max;
+  int32_t k;
+  int32_t index;            // hop number
+  uint32_t rng_stream;
+  int32_t pad_;
+};
+
+__device__ __forceinline__ int64_t seeds_of(const Hop& h) {
+  return h.n_seeds_host >= 0 ? h.n_seeds_host : *h.n_seeds;
+}
+// positions [0, seed_part) of hop 0 are the caller's seeds themselves
+__device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h.index == 0 ? s : 0; }
+// first mapping position that this hop has to flag and compact
+__device__ __forceinline__ int64_t first_position(const Hop& h, int64_t s) { return h.index == 0 ? 0 : s; }
+
+template <int NT, typename T>
+__device__ __forceinline__ T block_sum(T v, T* lds /* NT/64 */) {
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
+  __syncthreads();
+  T s = 0;
+#pragma unroll
+  for (int w = 0; w < NT / kWave; ++w) s += lds[w];
+  __syncthreads();
+  return s;
+}
+
+// Position inside the row for output slot l of a row of degree deg (all G lanes of the
+// group call this together); returns false when the slot is empty.
+template <int G>
+__device__ __forceinline__ bool pick_position(uint32_t deg, int k, bool replace, int l, int group_lane0,
+                                              uint64_t rng_seed, uint32_t rng_stream, int64_t row,
+                                              uint32_t* pos) {
+  if (replace) {
+    if (deg == 0 || l >= k) return false;
+    *pos = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), deg);
+    return true;
+  }
+  if (deg <= uint32_t(k)) {
+    *pos = uint32_t(l);
+    return uint32_t(l) < deg;
+  }
+  // Floyd: slot s draws from [0, deg-k+s]; a value already kept by a lower slot is replaced
+  // by deg-k+s, which no lower slot can hold.
+  constexpr uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << (G & 63)) - 1);
+  const uint32_t top = deg - uint32_t(k) + uint32_t(l);
+  uint32_t cand = 0xffffffffu;
+  if (l < k) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), top + 1u);
+  uint32_t kept = cand;
+  for (int s = 1; s < k; ++s) {
+    const uint32_t c = __shfl(cand, s, G);
+    const uint64_t hit = (__ballot(kept == c && l < s) >> group_lane0) & group_mask;
+    if (l == s && hit) kept = top;
+  }
+  *pos = kept;
+  return l < k;
+}
+
+// ---- packed edge list of one hop (off the critical path) -----------------------------
+
+// One block per 256-row tile: scan of the rows' pick counts.
+__device__ __forceinline__ void offsets_tile(const Hop& h, int tile) {
+  __shared__ int lds[kBlock / kWave];
+  __shared__ int bad;
+  if (threadIdx.x == 0) bad = 0;
+  __syncthreads();
+  const int64_t s = seeds_of(h);
+  const int64_t i = int64_t(tile) * kRowTile + threadIdx.x;
+  int c = 0;
+  if (i < s) {
+    const uint32_t rc = h.row_cnt[i];
+    if (rc == kBadRow) bad = 1; else c = int(rc);
+  }
+  int total;
+  const int ex = block_exclusive_scan<kBlock, int>(c, &total, lds);
+  if (i < s) h.row_off[i] = uint32_t(ex);
+  if (threadIdx.x == 0) {
+    h.tile_sum[tile] = total;
+    h.tile_flag[tile] = bad;
+  }
+}
+
+// One block per (256-row tile, 256 padded picks): writes the rows' edges at their packed
+// offsets.  src_local = rank of the picked id; dst_local = rank of the row's seed, which is
+// the row number itself except in hop 0, whose seeds may repeat.
+template <typename IdT, typename TableT>
+__device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, int64_t b) {
+  __shared__ int64_t lds[kBlock / kWave];
+  const int64_t s = seeds_of(h);
+  const int64_t tiles = (s + kRowTile - 1) / kRowTile;
+  const int k = h.k;
+  if (b == 0) {  // totals of the hop, written even when there is nothing to do
+    int64_t sum = 0;
+    int64_t bad = 0;
+    for (int64_t j = threadIdx.x; j < tiles; j += kBlock) {
+      sum += h.tile_sum[j];
+      bad += h.tile_flag[j];
+    }
+    sum = block_sum<kBlock, int64_t>(sum, lds);
+    bad = block_sum<kBlock, int64_t>(bad, lds);
+    if (threadIdx.x == 0) {
+      *h.nnz = sum;
+      *h.flags = bad != 0;
+    }
+  }
+  if (k == 0) return;
+  const int64_t tile = b / k;
+  const int chunk = int(b - tile * k);
+  if (tile >= tiles) return;
+  int64_t prefix;
+  if (h.tile_off) {
+    prefix = h.tile_off[tile];
+  } else {
+    int64_t part = 0;
+    for (int64_t j = threadIdx.x; j < tile; j += kBlock) part += h.tile_sum[j];
+    prefix = block_sum<kBlock, int64_t>(part, lds);
+  }
+  const int t = chunk * kBlock + threadIdx.x;  // padded pick inside the tile
+  const int r = t / k;
+  const int l = t - r * k;
+  const int64_t i = tile * kRowTile + r;
+  if (r >= kRowTile || i >= s) return;
+  const uint32_t rc = h.row_cnt[i];
+  if (rc == kBadRow || uint32_t(l) >= rc) return;
+  const int64_t o = prefix + h.row_off[i] + l;
+  const uint32_t src_slot = h.slot[seed_part(h, s) + i * k + l] & ~kFirstBit;
+  static_cast<IdT*>(h.src_local)[o] = IdT(table.value(src_slot));
+  static_cast<IdT*>(h.dst_local)[o] =
+      h.index == 0 ? IdT(table.value(h.slot[i] & ~kFirstBit)) : IdT(i);
+}
+
+inline int64_t relabel_blocks(int64_t s_max, int k) {
+  return k > 0 ? ((s_max + kRowTile - 1) / kRowTile) * k : 1;
+}
+
+// ---- critical path ------------------------------------------------------------------------
+
+template <typename IdT, typename PtrT, typename TableT, int G>
+__global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64_t fill_blocks, TableT table,
+                                                          TierView<PtrT> indptr, TierView<IdT> indices,
+                                                          bool replace, uint64_t rng_seed) {
+  if (int64_t(blockIdx.x) >= fill_blocks) {  // surplus blocks: edge list of the previous hop
+    relabel_tile<IdT, TableT>(prev, table, int64_t(blockIdx.x) - fill_blocks);
+    return;
+  }
+  const int64_t s = seeds_of(h);
+  if (h.n_seeds_out && blockIdx.x == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
+  const int64_t gid = int64_t(blockIdx.x) * kBlock + threadIdx.x;
+  const int64_t i = gid / G;
+  const int l = int(gid % G);
+  if (i >= s) return;  // whole groups leave together
+  const int group_lane0 = (threadIdx.x & (kWave - 1)) - l;
+  const IdT seed = static_cast<const IdT*>(h.seeds)[i];
+  const int64_t row = int64_t(seed);
+  const int64_t b = int64_t(indptr.at(row));
+  const int64_t e = int64_t(indptr.at(row + 1));
+  const int64_t deg64 = e - b;
+  const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
+  const uint32_t deg = bad ? 0u : uint32_t(deg64);
+  const int k = h.k;
+  const int64_t sp = seed_part(h, s);
+  if (l == 0) {
+    h.row_cnt[i] = bad ? kBadRow : (replace ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
+    if (h.index == 0) h.slot[i] = table.insert(seed, uint32_t(i));
+  }
+  uint32_t pos;
+  const bool have = pick_position<G>(deg, k, replace, l, group_lane0, rng_seed, h.rng_stream, row, &pos);
+  if (l < k) {
+    const int64_t rel = sp + i * k + l;
+    uint32_t sl = kInvalidSlot;
+    if (have) {
+      const IdT col = indices.at(b + pos);
+      sl = table.insert(col, uint32_t(first_position(h, s) + rel));
+    }
+    h.slot[rel] = sl;
+  }
+}
+
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_blocks, TableT table) {
+  if (int64_t(blockIdx.x) >= flag_blocks) {  // surplus blocks: per-tile row offsets of this hop
+    offsets_tile(h, int(int64_t(blockIdx.x) - flag_blocks));
+    return;
+  }
+  __shared__ int lds[kBlock / kWave];
+  const int64_t s = seeds_of(h);
+  const int64_t len = seed_part(h, s) + s * h.k;
+  const int64_t p0 = first_position(h, s);
+  const int64_t base = int64_t(blockIdx.x) * kPosTile + threadIdx.x * kPosItems;
+  int c = 0;
+#pragma unroll
+  for (int j = 0; j < kPosItems; ++j) {
+    const int64_t rel = base + j;
+    if (rel < len) {
+      const uint32_t sl = h.slot[rel];
+      if (sl != kInvalidSlot && table.value(sl) == uint32_t(p0 + rel)) {
+        h.slot[rel] = sl | kFirstBit;
+        ++c;
+      }
+    }
+  }
+  c = block_sum<kBlock, int>(c, lds);
+  if (threadIdx.x == 0) h.pos_cnt[blockIdx.x] = c;
+}
+
+// Separate scans for very long tile lists (one block).
+__global__ __launch_bounds__(1024) void pos_scan_kernel(Hop h) {
+  const int64_t s = seeds_of(h);
+  const int64_t tiles = (seed_part(h, s) + s * h.k + kPosTile - 1) / kPosTile;
+  int64_t sum;
+  single_block_scan<1024, int, int64_t>(h.pos_cnt, h.pos_off, tiles, &sum);
+}
+__global__ __launch_bounds__(1024) void tile_scan_kernel(Hop h) {
+  const int64_t tiles = (seeds_of(h) + kRowTile - 1) / kRowTile;
+  int64_t sum;
+  single_block_scan<1024, int, int64_t>(h.tile_sum, h.tile_off, tiles, &sum);
+}
+
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, TableT table) {
+  __shared__ int64_t lds64[kBlock / kWave];
+  __shared__ int lds[kBlock / kWave];
+  const int64_t s = seeds_of(h);
+  const int64_t len = seed_part(h, s) + s * h.k;
+  const int64_t tiles = (len + kPosTile - 1) / kPosTile;
+  const int64_t rank0 = first_position(h, s);  // hop 0 starts at rank 0, later hops after the seeds
+  const int64_t tile = blockIdx.x;
+  if (tile >= tiles && tile != 0) return;
+  // first occurrences in the tiles before this one (block 0 also needs the grand total)
+  int64_t before = 0, all = 0;
+  if (h.pos_off) {
+    before = tile < tiles ? h.pos_off[tile] : 0;
+    if (tile == 0 && tiles > 0) all = h.pos_off[tiles - 1] + h.pos_cnt[tiles - 1];
+  } else {
+    const int64_t upto = tile == 0 ? tiles : tile;
+    int64_t part = 0;
+    for (int64_t j = threadIdx.x; j < upto; j += kBlock) part += h.pos_cnt[j];
+    part = block_sum<kBlock, int64_t>(part, lds64);
+    if (tile == 0) all = part; else before = part;
+  }
+  if (tile == 0 && threadIdx.x == 0) *h.n_unique = rank0 + all;
+  if (tile >= tiles) return;
+  const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
+  uint32_t sl[kPosItems];
+  int c = 0;
+#pragma unroll
+  for (int j = 0; j < kPosItems; ++j) {
+    sl[j] = base + j < len ? h.slot[base + j] : kInvalidSlot;
+    if (sl[j] == kInvalidSlot) sl[j] = 0;  // bit 31 clear: not a first occurrence
+    c += (sl[j] & kFirstBit) != 0;
+  }
+  int total;
+  int64_t rank = rank0 + before + block_exclusive_scan<kBlock, int>(c, &total, lds);
+#pragma unroll
+  for (int j = 0; j < kPosItems; ++j) {
+    if (sl[j] & kFirstBit) {
+      const uint32_t slot = sl[j] & ~kFirstBit;
+      static_cast<IdT*>(h.frontier)[rank] = table.key(slot);
+      table.set_value(slot, uint32_t(rank));
+      ++rank;
+    }
+  }
+}
+
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kBlock) void hop_relabel_kernel(Hop h, TableT table) {
+  relabel_tile<IdT, TableT>(h, table, int64_t(blockIdx.x));
+}
+
+__global__ __launch_bounds__(kBlock) void clear_kernel(uint4* __restrict__ p, int64_t n16) {
+  const int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x;
+  if (i < n16) p[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+}
+
+// ---- host side -------------------------------------------------------------------------------
+
+enum class TableKind { kDirect, kPacked, kSplit };
+
+struct Plan {
+  int n_hops = 0;
+  TableKind kind = TableKind::kSplit;
+  int64_t s_max[DGS_MAX_HOPS + 1];
+  int64_t nnz_max[DGS_MAX_HOPS];
+  uint32_t capacity = 0;     // hash table slots (one table for all hops)
+  size_t table_bytes = 0;    // 0 for the direct table
+};
+
+dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, int32_t id_bytes,
+                     int64_t n_nodes, bool have_node_table, Plan* p) {
+  DGS_REQUIRE(n_hops >= 1 && n_hops <= DGS_MAX_HOPS, DGS_ERR_INVALID, "sample_blocks: %d hops (1..%d)", n_hops,
+              DGS_MAX_HOPS);
+  DGS_REQUIRE(fanouts != nullptr && n_seeds >= 0, DGS_ERR_INVALID, "sample_blocks: bad argument");
+  DGS_REQUIRE(width_ok(id_bytes), DGS_ERR_INVALID, "sample_blocks: id width %d is not 4 or 8", id_bytes);
+  p->n_hops = n_hops;
+  p->s_max[0] = n_seeds;
+  for (int h = 0; h < n_hops; ++h) {
+    DGS_REQUIRE(fanouts[h] >= 0 && fanouts[h] <= kMaxPicks, DGS_ERR_UNSUPPORTED,
+                "sample_blocks: fanout %lld outside 0..%d (use the per-hop operators)", (long long)fanouts[h],
+                kMaxPicks);
+    p->nnz_max[h] = p->s_max[h] * fanouts[h];
+    p->s_max[h + 1] = p->s_max[h] + p->nnz_max[h];
+    DGS_REQUIRE(p->s_max[h + 1] <= kMaxPositions, DGS_ERR_UNSUPPORTED,
+                "sample_blocks: worst-case frontier of hop %d exceeds 2^30 ids", h);
+  }
+  if (have_node_table) {
+    DGS_REQUIRE(n_nodes >= 0 && n_nodes < 0x7fffffffLL, DGS_ERR_UNSUPPORTED,
+                "sample_blocks: a node table needs fewer than 2^31 nodes (have %lld)", (long long)n_nodes);
+    p->kind = TableKind::kDirect;
+  } else {
+    // ids fit the packed slot when every node id is below 2^32 - 1
+    p->kind = id_bytes == 4 || (n_nodes >= 0 && n_nodes < 0xffffffffLL) ? TableKind::kPacked : TableKind::kSplit;
+    // test hook: exercise the split (id array + value array) table on small graphs
+    if (id_bytes == 8 && getenv("DGS_FORCE_SPLIT_TABLE") != nullptr) p->kind = TableKind::kSplit;
+    p->capacity = table_capacity(p->s_max[n_hops]);
+    p->table_bytes = size_t(p->capacity) * (p->kind == TableKind::kPacked ? 8 : size_t(id_bytes) + 4);
+  }
+  return DGS_OK;
+}
+
+// Lays the workspace out; with base == nullptr only the size is computed.
+size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void** table) {
+  Carver c(base);
+  char* t = c.take<char>(p.table_bytes);
+  if (table) *table = t;
+  for (int h = 0; h < p.n_hops; ++h) {
+    const size_t s = size_t(p.s_max[h]);
+    const size_t len = (h == 0 ? s : 0) + size_t(p.nnz_max[h]);
+    const size_t row_tiles = (s + kRowTile - 1) / kRowTile;
+    const size_t pos_tiles = (len + kPosTile - 1) / kPosTile;
+    Hop v{};
+    v.row_cnt = c.take<uint32_t>(s);
+    v.row_off = c.take<uint32_t>(s);
+    v.tile_sum = c.take<int>(row_tiles);
+    v.tile_flag = c.take<int>(row_tiles);
+    v.tile_off = row_tiles > size_t(kInlineTiles) ? c.take<int64_t>(row_tiles) : nullptr;
+    v.slot = c.take<uint32_t>(len);
+    v.pos_cnt = c.take<int>(pos_tiles + 1);
+    v.pos_off = pos_tiles > size_t(kInlineTiles) ? c.take<int64_t>(pos_tiles) : nullptr;
+    v.s_max = p.s_max[h];
+    v.k = int32_t(fanouts[h]);
+    v.index = h;
+    if (hops) hops[h] = v;
+  }
+  return c.used + 256;
+}
+
+template <typename IdT, typename PtrT, typename TableT, int G>
+void launch_fill(const Hop& cur, const Hop& prev, int64_t surplus, const TableT& table, const dgs_view& indptr,
+                 const dgs_view& indices, bool replace, uint64_t rng_seed, hipStream_t st) {
+  const int64_t fill_blocks = (cur.s_max * G + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G>), dim3(uint32_t(fill_blocks + surplus)), dim3(kBlock), 0,
+                     st, cur, prev, fill_blocks, table, TierView<PtrT>(indptr), TierView<IdT>(indices), replace,
+                     rng_seed);
+}
+
+template <typename IdT, typename PtrT, typename TableT>
+dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_view& indptr,
+                      const dgs_view& indices, bool replace, uint64_t rng_seed, hipStream_t st) {
+  for (int h = 0; h < p.n_hops; ++h) {
+    const Hop& cur = hops[h];
+    const Hop prev = h > 0 ? hops[h - 1] : Hop{};
+    const int64_t surplus = h > 0 ? relabel_blocks(prev.s_max, prev.k) : 0;
+    if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
+    else if (cur.k <= 16) launch_fill<IdT, PtrT, TableT, 16>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
+    else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
+    else launch_fill<IdT, PtrT, TableT, 64>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
+    DGS_LAUNCH_CHECK();
+
+    const int64_t len_max = (h == 0 ? cur.s_max : 0) + cur.s_max * cur.k;
+    const int64_t pos_tiles = (len_max + kPosTile - 1) / kPosTile;
+    const int64_t row_tiles = (cur.s_max + kRowTile - 1) / kRowTile;
+    hipLaunchKernelGGL((hop_flag_kernel<IdT, TableT>), dim3(uint32_t(pos_tiles + row_tiles)), dim3(kBlock), 0, st,
+                       cur, pos_tiles, table);
+    DGS_LAUNCH_CHECK();
+    if (cur.pos_off) {
+      hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
+      DGS_LAUNCH_CHECK();
+    }
+    if (cur.tile_off) {
+      hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
+      DGS_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT>), dim3(uint32_t(pos_tiles > 0 ? pos_tiles : 1)),
+                       dim3(kBlock), 0, st, cur, table);
+    DGS_LAUNCH_CHECK();
+  }
+  const Hop& last = hops[p.n_hops - 1];
+  hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT>), dim3(uint32_t(relabel_blocks(last.s_max, last.k))),
+                     dim3(kBlock), 0, st, last, table);
+  DGS_LAUNCH_CHECK();
+  return DGS_OK;
+}
+
+template <typename IdT, typename PtrT>
+dgs_status run_blocks_table(const Plan& p, Hop* hops, void* hash_table, void* node_table, uint32_t epoch,
+                            const dgs_view& indptr, const dgs_view& indices, bool replace, uint64_t rng_seed,
+                            hipStream_t st) {
+  if (p.kind == TableKind::kDirect)
+    return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch), indptr, indices,
+                                                   replace, rng_seed, st);
+  const int64_t n16 = int64_t(p.table_bytes / 16);
+  hipLaunchKernelGGL(clear_kernel, dim3(uint32_t((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
+                     static_cast<uint4*>(hash_table), n16);
+  DGS_LAUNCH_CHECK();
+  if (p.kind == TableKind::kPacked)
+    return run_blocks<IdT, PtrT, Table<IdT, true>>(p, hops, Table<IdT, true>(hash_table, p.capacity), indptr,
+                                                   indices, replace, rng_seed, st);
+  return run_blocks<IdT, PtrT, Table<IdT, false>>(p, hops, Table<IdT, false>(hash_table, p.capacity), indptr,
+                                                  indices, replace, rng_seed, st);
+}
+
+}  // namespace
+}  // namespace dgs
+
+DGS_API dgs_status dgs_sample_blocks_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops,
+                                          int64_t* seeds_max, int64_t* edges_max) {
+  dgs::Plan p;
+  dgs_status s = dgs::make_plan(n_seeds, fanouts, n_hops, 8, -1, false, &p);
+  if (s != DGS_OK) return s;
+  DGS_REQUIRE(seeds_max && edges_max, DGS_ERR_INVALID, "sample_blocks_plan: null output");
+  for (int h = 0; h <= n_hops; ++h) seeds_max[h] = p.s_max[h];
+  for (int h = 0; h < n_hops; ++h) edges_max[h] = p.nnz_max[h];
+  return DGS_OK;
+}
+
+DGS_API size_t dgs_sample_blocks_workspace_bytes(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops,
+                                                 int32_t id_bytes) {
+  dgs::Plan p;
+  // sized for the split hash table, the largest of the layouts
+  if (dgs::make_plan(n_seeds, fanouts, n_hops, id_bytes, -1, false, &p) != DGS_OK) return 0;
+  p.kind = dgs::TableKind::kSplit;
+  p.table_bytes = size_t(p.capacity) * (size_t(id_bytes) + 4);
+  return dgs::layout(p, fanouts, nullptr, nullptr, nullptr);
+}
+
+DGS_API size_t dgs_node_table_bytes(int64_t n_nodes) {
+  return n_nodes > 0 && n_nodes < 0x7fffffffLL ? size_t(n_nodes) * 8 : 0;
+}
+
+DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
+                                     dgs_view indices, const int64_t* fanouts, int32_t n_hops, int32_t replace,
+                                     uint64_t rng_seed, uint32_t first_stream, void* node_table,
+                                     uint32_t node_table_epoch, void* frontier, const dgs_block_out* outs,
+                                     int64_t* sizes_dev, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace dgs;
+  Plan p;
+  // node count = indptr entries - 1
+  dgs_status s = make_plan(n_seeds, fanouts, n_hops, id_bytes, indptr.total - 1, node_table != nullptr, &p);
+  if (s != DGS_OK) return s;
+  DGS_REQUIRE(width_ok(indptr.elem_bytes), DGS_ERR_INVALID, "sample_blocks: indptr width %d", indptr.elem_bytes);
+  DGS_REQUIRE(indices.elem_bytes == id_bytes, DGS_ERR_INVALID,
+              "sample_blocks: indices width %d differs from the seed width %d", indices.elem_bytes, id_bytes);
+  DGS_REQUIRE(outs != nullptr && sizes_dev != nullptr, DGS_ERR_INVALID, "sample_blocks: null output");
+  DGS_REQUIRE(node_table == nullptr || (node_table_epoch >= 1 && node_table_epoch < 0xfffffff0u), DGS_ERR_INVALID,
+              "sample_blocks: node table epoch %u outside 1..2^32-17 (refill the table with 0xFF and restart at 1)",
+              node_table_epoch);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n_seeds == 0) {  // nothing to launch: every size is zero
+    DGS_HIP_TRY(hipMemsetAsync(sizes_dev, 0, sizeof(int64_t) * size_t(3 * n_hops + 1), st));
+    return DGS_OK;
+  }
+  DGS_REQUIRE(seeds != nullptr && frontier != nullptr, DGS_ERR_INVALID, "sample_blocks: null seeds or frontier");
+  DGS_REQUIRE(workspace != nullptr && workspace_bytes >= dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes),
+              DGS_ERR_WORKSPACE, "sample_blocks: workspace of %zu B, need %zu", workspace_bytes,
+              dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes));
+  DGS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, DGS_ERR_WORKSPACE,
+              "sample_blocks: workspace must be 256-byte aligned");
+  Hop hops[DGS_MAX_HOPS];
+  void* hash_table = nullptr;
+  layout(p, fanouts, workspace, hops, &hash_table);
+  for (int h = 0; h < n_hops; ++h) {
+    Hop& t = hops[h];
+    DGS_REQUIRE(p.nnz_max[h] == 0 || (outs[h].src_local && outs[h].dst_local), DGS_ERR_INVALID,
+                "sample_blocks: null edge buffers for hop %d", h);
+    t.seeds = h == 0 ? seeds : frontier;
+    t.n_seeds = sizes_dev + h;
+    t.n_seeds_host = h == 0 ? n_seeds : -1;
+    t.n_seeds_out = h == 0 ? sizes_dev : nullptr;
+    t.n_unique = sizes_dev + h + 1;
+    t.nnz = sizes_dev + n_hops + 1 + h;
+    t.flags = sizes_dev + 2 * n_hops + 1 + h;
+    t.frontier = frontier;
+    t.src_local = outs[h].src_local;
+    t.dst_local = outs[h].dst_local;
+    t.rng_stream = first_stream + uint32_t(h);
+  }
+  const bool rep = replace != 0;
+  if (id_bytes == 8)
+    return indptr.elem_bytes == 8
+               ? run_blocks_table<int64_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st)
+               : run_blocks_table<int64_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st);
+  return indptr.elem_bytes == 8
+             ? run_blocks_table<int32_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st)
+             : run_blocks_table<int32_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st);
+}

@@ -43,17 +43,37 @@ def create_chunktensor(tensor, num_gpus, available_mem, cache_rate=1.0, root_ran
 
 
 class ChunkTensorSampler:
-    """chunktensor_sampler.py:63-118 (uniform sampling only)."""
+    """chunktensor_sampler.py:63-118 (uniform sampling only).
 
-    def __init__(self, fanouts, chunk_indptr, chunk_indices, replace=False):
+    sample_blocks runs the upstream loop -- per hop one sampling call and one relabel call,
+    over reversed(fanouts) -- through the single fused operator when every fanout is at
+    most 64 (`fused=False` forces the per-hop operators; both give identical results).
+    """
+
+    FUSED_MAX_FANOUT = 64
+
+    def __init__(self, fanouts, chunk_indptr, chunk_indices, replace=False, fused=True):
         self.chunk_indptr = chunk_indptr
         self.chunk_indices = chunk_indices
         self.fanouts = list(fanouts)
         self.replace = replace
+        self.fused = fused and all(0 <= f <= self.FUSED_MAX_FANOUT for f in self.fanouts)
+
+    @staticmethod
+    def _blocks(seeds, frontiers, srcs, dsts):
+        blocks = []
+        for frontier, src, dst in zip(frontiers, srcs, dsts):
+            blocks.insert(0, Block(src, dst, frontier.numel(), seeds.numel(), frontier, seeds))
+            seeds = frontier
+        return blocks
 
     def sample_blocks(self, g, seed_nodes, exclude_eids=None):
         """Returns (input_nodes, seed_nodes, blocks); `g` is unused, as upstream."""
         seeds = seed_nodes.cuda()
+        if self.fused:
+            frontiers, srcs, dsts = torch.ops.dgs_ops._CAPI_sample_blocks(
+                seeds, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace)
+            return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts)
         blocks = []
         frontier = seeds
         for fan_out in reversed(self.fanouts):
@@ -64,3 +84,17 @@ class ChunkTensorSampler:
             blocks.insert(0, Block(coo_col, coo_row, frontier.numel(), seeds.numel(), frontier, seeds))
             seeds = frontier
         return frontier, seed_nodes, blocks
+
+    def sample_blocks_and_index(self, g, seed_nodes, chunk_features):
+        """sample_blocks followed by chunk_features._CAPI_index(input_nodes)
+        (oppo_bench/single_node/chunktensor.py:142-151), with the gather enqueued behind
+        the last hop before any length is read back.  Returns (input_nodes, seed_nodes,
+        blocks, features_of_input_nodes)."""
+        seeds = seed_nodes.cuda()
+        if not self.fused:
+            frontier, _, blocks = self.sample_blocks(g, seed_nodes)
+            return frontier, seed_nodes, blocks, chunk_features._CAPI_index(frontier)
+        frontiers, srcs, dsts, x = torch.ops.dgs_ops._CAPI_sample_blocks_and_index(
+            seeds, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
+            chunk_features)
+        return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts), x

@@ -129,6 +129,18 @@ dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
                            int32_t tier, void* stream);
 
 /*
+ * Same gather with the row count read from device memory when the kernel runs:
+ * `n_rows_dev` points to an int64 <= n_max; the launch is sized for n_max rows and
+ * `out` must hold n_max rows.  Lets a caller enqueue the gather of a frontier whose
+ * length a previous kernel on the same stream is still computing.  No counterpart in
+ * the reference (which reads every length back to the host first).
+ */
+dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
+                               int32_t index_bytes, int64_t n_max,
+                               const int64_t* n_rows_dev, void* out, int32_t tier,
+                               void* stream);
+
+/*
  * Stable partition of an index list into (device-resident rows, host-resident
  * rows): row r is "host" iff r >= threshold / row_elems
  * (src/cuda/index_with_chunk_tensor.cu:55-108; the "remote" class is empty at
@@ -233,6 +245,61 @@ dgs_status dgs_unique_relabel(dgs_segments mapping, dgs_segments requiring,
                               int64_t* num_unique_dev, dgs_segments out,
                               void* workspace, size_t workspace_bytes,
                               void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Multi-hop driver                                                          */
+/* ------------------------------------------------------------------------ */
+
+#define DGS_MAX_HOPS 8
+/* Caller-allocated edge outputs of one hop, each sized for the worst case reported by
+ * dgs_sample_blocks_plan (edges_max[h] ids). */
+typedef struct dgs_block_out {
+  void* src_local; /* rank of every picked neighbour in the hop's frontier */
+  void* dst_local; /* rank of every edge's seed in the hop's frontier      */
+} dgs_block_out;
+
+/*
+ * All hops of ChunkTensorSampler.sample_blocks
+ * (oppo_bench/single_node/utils/chunktensor_sampler.py:93-118) as one sequence of
+ * kernels with no host synchronisation: for hop h (fanouts[h], ALREADY in hop order,
+ * i.e. the reversed model fanouts) sample the current seeds, relabel
+ * ([seeds, picked], [seed of edge, picked]) and continue with the frontier as seeds.
+ * Results are identical to calling dgs_sample_neighbors (rng_stream = first_stream + h)
+ * and dgs_unique_relabel per hop.
+ *
+ * Because a hop's frontier starts with its seeds, the frontiers of successive hops are
+ * prefixes of one array: `frontier` (capacity seeds_max[n_hops] ids) receives it, and
+ * hop h's frontier is frontier[0 .. sizes[h+1]).
+ *
+ *   dgs_sample_blocks_plan : worst-case sizes; seeds_max has n_hops + 1 entries
+ *                            (seeds_max[0] = n_seeds), edges_max has n_hops
+ *   sizes_dev              : device int64[3 * n_hops + 1]:
+ *                            [0 .. n_hops]                 seeds of hop h (h = n_hops: final frontier size)
+ *                            [n_hops + 1 .. 2 n_hops]      edges of hop h
+ *                            [2 n_hops + 1 .. 3 n_hops]    non-zero if a row of hop h had degree >= 2^32
+ *   node_table / epoch     : optional persistent direct-address table of
+ *                            dgs_node_table_bytes(n_nodes) bytes (n_nodes = indptr entries - 1,
+ *                            < 2^31), filled with 0xFF bytes before its first use and then never
+ *                            cleared: pass a strictly increasing epoch (1, 2, 3, ...) with every
+ *                            call that uses it, and do not share it between calls that may run
+ *                            concurrently.  With NULL the call builds a hash table inside the
+ *                            workspace instead (one extra clearing launch, slower inserts).
+ * Fanouts above 64 are DGS_ERR_UNSUPPORTED here (use the per-hop entry points).
+ */
+dgs_status dgs_sample_blocks_plan(int64_t n_seeds, const int64_t* fanouts,
+                                  int32_t n_hops, int64_t* seeds_max,
+                                  int64_t* edges_max);
+size_t dgs_sample_blocks_workspace_bytes(int64_t n_seeds, const int64_t* fanouts,
+                                         int32_t n_hops, int32_t id_bytes);
+size_t dgs_node_table_bytes(int64_t n_nodes);
+dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seeds,
+                             dgs_view indptr, dgs_view indices,
+                             const int64_t* fanouts, int32_t n_hops, int32_t replace,
+                             uint64_t rng_seed, uint32_t first_stream,
+                             void* node_table, uint32_t node_table_epoch,
+                             void* frontier, const dgs_block_out* outs,
+                             int64_t* sizes_dev, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Small utilities                                                           */

@@ -181,3 +181,78 @@ def test_sample_blocks_driver(pkg, oracle, graph):
         ft = pkg.create_chunktensor(feats, 1, 10 ** 12, cache_rate=0.5)
         x = ft._CAPI_index(frontier)
         assert torch.equal(x.cpu(), feats[frontier.cpu()])
+
+
+def _check_blocks(blocks_gpu, o_blocks):
+    assert len(blocks_gpu) == len(o_blocks)
+    for b, ob in zip(blocks_gpu, o_blocks):
+        assert np.array_equal(_np(b.src_local), ob[0]) and np.array_equal(_np(b.dst_local), ob[1])
+        assert (b.num_src, b.num_dst) == (ob[2], ob[3])
+        assert np.array_equal(_np(b.src_ids), ob[4]) and np.array_equal(_np(b.dst_ids), ob[5])
+
+
+@pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int64, np.int64), (np.int32, np.int64), (np.int32, np.int32)])
+@pytest.mark.parametrize("fanouts,replace", [([15, 10, 5], False), ([5], False), ([3, 0, 4], False), ([64, 2], False),
+                                             ([7, 9], True), ([20, 15, 10], False)])
+def test_fused_sample_blocks_parity(pkg, oracle, id_dtype, ptr_dtype, fanouts, replace):
+    rng = np.random.default_rng(len(fanouts) * 31 + fanouts[0])
+    indptr, indices = powerlaw_graph(rng, 30000, 12, 2000, id_dtype=id_dtype, ptr_dtype=ptr_dtype)
+    t_ip, t_ix = torch.from_numpy(indptr), torch.from_numpy(indices)
+    ip_ct = pkg.create_chunktensor(t_ip, 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(t_ix, 1, 1 << 40, cache_rate=0.6)  # part of the edges in host memory
+    feats = torch.randn((30000, 36))
+    ft = pkg.create_chunktensor(feats, 1, 1 << 40, cache_rate=0.3)
+    seeds = rng.integers(0, 30000, size=700).astype(id_dtype)  # may hold duplicates
+    fused = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, replace=replace)
+    per_hop = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, replace=replace, fused=False)
+    assert fused.fused and not per_hop.fused
+    o_frontier, _, o_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, replace, 2718, 40)
+    for sampler in (fused, per_hop):
+        pkg.set_rng_state(2718, 40)
+        frontier, out_seeds, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
+        assert pkg.ops._CAPI_get_rng_state() == [2718, 40 + len(fanouts)]
+        assert np.array_equal(_np(frontier), o_frontier)
+        _check_blocks(blocks, o_blocks)
+        pkg.set_rng_state(2718, 40)
+        frontier, _, blocks, x = sampler.sample_blocks_and_index(None, torch.from_numpy(seeds), ft)
+        assert np.array_equal(_np(frontier), o_frontier)
+        _check_blocks(blocks, o_blocks)
+        assert torch.equal(x.cpu(), feats[torch.from_numpy(o_frontier).long()])
+
+
+def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph, monkeypatch):
+    capi = pkg.capi
+    indptr, indices = graph
+    ip, ix = _dev(indptr), _dev(indices)
+    rng = np.random.default_rng(77)
+    seeds = rng.permutation(20000)[:1024].astype(np.int64)
+    o_frontier, _, o_blocks = oracle.sample_blocks(seeds, indptr, indices, [15, 10, 5], False, 99, 7)
+    feats = torch.randn((20000, 100), device="cuda")
+    n_nodes = indptr.size - 1
+    node_table = torch.full((capi.lib.dgs_node_table_bytes(n_nodes) // 8,), -1, dtype=torch.int64, device="cuda")
+    epoch = 0
+    # hash table in the workspace (packed, then split slots), then the persistent node table twice
+    for mode in ("packed", "split", "direct", "direct"):
+        if mode == "split":
+            monkeypatch.setenv("DGS_FORCE_SPLIT_TABLE", "1")
+        else:
+            monkeypatch.delenv("DGS_FORCE_SPLIT_TABLE", raising=False)
+        kw = {}
+        if mode == "direct":
+            epoch += 1
+            kw = dict(node_table=node_table, epoch=epoch)
+        hops, x, flags = capi.sample_blocks(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), [5, 10, 15],
+                                            False, 99, 7, capi.tensor_view(feats), 100, torch.float32, **kw)
+        assert flags == [0, 0, 0] and len(hops) == 3
+        assert np.array_equal(_np(hops[-1][0]), o_frontier)
+        for (f, s, d), ob in zip(hops, reversed(o_blocks)):
+            assert np.array_equal(_np(f), ob[4]) and np.array_equal(_np(s), ob[0]) and np.array_equal(_np(d), ob[1])
+        assert torch.equal(x, feats[hops[-1][0]])
+    # no seeds: everything empty
+    hops, x, flags = capi.sample_blocks(_dev(seeds[:0]), capi.tensor_view(ip), capi.tensor_view(ix), [5, 10], False,
+                                        1, 0)
+    assert all(f.numel() == 0 and s.numel() == 0 for f, s, d in hops) and flags == [0, 0]
+    # fanouts above 64 are refused by the fused entry point
+    fan = (capi.c_i64 * 1)(65)
+    out = (capi.c_i64 * 2)()
+    assert capi.lib.dgs_sample_blocks_plan(10, fan, 1, out, out) == capi.DGS_ERR_UNSUPPORTED
