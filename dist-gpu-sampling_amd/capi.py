@@ -70,6 +70,8 @@ SIGNATURES = {
                                          c_u64, c_u32, c_vp, c_u32, c_vp, ctypes.POINTER(BlockOut), c_vp, c_vp,
                                          c_sz, c_vp]),
     "dgs_read_back": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp]),
+    "dgs_read_back_begin": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp, ctypes.POINTER(c_vp)]),
+    "dgs_read_back_wait": (ctypes.c_int, [c_vp]),
 }
 
 if not os.path.exists(LIB_PATH):

@@ -61,6 +61,27 @@ std::vector<int64_t> read_back(const torch::Tensor& dev, int64_t count) {
   return std::vector<int64_t>(p, p + count);
 }
 
+// The same read split around other launches: the copy is enqueued now, the host waits later.
+struct PendingRead {
+  void* ticket = nullptr;
+  int64_t count = 0;
+  const int64_t* host = nullptr;
+  std::vector<int64_t> wait() {
+    check(dgs_read_back_wait(ticket));
+    return std::vector<int64_t>(host, host + count);
+  }
+};
+PendingRead read_back_begin(const torch::Tensor& dev, int64_t count) {
+  thread_local torch::Tensor pinned =
+      torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+  TORCH_CHECK(count <= 32);
+  PendingRead r;
+  r.count = count;
+  r.host = pinned.data_ptr<int64_t>();
+  check(dgs_read_back_begin(pinned.data_ptr(), dev.data_ptr(), sizeof(int64_t) * count, current_stream(), &r.ticket));
+  return r;
+}
+
 // ---- generator state for the sampling ops ------------------------------------
 std::mutex g_rng_mutex;
 uint64_t g_rng_seed = 7777;  // upstream's constant, used until the caller sets one
@@ -401,13 +422,18 @@ sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<Chunk
   check(dgs_sample_blocks(seeds.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops, replace,
                           rng.first, rng.second, table.first, table.second, all.data_ptr(), outs.data(),
                           sizes_dev.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
+  // lengths are final here; the gather runs while the host waits for them (and after)
+  PendingRead pending = read_back_begin(sizes_dev, n_sizes);
   torch::Tensor x;
   if (features) {
     x = torch::empty({seeds_max[hops], features->elem_stride()}, opt.dtype(features->dtype()));
-    check(dgs_gather_rows_dyn(features->view(), features->elem_stride(), all.data_ptr(), w, seeds_max[hops],
-                              sizes_dev.data_ptr<int64_t>() + hops, x.data_ptr(), DGS_TIER_ANY, st));
+    const dgs_status gs = dgs_gather_rows_dyn(features->view(), features->elem_stride(), all.data_ptr(), w,
+                                              seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops, x.data_ptr(),
+                                              DGS_TIER_ANY, st);
+    if (gs != DGS_OK) pending.wait();  // never leave a ticket behind
+    check(gs);
   }
-  const std::vector<int64_t> sz = read_back(sizes_dev, n_sizes);
+  const std::vector<int64_t> sz = pending.wait();
   for (int h = 0; h < hops; ++h) {
     TORCH_CHECK(sz[2 * hops + 1 + h] == 0, "sample_blocks: a seed row of hop ", h, " has a degree of 2^32 or more");
     frontier[h] = all.narrow(0, 0, sz[h + 1]);

@@ -6,27 +6,33 @@
 // (hop h has at most S_h = S_{h-1} (1 + k_{h-1}) seeds), lengths stay in device memory,
 // grids are sized for the worst case and surplus blocks retire at once.
 //
-// Two facts make the chain short:
-//   * ranks are decided by the ORDER of mapping positions only, so a hop may use the
-//     padded positions S + i*k + l (row i, pick l) instead of the packed ones: no
-//     count/scan has to run before the picks are inserted;
-//   * the frontier of hop h is the seed list of hop h+1 and its ids already sit in the
-//     table with value = rank = position, so ONE table serves all hops, seeds are never
-//     re-inserted, only the picked ids of a hop are flagged and compacted, and the
-//     frontier is a single array that grows hop by hop.
+// What makes the chain short and cheap:
+//   * ranks depend on the ORDER of mapping positions only, so every pick gets the padded
+//     position P_h + i*k + l (hop h, row i, pick l; P_h is a host-side constant): no
+//     count/scan has to run before the picks are inserted, and positions are unique over
+//     the whole call;
+//   * a hop's frontier is the next hop's seed list, so ONE table serves all hops, holding
+//     for every id the smallest position at which it was seen; seeds are never
+//     re-inserted and the frontier is a single array that grows hop by hop;
+//   * the table is touched once per pick: the atomicMin that inserts a position also
+//     tells whether it is (so far) the smallest of its id and which position it displaced;
+//     the displaced one is marked lost.  "First occurrence" is then decided from two
+//     streamed arrays, without a second random read of the table.  Random 8-byte
+//     accesses are what bounds these kernels (about 42 G transactions/s on MI355X), so
+//     a hop costs two of them per pick: the indices read and the table atomic.
 //
 // Critical path per hop (3 launches): fill -> flag -> compact.
 //   fill     G lanes per seed row (G = 8..64): indptr pair, picks by the dgs-philox-1
-//            contract, picked id inserted at its padded position; keeps slot + row count.
-//   flag     a position is a first occurrence iff the table holds that position; counts
-//            per 1024-position tile.
+//            contract, one insert_min per pick.
+//   flag     finalises the first-occurrence bit (hop 0, whose seed list may repeat ids and
+//            whose lost marks nobody cleared, asks the table instead) and counts per
+//            1024-position tile.
 //   compact  every block sums the tile counts before its own (the list is short), ranks
-//            its first occurrences, appends them to the frontier, stores the rank in the
-//            table.
-// Off the critical path, riding as surplus blocks of the next launches: per-row pick
-// counts are scanned per 256-row tile (with flag), and the packed edge list
-// (src_local, dst_local) is written once ranks exist (with the next hop's fill, or a
-// final launch).
+//            its first occurrences, appends them to the frontier and records the rank
+//            at the position.
+// Off the critical path, as surplus blocks of later launches: per-row pick counts are
+// scanned per 256-row tile, and the packed edge list (src_local, dst_local) is written
+// (rank of a pick = rank recorded at its id's smallest position).
 #include <cstdlib>
 
 #include "common.h"
@@ -59,13 +65,16 @@ struct Hop {
   int* tile_sum;            // [row tiles]
   int* tile_flag;           // [row tiles]
   int64_t* tile_off;        // [row tiles] only when row tiles > kInlineTiles
-  uint32_t* slot;           // [seed part + s_max * k] table slot of every padded position
-  int* pos_cnt;             // [position tiles] first occurrences per tile
+  uint32_t* slot;           // [all positions] table slot of a position, bit 31 = first occurrence
+  uint32_t* rank_at;        // [all positions] rank of the id first seen at that position
+  uint8_t* lost;            // [all positions] non-zero: a smaller position of the same id exists
+  int* pos_cnt;             // [position tiles of this hop] first occurrences per tile
   int64_t* pos_off;         // [position tiles] only when position tiles > kInlineTiles
   void* frontier;           // growing array of distinct ids
   void* src_local;          // out [nnz]
   void* dst_local;          // out [nnz]
   int64_t s_max;
+  int64_t pos_base;         // first position of this hop (P_h)
   int32_t k;
   int32_t index;            // hop number
   uint32_t rng_stream;
@@ -75,10 +84,16 @@ struct Hop {
 __device__ __forceinline__ int64_t seeds_of(const Hop& h) {
   return h.n_seeds_host >= 0 ? h.n_seeds_host : *h.n_seeds;
 }
-// positions [0, seed_part) of hop 0 are the caller's seeds themselves
+// the first seed_part positions of hop 0 are the caller's seeds themselves
 __device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h.index == 0 ? s : 0; }
-// first mapping position that this hop has to flag and compact
-__device__ __forceinline__ int64_t first_position(const Hop& h, int64_t s) { return h.index == 0 ? 0 : s; }
+// rank of the first id this hop can add: later hops append behind their seeds
+__device__ __forceinline__ int64_t first_rank(const Hop& h, int64_t s) { return h.index == 0 ? 0 : s; }
+// rank of the id at position p, given p's slot word
+template <typename TableT>
+__device__ __forceinline__ uint32_t rank_of(const Hop& h, const TableT& table, int64_t p, uint32_t slot_word) {
+  if (slot_word & kFirstBit) return h.rank_at[p];
+  return h.rank_at[table.value(slot_word)];  // smallest position of the id: a first occurrence
+}
 
 template <int NT, typename T>
 __device__ __forceinline__ T block_sum(T v, T* lds /* NT/64 */) {
@@ -191,10 +206,10 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   const uint32_t rc = h.row_cnt[i];
   if (rc == kBadRow || uint32_t(l) >= rc) return;
   const int64_t o = prefix + h.row_off[i] + l;
-  const uint32_t src_slot = h.slot[seed_part(h, s) + i * k + l] & ~kFirstBit;
-  static_cast<IdT*>(h.src_local)[o] = IdT(table.value(src_slot));
+  const int64_t p = h.pos_base + seed_part(h, s) + i * k + l;
+  static_cast<IdT*>(h.src_local)[o] = IdT(rank_of(h, table, p, h.slot[p]));
   static_cast<IdT*>(h.dst_local)[o] =
-      h.index == 0 ? IdT(table.value(h.slot[i] & ~kFirstBit)) : IdT(i);
+      h.index == 0 ? IdT(rank_of(h, table, h.pos_base + i, h.slot[h.pos_base + i])) : IdT(i);
 }
 
 inline int64_t relabel_blocks(int64_t s_max, int k) {
@@ -203,12 +218,24 @@ inline int64_t relabel_blocks(int64_t s_max, int k) {
 
 // ---- critical path ------------------------------------------------------------------------
 
+// Marks `displaced` (a position of this call) as no longer the smallest of its id.
+__device__ __forceinline__ void mark_lost(const Hop& h, uint32_t displaced) {
+  if (displaced != kNoPosition) h.lost[displaced] = 1;
+}
+
 template <typename IdT, typename PtrT, typename TableT, int G>
-__global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64_t fill_blocks, TableT table,
-                                                          TierView<PtrT> indptr, TierView<IdT> indices,
-                                                          bool replace, uint64_t rng_seed) {
-  if (int64_t(blockIdx.x) >= fill_blocks) {  // surplus blocks: edge list of the previous hop
-    relabel_tile<IdT, TableT>(prev, table, int64_t(blockIdx.x) - fill_blocks);
+__global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64_t fill_blocks,
+                                                          int64_t relabel_count, uint4* clear_begin,
+                                                          int64_t clear_n16, TableT table, TierView<PtrT> indptr,
+                                                          TierView<IdT> indices, bool replace, uint64_t rng_seed) {
+  if (int64_t(blockIdx.x) >= fill_blocks) {
+    const int64_t b = int64_t(blockIdx.x) - fill_blocks;
+    if (b < relabel_count) {  // surplus blocks: edge list of the previous hop
+      relabel_tile<IdT, TableT>(prev, table, b);
+    } else {                  // surplus blocks of hop 0: clear the lost marks of the later hops
+      const int64_t i = (b - relabel_count) * kBlock + threadIdx.x;
+      if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
     return;
   }
   const int64_t s = seeds_of(h);
@@ -226,21 +253,30 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
   const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
   const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;
-  const int64_t sp = seed_part(h, s);
   if (l == 0) {
     h.row_cnt[i] = bad ? kBadRow : (replace ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
-    if (h.index == 0) h.slot[i] = table.insert(seed, uint32_t(i));
+    if (h.index == 0) {  // the caller's seeds open the mapping list; flag() decides their first bits
+      bool first;
+      uint32_t displaced;
+      h.slot[h.pos_base + i] = table.insert_min(seed, uint32_t(h.pos_base + i), &first, &displaced);
+    }
   }
   uint32_t pos;
   const bool have = pick_position<G>(deg, k, replace, l, group_lane0, rng_seed, h.rng_stream, row, &pos);
   if (l < k) {
-    const int64_t rel = sp + i * k + l;
-    uint32_t sl = kInvalidSlot;
+    const int64_t p = h.pos_base + seed_part(h, s) + i * k + l;
+    uint32_t word = kInvalidSlot;
     if (have) {
       const IdT col = indices.at(b + pos);
-      sl = table.insert(col, uint32_t(first_position(h, s) + rel));
+      bool first;
+      uint32_t displaced;
+      word = table.insert_min(col, uint32_t(p), &first, &displaced);
+      if (h.index != 0) {
+        if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
+        mark_lost(h, displaced);
+      }
     }
-    h.slot[rel] = sl;
+    h.slot[p] = word;
   }
 }
 
@@ -253,17 +289,22 @@ __global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_bl
   __shared__ int lds[kBlock / kWave];
   const int64_t s = seeds_of(h);
   const int64_t len = seed_part(h, s) + s * h.k;
-  const int64_t p0 = first_position(h, s);
   const int64_t base = int64_t(blockIdx.x) * kPosTile + threadIdx.x * kPosItems;
   int c = 0;
 #pragma unroll
   for (int j = 0; j < kPosItems; ++j) {
     const int64_t rel = base + j;
     if (rel < len) {
-      const uint32_t sl = h.slot[rel];
-      if (sl != kInvalidSlot && table.value(sl) == uint32_t(p0 + rel)) {
-        h.slot[rel] = sl | kFirstBit;
-        ++c;
+      const int64_t p = h.pos_base + rel;
+      const uint32_t w = h.slot[p];
+      if (w == kInvalidSlot) continue;
+      if (h.index == 0) {
+        if (table.value(w) == uint32_t(p)) {
+          h.slot[p] = w | kFirstBit;
+          ++c;
+        }
+      } else if (w & kFirstBit) {
+        if (h.lost[p]) h.slot[p] = w & ~kFirstBit; else ++c;
       }
     }
   }
@@ -291,7 +332,7 @@ __global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, TableT table
   const int64_t s = seeds_of(h);
   const int64_t len = seed_part(h, s) + s * h.k;
   const int64_t tiles = (len + kPosTile - 1) / kPosTile;
-  const int64_t rank0 = first_position(h, s);  // hop 0 starts at rank 0, later hops after the seeds
+  const int64_t rank0 = first_rank(h, s);
   const int64_t tile = blockIdx.x;
   if (tile >= tiles && tile != 0) return;
   // first occurrences in the tiles before this one (block 0 also needs the grand total)
@@ -309,22 +350,21 @@ __global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, TableT table
   if (tile == 0 && threadIdx.x == 0) *h.n_unique = rank0 + all;
   if (tile >= tiles) return;
   const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
-  uint32_t sl[kPosItems];
+  uint32_t w[kPosItems];
   int c = 0;
 #pragma unroll
   for (int j = 0; j < kPosItems; ++j) {
-    sl[j] = base + j < len ? h.slot[base + j] : kInvalidSlot;
-    if (sl[j] == kInvalidSlot) sl[j] = 0;  // bit 31 clear: not a first occurrence
-    c += (sl[j] & kFirstBit) != 0;
+    w[j] = base + j < len ? h.slot[h.pos_base + base + j] : kInvalidSlot;
+    if (w[j] == kInvalidSlot) w[j] = 0;  // bit 31 clear: not a first occurrence
+    c += (w[j] & kFirstBit) != 0;
   }
   int total;
   int64_t rank = rank0 + before + block_exclusive_scan<kBlock, int>(c, &total, lds);
 #pragma unroll
   for (int j = 0; j < kPosItems; ++j) {
-    if (sl[j] & kFirstBit) {
-      const uint32_t slot = sl[j] & ~kFirstBit;
-      static_cast<IdT*>(h.frontier)[rank] = table.key(slot);
-      table.set_value(slot, uint32_t(rank));
+    if (w[j] & kFirstBit) {
+      static_cast<IdT*>(h.frontier)[rank] = table.key(w[j] & ~kFirstBit);
+      h.rank_at[h.pos_base + base + j] = uint32_t(rank);
       ++rank;
     }
   }
@@ -390,6 +430,11 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
   Carver c(base);
   char* t = c.take<char>(p.table_bytes);
   if (table) *table = t;
+  const size_t positions = size_t(p.s_max[p.n_hops]);  // sum over hops of (seed part + s_max * k)
+  uint32_t* slot = c.take<uint32_t>(positions);
+  uint32_t* rank_at = c.take<uint32_t>(positions);
+  uint8_t* lost = c.take<uint8_t>(positions + 16);
+  int64_t pos_base = 0;
   for (int h = 0; h < p.n_hops; ++h) {
     const size_t s = size_t(p.s_max[h]);
     const size_t len = (h == 0 ? s : 0) + size_t(p.nnz_max[h]);
@@ -401,24 +446,31 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
     v.tile_sum = c.take<int>(row_tiles);
     v.tile_flag = c.take<int>(row_tiles);
     v.tile_off = row_tiles > size_t(kInlineTiles) ? c.take<int64_t>(row_tiles) : nullptr;
-    v.slot = c.take<uint32_t>(len);
+    v.slot = slot;
+    v.rank_at = rank_at;
+    v.lost = lost;
     v.pos_cnt = c.take<int>(pos_tiles + 1);
     v.pos_off = pos_tiles > size_t(kInlineTiles) ? c.take<int64_t>(pos_tiles) : nullptr;
     v.s_max = p.s_max[h];
+    v.pos_base = pos_base;
     v.k = int32_t(fanouts[h]);
     v.index = h;
     if (hops) hops[h] = v;
+    pos_base += int64_t(len);
   }
   return c.used + 256;
 }
 
 template <typename IdT, typename PtrT, typename TableT, int G>
-void launch_fill(const Hop& cur, const Hop& prev, int64_t surplus, const TableT& table, const dgs_view& indptr,
-                 const dgs_view& indices, bool replace, uint64_t rng_seed, hipStream_t st) {
+void launch_fill(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* clear_begin, int64_t clear_n16,
+                 const TableT& table, const dgs_view& indptr, const dgs_view& indices, bool replace,
+                 uint64_t rng_seed, hipStream_t st) {
   const int64_t fill_blocks = (cur.s_max * G + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G>), dim3(uint32_t(fill_blocks + surplus)), dim3(kBlock), 0,
-                     st, cur, prev, fill_blocks, table, TierView<PtrT>(indptr), TierView<IdT>(indices), replace,
-                     rng_seed);
+  const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G>),
+                     dim3(uint32_t(fill_blocks + relabel_count + clear_blocks)), dim3(kBlock), 0, st, cur, prev,
+                     fill_blocks, relabel_count, clear_begin, clear_n16, table, TierView<PtrT>(indptr),
+                     TierView<IdT>(indices), replace, rng_seed);
 }
 
 template <typename IdT, typename PtrT, typename TableT>
@@ -428,10 +480,20 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
     const Hop& cur = hops[h];
     const Hop prev = h > 0 ? hops[h - 1] : Hop{};
     const int64_t surplus = h > 0 ? relabel_blocks(prev.s_max, prev.k) : 0;
-    if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
-    else if (cur.k <= 16) launch_fill<IdT, PtrT, TableT, 16>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
-    else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
-    else launch_fill<IdT, PtrT, TableT, 64>(cur, prev, surplus, table, indptr, indices, replace, rng_seed, st);
+    // the launch of hop 0 also clears the lost marks of all later hops (16-byte granules; the
+    // first one may reach back into hop 0's own range, whose marks are never read or written)
+    uint4* clear_begin = nullptr;
+    int64_t clear_n16 = 0;
+    if (h == 0 && p.n_hops > 1) {
+      const int64_t first = hops[1].pos_base / 16 * 16;
+      const int64_t last = (p.s_max[p.n_hops] + 15) / 16 * 16;  // the array has 16 spare bytes
+      clear_begin = reinterpret_cast<uint4*>(cur.lost + first);
+      clear_n16 = last > first ? (last - first) / 16 : 0;
+    }
+    if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
+    else if (cur.k <= 16) launch_fill<IdT, PtrT, TableT, 16>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
+    else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
+    else launch_fill<IdT, PtrT, TableT, 64>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     DGS_LAUNCH_CHECK();
 
     const int64_t len_max = (h == 0 ? cur.s_max : 0) + cur.s_max * cur.k;

@@ -3,6 +3,8 @@
 // (upstream src/chunk_tensor.cc:112-139) have no counterpart here.
 #include <atomic>
 #include <cstdarg>
+#include <mutex>
+#include <vector>
 #include <cstring>
 #include <new>
 
@@ -166,5 +168,46 @@ DGS_API dgs_status dgs_read_back(void* host_dst, const void* dev_src, size_t n_b
   hipStream_t st = static_cast<hipStream_t>(stream);
   DGS_HIP_TRY(hipMemcpyAsync(host_dst, dev_src, n_bytes, hipMemcpyDeviceToHost, st));
   DGS_HIP_TRY(hipStreamSynchronize(st));
+  return DGS_OK;
+}
+
+namespace dgs {
+// Recycled events for dgs_read_back_begin/_wait (default flags plus no timing).
+static std::mutex g_event_mutex;
+static std::vector<hipEvent_t> g_event_pool;
+}  // namespace dgs
+
+DGS_API dgs_status dgs_read_back_begin(void* host_dst, const void* dev_src, size_t n_bytes, void* stream,
+                                       void** ticket) {
+  DGS_REQUIRE(host_dst != nullptr && dev_src != nullptr && ticket != nullptr, DGS_ERR_INVALID,
+              "read_back_begin: null pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipEvent_t ev = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
+    if (!dgs::g_event_pool.empty()) {
+      ev = dgs::g_event_pool.back();
+      dgs::g_event_pool.pop_back();
+    }
+  }
+  if (ev == nullptr) DGS_HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  DGS_HIP_TRY(hipMemcpyAsync(host_dst, dev_src, n_bytes, hipMemcpyDeviceToHost, st));
+  DGS_HIP_TRY(hipEventRecord(ev, st));
+  *ticket = ev;
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_read_back_wait(void* ticket) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "read_back_wait: null ticket");
+  hipEvent_t ev = static_cast<hipEvent_t>(ticket);
+  const hipError_t e = hipEventSynchronize(ev);
+  {
+    std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
+    dgs::g_event_pool.push_back(ev);
+  }
+  if (e != hipSuccess) {
+    dgs::set_error("read_back_wait: %s", hipGetErrorString(e));
+    return DGS_ERR_HIP;
+  }
   return DGS_OK;
 }

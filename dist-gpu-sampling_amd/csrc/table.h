@@ -1,7 +1,9 @@
 // Device-side open-addressing tables for unique/relabel (linear probing, capacity 2^m).
 //
 // A table maps a node id to the smallest position at which it occurs in the mapping
-// list; after compaction the same field holds the id's rank among the distinct ids.
+// list.  unique.hip later overwrites that field with the id's rank (set_value); the
+// multi-hop pipeline keeps positions and learns from insert_min() whether a position
+// is, so far, the smallest of its id and which position it displaced.
 //   packed   one 64-bit word per slot: id in the high half, position/rank in the low
 //            half (ids must be < 2^32 - 1); insertion is a single 64-bit atomic;
 //   split    id array + uint32 value array (any 64-bit id >= 0).
@@ -26,6 +28,8 @@ template <typename IdT> struct AtomicWord;
 template <> struct AtomicWord<int64_t> { using type = unsigned long long; };
 template <> struct AtomicWord<int32_t> { using type = unsigned int; };
 
+constexpr uint32_t kNoPosition = 0xffffffffu;
+
 template <typename IdT, bool PACKED> struct Table;
 
 template <typename IdT>
@@ -49,6 +53,27 @@ struct Table<IdT, true> {
       }
       if (uint32_t(cur >> 32) == uint32_t(key)) {
         if (uint32_t(cur) > idx) atomicMin(slots + pos, packed);
+        return pos;
+      }
+      pos = (pos + 1) & mask;
+    }
+  }
+  // Same, reporting whether idx became the smallest position of its key (*first) and, if it
+  // replaced a larger one, which (*displaced, else kNoPosition).
+  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced) const {
+    const unsigned long long packed = (static_cast<unsigned long long>(uint32_t(key)) << 32) | idx;
+    uint32_t pos = hash_id(uint32_t(key)) & mask;
+    *displaced = kNoPosition;
+    for (;;) {
+      unsigned long long cur = slots[pos];
+      if (cur == kEmpty) {
+        cur = atomicCAS(slots + pos, kEmpty, packed);
+        if (cur == kEmpty) { *first = true; return pos; }
+      }
+      if (uint32_t(cur >> 32) == uint32_t(key)) {
+        const unsigned long long old = atomicMin(slots + pos, packed);
+        *first = old > packed;
+        if (*first) *displaced = uint32_t(old);
         return pos;
       }
       pos = (pos + 1) & mask;
@@ -96,6 +121,20 @@ struct Table<IdT, false> {
     atomicMin(vals + pos, idx);
     return pos;
   }
+  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced) const {
+    using W = typename AtomicWord<IdT>::type;
+    uint32_t pos = hash_id(uint64_t(int64_t(key))) & mask;
+    for (;;) {
+      IdT cur = keys[pos];
+      if (cur == IdT(-1)) cur = IdT(atomicCAS(reinterpret_cast<W*>(keys + pos), W(IdT(-1)), W(key)));
+      if (cur == IdT(-1) || cur == key) break;
+      pos = (pos + 1) & mask;
+    }
+    const uint32_t old = atomicMin(vals + pos, idx);
+    *first = old > idx;
+    *displaced = (*first && old != 0xffffffffu) ? old : kNoPosition;
+    return pos;
+  }
   __device__ __forceinline__ uint32_t value(uint32_t slot) const { return vals[slot]; }
   __device__ __forceinline__ IdT key(uint32_t slot) const { return keys[slot]; }
   __device__ __forceinline__ void set_value(uint32_t slot, uint32_t v) const { vals[slot] = v; }
@@ -124,17 +163,16 @@ struct DirectTable {
   __host__ __device__ DirectTable(void* base, uint32_t epoch)
       : entries(static_cast<unsigned long long*>(base)), tag(~epoch) {}
 
-  __device__ __forceinline__ uint32_t insert(IdT key, uint32_t idx) const {
+  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced) const {
     const unsigned long long v = (static_cast<unsigned long long>(tag) << 32) | idx;
-    unsigned long long* e = entries + uint32_t(key);
-    if (*e > v) atomicMin(e, v);  // a stale read can only be larger than the truth
+    const unsigned long long old = atomicMin(entries + uint32_t(key), v);
+    *first = old > v;
+    // an entry of this use that was larger: that position is no longer its id's smallest
+    *displaced = (*first && uint32_t(old >> 32) == tag) ? uint32_t(old) : kNoPosition;
     return uint32_t(key);
   }
   __device__ __forceinline__ uint32_t value(uint32_t slot) const { return uint32_t(entries[slot]); }
   __device__ __forceinline__ IdT key(uint32_t slot) const { return IdT(slot); }
-  __device__ __forceinline__ void set_value(uint32_t slot, uint32_t v) const {
-    reinterpret_cast<uint32_t*>(entries)[2 * size_t(slot)] = v;  // low half (little endian)
-  }
 };
 
 // capacity for n keys: power of two >= 1.4 n (load factor <= 0.72, ~0.5 typical), >= 1024

@@ -312,6 +312,16 @@ dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seed
  */
 dgs_status dgs_read_back(void* host_dst, const void* dev_src, size_t n_bytes,
                          void* stream);
+/*
+ * The same read in two halves: _begin enqueues the copy on `stream` and marks that point,
+ * _wait blocks until the copy (not later work on the stream) has finished.  Work enqueued
+ * between the two keeps the GPU busy while the host waits for the lengths.  `host_dst`
+ * should be pinned memory and must stay untouched until _wait returns.  Every ticket must
+ * be waited on exactly once.
+ */
+dgs_status dgs_read_back_begin(void* host_dst, const void* dev_src, size_t n_bytes,
+                               void* stream, void** ticket);
+dgs_status dgs_read_back_wait(void* ticket);
 
 #ifdef __cplusplus
 }
