@@ -256,3 +256,21 @@ def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph, monkeypat
     fan = (capi.c_i64 * 1)(65)
     out = (capi.c_i64 * 2)()
     assert capi.lib.dgs_sample_blocks_plan(10, fan, 1, out, out) == capi.DGS_ERR_UNSUPPORTED
+
+
+def test_fused_long_tile_lists(pkg, oracle):
+    # > 2048 position tiles and > 2048 row tiles in the last hop: the separate scan launches
+    rng = np.random.default_rng(5)
+    indptr, indices = powerlaw_graph(rng, 1_000_000, 6, 200, zero_frac=0.1)
+    seeds = rng.permutation(1_000_000)[:60_000].astype(np.int64)
+    fanouts = [9, 40]  # hop order: 40 first, then 9 over ~1.5M rows
+    o_frontier, _, o_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, True, 11, 0)
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, replace=True)
+    pkg.set_rng_state(11, 0)
+    frontier, _, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
+    assert np.array_equal(_np(frontier), o_frontier)
+    _check_blocks(blocks, o_blocks)
+    # the launch plan is sized by the worst case: 60000 * 41 rows and 9 times as many positions
+    assert 60_000 * 41 > 2048 * 256 and blocks[0].num_dst > 200_000
