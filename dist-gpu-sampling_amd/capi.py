@@ -68,10 +68,14 @@ SIGNATURES = {
     "dgs_node_table_bytes": (c_sz, [c_i64]),
     "dgs_sample_blocks": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, ctypes.POINTER(c_i64), c_i32, c_i32,
                                          c_u64, c_u32, c_vp, c_u32, c_vp, ctypes.POINTER(BlockOut), c_vp, c_vp,
-                                         c_sz, c_vp]),
+                                         ctypes.POINTER(c_vp), c_vp, c_sz, c_vp]),
     "dgs_read_back": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp]),
     "dgs_read_back_begin": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp, ctypes.POINTER(c_vp)]),
     "dgs_read_back_wait": (ctypes.c_int, [c_vp]),
+    "dgs_ticket_record": (ctypes.c_int, [c_vp, ctypes.POINTER(c_vp)]),
+    "dgs_ticket_stream_wait": (ctypes.c_int, [c_vp, c_vp]),
+    "dgs_ticket_wait": (ctypes.c_int, [c_vp]),
+    "dgs_ticket_release": (ctypes.c_int, [c_vp]),
 }
 
 if not os.path.exists(LIB_PATH):
@@ -239,7 +243,7 @@ def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_se
     ws = _ws(nb, seeds.device)
     check(lib.dgs_sample_blocks(seeds.data_ptr(), w, n, indptr_view, indices_view, fan, hops, int(replace),
                                 rng_seed, first_stream, node_table.data_ptr() if node_table is not None else None,
-                                epoch, frontier.data_ptr(), outs, sizes.data_ptr(), ws.data_ptr(), nb,
+                                epoch, frontier.data_ptr(), outs, sizes.data_ptr(), None, None, ws.data_ptr(), nb,
                                 stream_ptr()))
     x = None
     if feature_view is not None:

@@ -211,6 +211,7 @@ class ChunkTensor : public torch::CustomClassHolder {
   }
 
   const dgs_view& view() const { return view_; }
+  c10::Device device() const { return device_; }
   torch::ScalarType dtype() const { return dtype_; }
   int64_t elem_stride() const { return elem_stride_; }
 
@@ -382,15 +383,20 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> TensorRelabel(std::vector<
 }
 
 // All hops of the sampler loop (chunktensor_sampler.py:93-118) in one call with a single
-// blocking length read at the end.  `fanouts` is in hop order (the reversed model
-// fanouts).  Returns per hop, nearest the seeds first: frontier (= the hop's source ids,
-// seeds first), src_local, dst_local -- and, when `features` is given, the gathered
-// feature rows of the last frontier, enqueued before the lengths are known.
-std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor>
+// blocking wait for the lengths.  `fanouts` is in hop order (the reversed model fanouts).
+// Returns per hop, nearest the seeds first: frontier (= the hop's source ids, seeds first;
+// all views of one array), src_local, dst_local -- and, when `features` is given, the
+// gathered feature rows of the last frontier, enqueued before the lengths are known.
+//
+// Seeds may also arrive on the host, as the upstream sampler receives them
+// (chunktensor_sampler.py:94); they are uploaded on the caller's stream.  (Running the
+// sampling half on a second stream so that it overlaps the previous call's gather was
+// measured and dropped: the cross-stream waits cost more than the overlap saved.)
+std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor,
+           torch::Tensor>
 sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<ChunkTensor>& indptr,
                    const c10::intrusive_ptr<ChunkTensor>& indices, const std::vector<int64_t>& fanouts,
                    bool replace, const c10::intrusive_ptr<ChunkTensor>& features) {
-  DGS_CHECK_GPU(seeds_in);
   const int32_t w = id_width(seeds_in, "seeds");
   TORCH_CHECK(seeds_in.scalar_type() == indices->dtype(), "seeds (", seeds_in.scalar_type(), ") and indices (",
               indices->dtype(), ") must have the same dtype");
@@ -398,11 +404,21 @@ sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<Chunk
               "indptr store must be int32 or int64");
   const int32_t hops = static_cast<int32_t>(fanouts.size());
   TORCH_CHECK(hops >= 1 && hops <= DGS_MAX_HOPS, "sample_blocks: between 1 and ", DGS_MAX_HOPS, " fanouts");
-  torch::Tensor seeds = seeds_in.contiguous().view({-1});
-  const int64_t n = seeds.numel();
+  const int64_t n = seeds_in.numel();
   std::vector<int64_t> seeds_max(hops + 1), edges_max(hops);
   check(dgs_sample_blocks_plan(n, fanouts.data(), hops, seeds_max.data(), edges_max.data()));
+  const int n_sizes = 3 * hops + 1;
+  TORCH_CHECK(n_sizes <= 32);
 
+  const c10::Device dev = indptr->device();
+  TORCH_CHECK(seeds_in.device().is_cpu() || seeds_in.device() == dev, "seeds must be on the host or on ", dev);
+  void* st = current_stream();
+
+  thread_local torch::Tensor pinned =
+      torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+  int64_t* sizes_host = pinned.data_ptr<int64_t>();
+
+  torch::Tensor seeds = seeds_in.to(dev, /*non_blocking=*/true).contiguous().view({-1});
   const auto opt = seeds.options();
   std::vector<torch::Tensor> frontier(hops), src(hops), dst(hops);
   std::vector<dgs_block_out> outs(hops);
@@ -412,28 +428,28 @@ sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<Chunk
     dst[h] = torch::empty({edges_max[h]}, opt);
     outs[h] = dgs_block_out{src[h].data_ptr(), dst[h].data_ptr()};
   }
-  const int n_sizes = 3 * hops + 1;
   torch::Tensor sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
   const size_t ws_bytes = dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
-  torch::Tensor ws = device_bytes(ws_bytes, seeds.device());
+  torch::Tensor ws = device_bytes(ws_bytes, dev);
   const auto rng = next_rng(static_cast<uint32_t>(hops));
   const auto table = indptr->node_table();
-  void* st = current_stream();
+  void* ticket = nullptr;
   check(dgs_sample_blocks(seeds.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops, replace,
                           rng.first, rng.second, table.first, table.second, all.data_ptr(), outs.data(),
-                          sizes_dev.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
-  // lengths are final here; the gather runs while the host waits for them (and after)
-  PendingRead pending = read_back_begin(sizes_dev, n_sizes);
+                          sizes_dev.data_ptr<int64_t>(), sizes_host, &ticket, ws.data_ptr(), ws_bytes, st));
+  // the lengths are final at the ticket; the gather is enqueued before the host waits for them
   torch::Tensor x;
+  dgs_status gs = DGS_OK;
   if (features) {
-    x = torch::empty({seeds_max[hops], features->elem_stride()}, opt.dtype(features->dtype()));
-    const dgs_status gs = dgs_gather_rows_dyn(features->view(), features->elem_stride(), all.data_ptr(), w,
-                                              seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops, x.data_ptr(),
-                                              DGS_TIER_ANY, st);
-    if (gs != DGS_OK) pending.wait();  // never leave a ticket behind
-    check(gs);
+    x = torch::empty({seeds_max[hops], features->elem_stride()},
+                     torch::TensorOptions().dtype(features->dtype()).device(dev));
+    gs = dgs_gather_rows_dyn(features->view(), features->elem_stride(), all.data_ptr(), w, seeds_max[hops],
+                             sizes_dev.data_ptr<int64_t>() + hops, x.data_ptr(), DGS_TIER_ANY, st);
   }
-  const std::vector<int64_t> sz = pending.wait();
+  const dgs_status ws_status = dgs_ticket_wait(ticket);  // never leave a ticket behind
+  check(gs);
+  check(ws_status);
+  const std::vector<int64_t> sz(sizes_host, sizes_host + n_sizes);
   for (int h = 0; h < hops; ++h) {
     TORCH_CHECK(sz[2 * hops + 1 + h] == 0, "sample_blocks: a seed row of hop ", h, " has a degree of 2^32 or more");
     frontier[h] = all.narrow(0, 0, sz[h + 1]);
@@ -441,17 +457,19 @@ sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<Chunk
     dst[h] = dst[h].narrow(0, 0, sz[hops + 1 + h]);
   }
   if (features) x = x.narrow(0, 0, sz[hops]);
-  return std::make_tuple(frontier, src, dst, x);
+  return std::make_tuple(frontier, src, dst, x, seeds);
 }
 
-std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>> SampleBlocks(
-    torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr, c10::intrusive_ptr<ChunkTensor> indices,
-    std::vector<int64_t> fanouts, bool replace) {
-  auto r = sample_blocks_impl(seeds, indptr, indices, fanouts, replace, c10::intrusive_ptr<ChunkTensor>());
-  return std::make_tuple(std::get<0>(r), std::get<1>(r), std::get<2>(r));
-}
-
+// Both operators also return the seeds as a device tensor (the upload they did anyway).
 std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor>
+SampleBlocks(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr, c10::intrusive_ptr<ChunkTensor> indices,
+             std::vector<int64_t> fanouts, bool replace) {
+  auto r = sample_blocks_impl(seeds, indptr, indices, fanouts, replace, c10::intrusive_ptr<ChunkTensor>());
+  return std::make_tuple(std::get<0>(r), std::get<1>(r), std::get<2>(r), std::get<4>(r));
+}
+
+std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor,
+           torch::Tensor>
 SampleBlocksAndIndex(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr,
                      c10::intrusive_ptr<ChunkTensor> indices, std::vector<int64_t> fanouts, bool replace,
                      c10::intrusive_ptr<ChunkTensor> features) {

@@ -60,6 +60,9 @@ struct Hop {
   int64_t* n_unique;        // device scalar: frontier size after this hop
   int64_t* nnz;             // device scalar: edges of this hop
   int64_t* flags;           // device scalar: non-zero on a bad row
+  int64_t* host_sizes;      // optional pinned mirror of the whole sizes array (NULL: none)
+  int32_t n_hops;           // layout of the mirror: [0..H] seeds, then H edge counts, then H flags
+  int32_t pad0_;
   uint32_t* row_cnt;        // [s_max] picks of every row (kBadRow on error)
   uint32_t* row_off;        // [s_max] exclusive offset of the row inside its 256-row tile
   int* tile_sum;            // [row tiles]
@@ -172,20 +175,6 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   const int64_t s = seeds_of(h);
   const int64_t tiles = (s + kRowTile - 1) / kRowTile;
   const int k = h.k;
-  if (b == 0) {  // totals of the hop, written even when there is nothing to do
-    int64_t sum = 0;
-    int64_t bad = 0;
-    for (int64_t j = threadIdx.x; j < tiles; j += kBlock) {
-      sum += h.tile_sum[j];
-      bad += h.tile_flag[j];
-    }
-    sum = block_sum<kBlock, int64_t>(sum, lds);
-    bad = block_sum<kBlock, int64_t>(bad, lds);
-    if (threadIdx.x == 0) {
-      *h.nnz = sum;
-      *h.flags = bad != 0;
-    }
-  }
   if (k == 0) return;
   const int64_t tile = b / k;
   const int chunk = int(b - tile * k);
@@ -213,7 +202,7 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
 }
 
 inline int64_t relabel_blocks(int64_t s_max, int k) {
-  return k > 0 ? ((s_max + kRowTile - 1) / kRowTile) * k : 1;
+  return ((s_max + kRowTile - 1) / kRowTile) * k;
 }
 
 // ---- critical path ------------------------------------------------------------------------
@@ -347,7 +336,29 @@ __global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, TableT table
     part = block_sum<kBlock, int64_t>(part, lds64);
     if (tile == 0) all = part; else before = part;
   }
-  if (tile == 0 && threadIdx.x == 0) *h.n_unique = rank0 + all;
+  if (tile == 0) {
+    // this hop's lengths, written even when there is nothing to do: frontier size, edge count
+    // (row tiles were scanned by the surplus blocks of the flag launch) and error flag
+    const int64_t row_tiles = (s + kRowTile - 1) / kRowTile;
+    int64_t edges = 0, bad = 0;
+    for (int64_t j = threadIdx.x; j < row_tiles; j += kBlock) {
+      edges += h.tile_sum[j];
+      bad += h.tile_flag[j];
+    }
+    edges = block_sum<kBlock, int64_t>(edges, lds64);
+    bad = block_sum<kBlock, int64_t>(bad, lds64);
+    if (threadIdx.x == 0) {
+      *h.n_unique = rank0 + all;
+      *h.nnz = edges;
+      *h.flags = bad != 0;
+      if (h.host_sizes) {
+        if (h.index == 0) h.host_sizes[0] = s;
+        h.host_sizes[h.index + 1] = rank0 + all;
+        h.host_sizes[h.n_hops + 1 + h.index] = edges;
+        h.host_sizes[2 * h.n_hops + 1 + h.index] = bad != 0;
+      }
+    }
+  }
   if (tile >= tiles) return;
   const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
   uint32_t w[kPosItems];
@@ -475,7 +486,8 @@ void launch_fill(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* 
 
 template <typename IdT, typename PtrT, typename TableT>
 dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_view& indptr,
-                      const dgs_view& indices, bool replace, uint64_t rng_seed, hipStream_t st) {
+                      const dgs_view& indices, bool replace, uint64_t rng_seed, void** sizes_ticket,
+                      hipStream_t st) {
   for (int h = 0; h < p.n_hops; ++h) {
     const Hop& cur = hops[h];
     const Hop prev = h > 0 ? hops[h - 1] : Hop{};
@@ -514,29 +526,36 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
                        dim3(kBlock), 0, st, cur, table);
     DGS_LAUNCH_CHECK();
   }
+  // every length is final here: mark the point the caller may wait for
+  if (sizes_ticket) {
+    const dgs_status ts = dgs_ticket_record(st, sizes_ticket);
+    if (ts != DGS_OK) return ts;
+  }
   const Hop& last = hops[p.n_hops - 1];
-  hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT>), dim3(uint32_t(relabel_blocks(last.s_max, last.k))),
-                     dim3(kBlock), 0, st, last, table);
-  DGS_LAUNCH_CHECK();
+  if (relabel_blocks(last.s_max, last.k) > 0) {
+    hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT>), dim3(uint32_t(relabel_blocks(last.s_max, last.k))),
+                       dim3(kBlock), 0, st, last, table);
+    DGS_LAUNCH_CHECK();
+  }
   return DGS_OK;
 }
 
 template <typename IdT, typename PtrT>
 dgs_status run_blocks_table(const Plan& p, Hop* hops, void* hash_table, void* node_table, uint32_t epoch,
                             const dgs_view& indptr, const dgs_view& indices, bool replace, uint64_t rng_seed,
-                            hipStream_t st) {
+                            void** sizes_ticket, hipStream_t st) {
   if (p.kind == TableKind::kDirect)
     return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch), indptr, indices,
-                                                   replace, rng_seed, st);
+                                                   replace, rng_seed, sizes_ticket, st);
   const int64_t n16 = int64_t(p.table_bytes / 16);
   hipLaunchKernelGGL(clear_kernel, dim3(uint32_t((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                      static_cast<uint4*>(hash_table), n16);
   DGS_LAUNCH_CHECK();
   if (p.kind == TableKind::kPacked)
     return run_blocks<IdT, PtrT, Table<IdT, true>>(p, hops, Table<IdT, true>(hash_table, p.capacity), indptr,
-                                                   indices, replace, rng_seed, st);
+                                                   indices, replace, rng_seed, sizes_ticket, st);
   return run_blocks<IdT, PtrT, Table<IdT, false>>(p, hops, Table<IdT, false>(hash_table, p.capacity), indptr,
-                                                  indices, replace, rng_seed, st);
+                                                  indices, replace, rng_seed, sizes_ticket, st);
 }
 
 }  // namespace
@@ -571,7 +590,8 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
                                      dgs_view indices, const int64_t* fanouts, int32_t n_hops, int32_t replace,
                                      uint64_t rng_seed, uint32_t first_stream, void* node_table,
                                      uint32_t node_table_epoch, void* frontier, const dgs_block_out* outs,
-                                     int64_t* sizes_dev, void* workspace, size_t workspace_bytes, void* stream) {
+                                     int64_t* sizes_dev, int64_t* sizes_host, void** sizes_ticket,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
   using namespace dgs;
   Plan p;
   // node count = indptr entries - 1
@@ -584,9 +604,15 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
   DGS_REQUIRE(node_table == nullptr || (node_table_epoch >= 1 && node_table_epoch < 0xfffffff0u), DGS_ERR_INVALID,
               "sample_blocks: node table epoch %u outside 1..2^32-17 (refill the table with 0xFF and restart at 1)",
               node_table_epoch);
+  DGS_REQUIRE((sizes_host == nullptr) == (sizes_ticket == nullptr), DGS_ERR_INVALID,
+              "sample_blocks: sizes_host and sizes_ticket go together");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n_seeds == 0) {  // nothing to launch: every size is zero
     DGS_HIP_TRY(hipMemsetAsync(sizes_dev, 0, sizeof(int64_t) * size_t(3 * n_hops + 1), st));
+    if (sizes_host) {
+      for (int i = 0; i < 3 * n_hops + 1; ++i) sizes_host[i] = 0;
+      return dgs_ticket_record(st, sizes_ticket);
+    }
     return DGS_OK;
   }
   DGS_REQUIRE(seeds != nullptr && frontier != nullptr, DGS_ERR_INVALID, "sample_blocks: null seeds or frontier");
@@ -609,6 +635,8 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
     t.n_unique = sizes_dev + h + 1;
     t.nnz = sizes_dev + n_hops + 1 + h;
     t.flags = sizes_dev + 2 * n_hops + 1 + h;
+    t.host_sizes = sizes_host;
+    t.n_hops = n_hops;
     t.frontier = frontier;
     t.src_local = outs[h].src_local;
     t.dst_local = outs[h].dst_local;
@@ -617,9 +645,9 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
   const bool rep = replace != 0;
   if (id_bytes == 8)
     return indptr.elem_bytes == 8
-               ? run_blocks_table<int64_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st)
-               : run_blocks_table<int64_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st);
+               ? run_blocks_table<int64_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st)
+               : run_blocks_table<int64_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st);
   return indptr.elem_bytes == 8
-             ? run_blocks_table<int32_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st)
-             : run_blocks_table<int32_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, st);
+             ? run_blocks_table<int32_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st)
+             : run_blocks_table<int32_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st);
 }

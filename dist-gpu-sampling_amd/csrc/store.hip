@@ -177,11 +177,8 @@ static std::mutex g_event_mutex;
 static std::vector<hipEvent_t> g_event_pool;
 }  // namespace dgs
 
-DGS_API dgs_status dgs_read_back_begin(void* host_dst, const void* dev_src, size_t n_bytes, void* stream,
-                                       void** ticket) {
-  DGS_REQUIRE(host_dst != nullptr && dev_src != nullptr && ticket != nullptr, DGS_ERR_INVALID,
-              "read_back_begin: null pointer");
-  hipStream_t st = static_cast<hipStream_t>(stream);
+DGS_API dgs_status dgs_ticket_record(void* stream, void** ticket) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_record: null ticket");
   hipEvent_t ev = nullptr;
   {
     std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
@@ -191,14 +188,25 @@ DGS_API dgs_status dgs_read_back_begin(void* host_dst, const void* dev_src, size
     }
   }
   if (ev == nullptr) DGS_HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-  DGS_HIP_TRY(hipMemcpyAsync(host_dst, dev_src, n_bytes, hipMemcpyDeviceToHost, st));
-  DGS_HIP_TRY(hipEventRecord(ev, st));
+  const hipError_t e = hipEventRecord(ev, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) {
+    std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
+    dgs::g_event_pool.push_back(ev);
+    dgs::set_error("ticket_record: %s", hipGetErrorString(e));
+    return DGS_ERR_HIP;
+  }
   *ticket = ev;
   return DGS_OK;
 }
 
-DGS_API dgs_status dgs_read_back_wait(void* ticket) {
-  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "read_back_wait: null ticket");
+DGS_API dgs_status dgs_ticket_stream_wait(void* stream, void* ticket) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_stream_wait: null ticket");
+  DGS_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(ticket), 0));
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_ticket_wait(void* ticket) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_wait: null ticket");
   hipEvent_t ev = static_cast<hipEvent_t>(ticket);
   const hipError_t e = hipEventSynchronize(ev);
   {
@@ -206,8 +214,25 @@ DGS_API dgs_status dgs_read_back_wait(void* ticket) {
     dgs::g_event_pool.push_back(ev);
   }
   if (e != hipSuccess) {
-    dgs::set_error("read_back_wait: %s", hipGetErrorString(e));
+    dgs::set_error("ticket_wait: %s", hipGetErrorString(e));
     return DGS_ERR_HIP;
   }
   return DGS_OK;
 }
+
+DGS_API dgs_status dgs_ticket_release(void* ticket) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_release: null ticket");
+  std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
+  dgs::g_event_pool.push_back(static_cast<hipEvent_t>(ticket));
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_read_back_begin(void* host_dst, const void* dev_src, size_t n_bytes, void* stream,
+                                       void** ticket) {
+  DGS_REQUIRE(host_dst != nullptr && dev_src != nullptr && ticket != nullptr, DGS_ERR_INVALID,
+              "read_back_begin: null pointer");
+  DGS_HIP_TRY(hipMemcpyAsync(host_dst, dev_src, n_bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+  return dgs_ticket_record(stream, ticket);
+}
+
+DGS_API dgs_status dgs_read_back_wait(void* ticket) { return dgs_ticket_wait(ticket); }

@@ -68,12 +68,13 @@ class ChunkTensorSampler:
         return blocks
 
     def sample_blocks(self, g, seed_nodes, exclude_eids=None):
-        """Returns (input_nodes, seed_nodes, blocks); `g` is unused, as upstream."""
-        seeds = seed_nodes.cuda()
+        """Returns (input_nodes, seed_nodes, blocks); `g` is unused, as upstream.  Host-side
+        seed_nodes (what upstream's DataLoader passes) are uploaded by the operator itself."""
         if self.fused:
-            frontiers, srcs, dsts = torch.ops.dgs_ops._CAPI_sample_blocks(
-                seeds, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace)
+            frontiers, srcs, dsts, seeds = torch.ops.dgs_ops._CAPI_sample_blocks(
+                seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace)
             return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts)
+        seeds = seed_nodes.cuda()
         blocks = []
         frontier = seeds
         for fan_out in reversed(self.fanouts):
@@ -90,11 +91,10 @@ class ChunkTensorSampler:
         (oppo_bench/single_node/chunktensor.py:142-151), with the gather enqueued behind
         the last hop before any length is read back.  Returns (input_nodes, seed_nodes,
         blocks, features_of_input_nodes)."""
-        seeds = seed_nodes.cuda()
         if not self.fused:
             frontier, _, blocks = self.sample_blocks(g, seed_nodes)
             return frontier, seed_nodes, blocks, chunk_features._CAPI_index(frontier)
-        frontiers, srcs, dsts, x = torch.ops.dgs_ops._CAPI_sample_blocks_and_index(
-            seeds, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
+        frontiers, srcs, dsts, x, seeds = torch.ops.dgs_ops._CAPI_sample_blocks_and_index(
+            seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
             chunk_features)
         return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts), x

@@ -277,6 +277,12 @@ typedef struct dgs_block_out {
  *                            [0 .. n_hops]                 seeds of hop h (h = n_hops: final frontier size)
  *                            [n_hops + 1 .. 2 n_hops]      edges of hop h
  *                            [2 n_hops + 1 .. 3 n_hops]    non-zero if a row of hop h had degree >= 2^32
+ *   sizes_host / ticket    : optional (both or neither).  sizes_host is pinned host memory
+ *                            that the device can write (hipHostMalloc); the kernels mirror
+ *                            sizes_dev into it, and *sizes_ticket marks the point on `stream`
+ *                            after which it is complete -- before the last hop's edge lists are
+ *                            written, so a caller can enqueue more work (a feature gather) and
+ *                            only then call dgs_ticket_wait.  Saves the device-to-host copy.
  *   node_table / epoch     : optional persistent direct-address table of
  *                            dgs_node_table_bytes(n_nodes) bytes (n_nodes = indptr entries - 1,
  *                            < 2^31), filled with 0xFF bytes before its first use and then never
@@ -298,7 +304,8 @@ dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seed
                              uint64_t rng_seed, uint32_t first_stream,
                              void* node_table, uint32_t node_table_epoch,
                              void* frontier, const dgs_block_out* outs,
-                             int64_t* sizes_dev, void* workspace,
+                             int64_t* sizes_dev, int64_t* sizes_host,
+                             void** sizes_ticket, void* workspace,
                              size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
@@ -322,6 +329,17 @@ dgs_status dgs_read_back(void* host_dst, const void* dev_src, size_t n_bytes,
 dgs_status dgs_read_back_begin(void* host_dst, const void* dev_src, size_t n_bytes,
                                void* stream, void** ticket);
 dgs_status dgs_read_back_wait(void* ticket);
+/*
+ * Tickets on their own: _record marks the current end of `stream`; _wait blocks the host
+ * until that point is reached (and retires the ticket: exactly one _wait per ticket);
+ * _stream_wait makes `stream` wait for it without blocking the host (call before _wait
+ * or _release); _release retires a ticket nobody on the host needs to wait for.
+ * dgs_read_back_wait is dgs_ticket_wait.
+ */
+dgs_status dgs_ticket_record(void* stream, void** ticket);
+dgs_status dgs_ticket_stream_wait(void* stream, void* ticket);
+dgs_status dgs_ticket_wait(void* ticket);
+dgs_status dgs_ticket_release(void* ticket);
 
 #ifdef __cplusplus
 }

@@ -274,3 +274,21 @@ def test_fused_long_tile_lists(pkg, oracle):
     _check_blocks(blocks, o_blocks)
     # the launch plan is sized by the worst case: 60000 * 41 rows and 9 times as many positions
     assert 60_000 * 41 > 2048 * 256 and blocks[0].num_dst > 200_000
+
+
+def test_host_seeds_are_accepted(pkg, oracle, graph):
+    # upstream's sampler receives host-side seed_nodes and uploads them itself
+    indptr, indices = graph
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    feats = torch.randn((20000, 16))
+    ft = pkg.create_chunktensor(feats, 1, 1 << 40)
+    seeds = torch.arange(100, 612)
+    sampler = pkg.ChunkTensorSampler([6, 3], ip_ct, ix_ct)
+    o_frontier, _, o_blocks = oracle.sample_blocks(seeds.numpy(), indptr, indices, [6, 3], False, 5, 9)
+    for s in (seeds, seeds.pin_memory(), seeds.cuda()):
+        pkg.set_rng_state(5, 9)
+        frontier, out_seeds, blocks, x = sampler.sample_blocks_and_index(None, s, ft)
+        assert out_seeds is s and np.array_equal(_np(frontier), o_frontier)
+        _check_blocks(blocks, o_blocks)
+        assert blocks[-1].dst_ids.is_cuda and torch.equal(x.cpu(), feats[frontier.cpu()])
