@@ -24,6 +24,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per gathered 400-byte row of workload c1, from rocprofv3 FETCH_SIZE (x2.0 after
+# calibration against a plain copy) and WRITE_SIZE (x1.0): 378.3 MB + 288.2 MB per 719,002 rows
+C1_GATHER_TRAFFIC_BYTES_PER_ROW = (378.3e6 + 288.2e6) / 719002.0
 
 WORKLOADS = {
     # BASELINE.json configs[1]: the configuration the metric is quoted on
@@ -257,7 +260,9 @@ def main():
         "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "gather_flat_kernel (ChunkTensor._CAPI_index)",
                      "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gather_gbps / HBM_PEAK_GBPS, "traffic": None},
+                     "frac": gather_gbps / HBM_PEAK_GBPS,
+                     "traffic": (C1_GATHER_TRAFFIC_BYTES_PER_ROW * rows / args.steps) if args.workload == "c1" else None,
+                     "algorithmic_bytes": bg / args.steps, "avg_launch_us": 1e3 * ms_gather},
         "graph_gen_s": t_gen,
     }
     if not args.no_cpu_baseline:
