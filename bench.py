@@ -137,12 +137,207 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0):
             "ms_gather": 1e3 * t_gather / done}
 
 
+def device_powerlaw_csc(n, e, max_deg, one_frac, id_dtype, gen, sort_by_degree):
+    """Power-law CSC built on the device (the large workloads never exist on the host)."""
+    u = torch.rand(n, generator=gen, device="cuda", dtype=torch.float64)
+    raw = (1.0 - u).pow(-1.0 / 1.25)
+    ones = torch.rand(n, generator=gen, device="cuda") < one_frac
+    lo, hi = 0.01, 1000.0
+    for _ in range(50):
+        mid = 0.5 * (lo + hi)
+        deg = (raw * mid).floor().clamp_(2, max_deg)
+        deg[ones] = 1
+        if deg.sum().item() > e:
+            hi = mid
+        else:
+            lo = mid
+    deg = (raw * lo).floor().clamp_(2, max_deg)
+    deg[ones] = 1
+    deg = deg.long()
+    rest = int(e - deg.sum().item())
+    deg[torch.nonzero((deg > 1) & (deg < max_deg - 1)).flatten()[:rest]] += 1
+    if sort_by_degree:  # node ids in decreasing in-degree: the hottest rows land in the HBM slice
+        deg = torch.sort(deg, descending=True).values
+    indptr = torch.zeros(n + 1, dtype=torch.int64, device="cuda")
+    torch.cumsum(deg, 0, out=indptr[1:])
+    e = int(indptr[-1].item())
+    indices = torch.empty(e, dtype=id_dtype, device="cuda")
+    for a in range(0, e, 1 << 28):
+        b = min(e, a + (1 << 28))
+        indices[a:b] = torch.randint(0, n, (b - a,), generator=gen, device="cuda", dtype=id_dtype)
+    return indptr, indices
+
+
+def store_from_device(dgs, t, capacity_bytes):
+    """ChunkTensor filled through its slice views from a device tensor."""
+    ct = dgs.ChunkTensor(list(t.shape), t.dtype, capacity_bytes)
+    flat = t.reshape(-1)
+    dev = ct._CAPI_get_sub_device_tensor()
+    dev.copy_(flat[: dev.numel()])
+    host = ct._CAPI_get_host_tensor()
+    for a in range(0, host.numel(), 1 << 28):
+        b = min(host.numel(), a + (1 << 28))
+        host[a:b].copy_(flat[dev.numel() + a: dev.numel() + b])
+    torch.cuda.synchronize()
+    return ct
+
+
+def time_call(fn, reps):
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(reps)]
+    fn()
+    torch.cuda.synchronize()
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return float(np.mean([a.elapsed_time(b) for a, b in ev])) * 1e-3
+
+
+def device_rmat_csc(scale_bits, e, gen):
+    """R-MAT (a, b, c, d) = (.57, .19, .19, .05) grouped by destination without sorting: the
+    destination bits are independent with P(bit = 1) = b + d, so in-degrees follow from the
+    per-node probability, and every source bit is drawn given the destination's bit."""
+    a, b, c, d = 0.57, 0.19, 0.19, 0.05
+    n = 1 << scale_bits
+    ids = torch.arange(n, device="cuda")
+    ones = torch.zeros(n, device="cuda", dtype=torch.float64)
+    for bit in range(scale_bits):
+        ones += ((ids >> bit) & 1).double()
+    lam = torch.exp(ones * np.log(b + d) + (scale_bits - ones) * np.log(a + c) + np.log(e))
+    deg = torch.poisson(lam.float(), generator=gen).long()
+    diff = int(e - deg.sum().item())
+    top = torch.argsort(lam, descending=True)[: abs(diff)]
+    deg[top] += 1 if diff > 0 else -1
+    deg.clamp_(min=0)
+    deg[0] += e - int(deg.sum().item())
+    indptr = torch.zeros(n + 1, dtype=torch.int64, device="cuda")
+    torch.cumsum(deg, 0, out=indptr[1:])
+    indices = torch.empty(e, dtype=torch.int32, device="cuda")
+    for lo in range(0, e, 1 << 26):
+        hi = min(e, lo + (1 << 26))
+        dst = torch.searchsorted(indptr, torch.arange(lo, hi, device="cuda"), right=True) - 1
+        src = torch.zeros(hi - lo, dtype=torch.int32, device="cuda")
+        for bit in range(scale_bits):
+            p1 = torch.where(((dst >> bit) & 1) == 1, d / (b + d), c / (a + c)).float()
+            src |= (torch.rand(hi - lo, generator=gen, device="cuda") < p1).int() << bit
+        indices[lo:hi] = src
+    return indptr, indices
+
+
+LARGE = {
+    # BASELINE.json configs[2]: large graph, all in HBM, bf16 x128, 4096 seeds from a 1% train subset
+    "c2": dict(graph="powerlaw", nodes=111_059_956, edges=1_615_685_872, dim=128, feat_dtype=torch.bfloat16,
+               hbm_rows=1.0, batch=4096, fanouts=[15, 10, 5], replace=False, train_frac=0.01, seed=20240603),
+    # configs[3]: same graph, f32 x256, top 40% of rows by in-degree in HBM, rest in pinned host memory
+    "c3": dict(graph="powerlaw", nodes=111_059_956, edges=1_615_685_872, dim=256, feat_dtype=torch.float32,
+               hbm_rows=0.4, batch=8192, fanouts=[20, 15, 10], replace=False, train_frac=1.0, seed=20240604),
+    # configs[4]: R-MAT scale 26, 2^30 edges, with replacement, fanouts [50, 50], 16384 seeds, f32 x64
+    "c4": dict(graph="rmat", nodes=1 << 26, edges=1 << 30, dim=64, feat_dtype=torch.float32,
+               hbm_rows=1.0, batch=16384, fanouts=[50, 50], replace=True, train_frac=1.0, seed=20240605),
+}
+
+
+def run_large(args, dgs):
+    """BASELINE.json configs[2..4], built on the device.  For the two-tier case (c3) the tiers
+    are also timed separately: device tier against HBM, host tier against PCIe Gen5 x16."""
+    cfg = LARGE[args.workload]
+    scale = args.scale
+    n, e = int(cfg["nodes"] * scale), int(cfg["edges"] * scale)
+    dim, fanouts, batch = cfg["dim"], cfg["fanouts"], cfg["batch"]
+    gen = torch.Generator(device="cuda").manual_seed(cfg["seed"])
+    t0 = time.perf_counter()
+    if cfg["graph"] == "rmat":
+        bits = int(round(np.log2(n)))
+        n = 1 << bits
+        indptr, indices = device_rmat_csc(bits, e, gen)
+    else:
+        indptr, indices = device_powerlaw_csc(n, e, 30_000, 0.05, torch.int32, gen,
+                                              sort_by_degree=cfg["hbm_rows"] < 1.0)
+    ct_ip = store_from_device(dgs, indptr, 1 << 62)
+    ct_ix = store_from_device(dgs, indices, 1 << 62)
+    del indptr, indices
+    hot_rows = int(n * cfg["hbm_rows"])
+    eb = torch.empty(0, dtype=cfg["feat_dtype"]).element_size()
+    ct_x = dgs.ChunkTensor([n, dim], cfg["feat_dtype"], hot_rows * dim * eb)
+    dev, host = ct_x._CAPI_get_sub_device_tensor(), ct_x._CAPI_get_host_tensor()
+    chunk = 1 << 26
+    for a in range(0, dev.numel(), chunk):
+        dev[a: a + chunk].normal_(generator=gen)
+    stage = torch.empty(chunk, device="cuda", dtype=cfg["feat_dtype"])
+    for a in range(0, host.numel(), chunk):
+        m = min(chunk, host.numel() - a)
+        stage[:m].normal_(generator=gen)
+        host[a: a + m].copy_(stage[:m])
+    del stage
+    torch.cuda.synchronize()
+    t_gen = time.perf_counter() - t0
+    sampler = dgs.ChunkTensorSampler(fanouts, ct_ip, ct_ix, replace=cfg["replace"])
+    pool = None
+    if cfg["train_frac"] < 1.0:  # seeds come from a fixed uniform subset of the nodes
+        pool = torch.randperm(n, generator=gen, device="cuda")[: int(n * cfg["train_frac"])].to(torch.int32)
+    seeds = []
+    for _ in range(args.steps + args.warmup):
+        r = torch.randint(0, n if pool is None else pool.numel(), (batch,), generator=gen, device="cuda")
+        seeds.append(r.to(torch.int32) if pool is None else pool[r])
+    dgs.set_rng_state(cfg["seed"], 0)
+    for i in range(args.warmup):
+        sampler.sample_blocks_and_index(None, seeds[i], ct_x)
+    torch.cuda.synchronize()
+    edges = rows = 0
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        frontier, _, blocks, x = sampler.sample_blocks_and_index(None, seeds[args.warmup + i], ct_x)
+        edges += sum(b.src_local.numel() for b in blocks)
+        rows += frontier.numel()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    del x
+    row_bytes = dim * eb
+    t_mixed = time_call(lambda: ct_x._CAPI_index(frontier), 3)
+    gather_gbps = frontier.numel() * (2 * row_bytes + 4) / t_mixed / 1e9
+    out = {
+        "metric": "sampled edges/s (sampling + relabel + feature gather per batch), 1 MI355X",
+        "value": edges / elapsed, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": 1e3 * elapsed / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {cfg['graph']} graph, {n} nodes / {e} edges CSC int64+int32, "
+                               f"features {str(cfg['feat_dtype']).split('.')[-1]} x{dim} ({n * row_bytes / 1e9:.1f} GB), "
+                               f"{int(100 * cfg['hbm_rows'])}% of rows in HBM, batch {batch}, fanouts {fanouts}, "
+                               f"{'with' if cfg['replace'] else 'without'} replacement", "scale": scale},
+        "avg_frontier_rows": rows / args.steps, "avg_edges_per_batch": edges / args.steps,
+        "gather_ms": 1e3 * t_mixed, "gather_GBps": gather_gbps, "graph_gen_s": t_gen,
+    }
+    if cfg["hbm_rows"] < 1.0:
+        local, _, host_ids = ct_x._CAPI_split_index(frontier)
+        host_ids = host_ids[host_ids > hot_rows]  # the row that straddles the boundary belongs to neither tier
+        t_local = time_call(lambda: ct_x._CAPI_local_index(local), 5)
+        t_host = time_call(lambda: ct_x._CAPI_host_index(host_ids), 3)
+        dev_gbps = local.numel() * (2 * row_bytes + 4) / t_local / 1e9
+        host_gbps = host_ids.numel() * row_bytes / t_host / 1e9
+        out.update({
+            "frontier_rows_device_tier": local.numel(), "frontier_rows_host_tier": host_ids.numel(),
+            "device_tier_gather_GBps": dev_gbps, "device_tier_ms": 1e3 * t_local,
+            "host_tier_gather_GBps": host_gbps, "host_tier_ms": 1e3 * t_host,
+            "host_tier_peak_GBps": 64.0, "host_tier_pcie_frac": host_gbps / 64.0,
+            "roofline": {"bound": "hbm", "kernel": "gather_flat_kernel (_CAPI_local_index, device tier)",
+                         "achieved": dev_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": dev_gbps / HBM_PEAK_GBPS, "traffic": None},
+        })
+    else:
+        out["roofline"] = {"bound": "hbm", "kernel": "gather_flat_kernel (_CAPI_index)", "achieved": gather_gbps,
+                           "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gather_gbps / HBM_PEAK_GBPS,
+                           "traffic": None}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + sorted(LARGE))
+    ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
@@ -155,8 +350,10 @@ def main():
         sys.exit("bench.py: no GPU visible")
 
     dgs = importlib.import_module("dist-gpu-sampling_amd")
-    cfg = WORKLOADS[args.workload]
     torch.cuda.set_device(0)
+    if args.workload in LARGE:
+        return run_large(args, dgs)
+    cfg = WORKLOADS[args.workload]
     t0 = time.perf_counter()
     indptr, indices, feats, _ = make_graph(cfg)
     t_gen = time.perf_counter() - t0
