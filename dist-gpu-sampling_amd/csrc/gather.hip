@@ -17,6 +17,9 @@ constexpr int kGatherUnroll = 4;
 constexpr int kChunksPerBlock = kGatherThreads * kGatherUnroll;
 // largest chunks-per-row for which the multiply-high division below is exact
 constexpr uint32_t kMaxFlatChunksPerRow = 32768;
+// A launch sized for a worst-case row count (dgs_gather_rows_dyn) is capped at this many blocks;
+// blocks stride over the tiles, so a mostly unused worst case does not cost 10^5 empty blocks.
+constexpr int64_t kMaxDynGrid = 32768;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -39,37 +42,39 @@ __device__ __forceinline__ const char* resolve(const char* dev, const char* host
 // chunk c -> row c / cpr, column c % cpr; the division runs on a block-local
 // 32-bit offset with a precomputed reciprocal (exact while
 // (cpr + kChunksPerBlock) * cpr < 2^32, guaranteed by kMaxFlatChunksPerRow).
-template <int VEC, int TIER, typename IndexT>
+template <int VEC, int TIER, typename IndexT, bool STRIDE>
 __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, uint32_t cpr, uint32_t magic, const IndexT* __restrict__ index,
     int64_t total_chunks, const int64_t* __restrict__ n_rows_dev, char* __restrict__ out) {
   using C = typename Chunk<VEC>::type;
-  const int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock;
   if (n_rows_dev) total_chunks = *n_rows_dev * cpr;  // row count decided on the device
-  if (c0 >= total_chunks) return;
-  const int64_t row0 = c0 / cpr;
-  const uint32_t rem0 = uint32_t(c0 - row0 * cpr);
+  // STRIDE: the grid is smaller than the tile count (capped launch), blocks stride over the tiles
+  for (int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock; c0 < total_chunks;
+       c0 += STRIDE ? int64_t(gridDim.x) * kChunksPerBlock : total_chunks) {
+    const int64_t row0 = c0 / cpr;
+    const uint32_t rem0 = uint32_t(c0 - row0 * cpr);
 
-  C val[kGatherUnroll];
-  bool ok[kGatherUnroll];
+    C val[kGatherUnroll];
+    bool ok[kGatherUnroll];
 #pragma unroll
-  for (int u = 0; u < kGatherUnroll; ++u) {
-    const uint32_t t = u * kGatherThreads + threadIdx.x;
-    ok[u] = c0 + t < total_chunks;
-    if (ok[u]) {
-      const uint32_t lc = rem0 + t;
-      const uint32_t q = cpr == 1 ? lc : __umulhi(lc, magic);
-      const uint32_t col = lc - q * cpr;
-      const int64_t src_row = int64_t(index[row0 + q]);
-      const int64_t g = src_row * row_bytes + int64_t(col) * VEC;
-      val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+    for (int u = 0; u < kGatherUnroll; ++u) {
+      const uint32_t t = u * kGatherThreads + threadIdx.x;
+      ok[u] = c0 + t < total_chunks;
+      if (ok[u]) {
+        const uint32_t lc = rem0 + t;
+        const uint32_t q = cpr == 1 ? lc : __umulhi(lc, magic);
+        const uint32_t col = lc - q * cpr;
+        const int64_t src_row = int64_t(index[row0 + q]);
+        const int64_t g = src_row * row_bytes + int64_t(col) * VEC;
+        val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+      }
     }
-  }
 #pragma unroll
-  for (int u = 0; u < kGatherUnroll; ++u) {
-    const uint32_t t = u * kGatherThreads + threadIdx.x;
-    if (ok[u]) __builtin_nontemporal_store(val[u], reinterpret_cast<C*>(out + (c0 + t) * VEC));
+    for (int u = 0; u < kGatherUnroll; ++u) {
+      const uint32_t t = u * kGatherThreads + threadIdx.x;
+      if (ok[u]) __builtin_nontemporal_store(val[u], reinterpret_cast<C*>(out + (c0 + t) * VEC));
+    }
   }
 }
 
@@ -105,14 +110,21 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
   const char* host = static_cast<const char*>(v.host);
   if (cpr <= kMaxFlatChunksPerRow) {
     const int64_t total_chunks = n * cpr;
-    const int64_t blocks = (total_chunks + kChunksPerBlock - 1) / kChunksPerBlock;
-    DGS_REQUIRE(blocks <= 0x7fffffff, DGS_ERR_UNSUPPORTED, "gather: %lld rows of %lld B exceed one launch",
-                (long long)n, (long long)row_bytes);
+    const int64_t tiles = (total_chunks + kChunksPerBlock - 1) / kChunksPerBlock;
+    int64_t blocks = tiles;
+    if (n_dev != nullptr && blocks > kMaxDynGrid) blocks = kMaxDynGrid;
+    if (blocks > 0x7fffffff) blocks = 0x7fffffff;
     const uint32_t magic = cpr > 1 ? uint32_t((uint64_t(1) << 32) / uint64_t(cpr)) + 1u : 0u;
-    hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT>), dim3(uint32_t(blocks)),
-                       dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
-                       magic, static_cast<const IndexT*>(index), total_chunks, n_dev,
-                       static_cast<char*>(out));
+    if (blocks < tiles)
+      hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, true>), dim3(uint32_t(blocks)),
+                         dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
+                         magic, static_cast<const IndexT*>(index), total_chunks, n_dev,
+                         static_cast<char*>(out));
+    else
+      hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, false>), dim3(uint32_t(blocks)),
+                         dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
+                         magic, static_cast<const IndexT*>(index), total_chunks, n_dev,
+                         static_cast<char*>(out));
   } else {
     const int64_t bpr = (cpr + kChunksPerBlock - 1) / kChunksPerBlock;
     DGS_REQUIRE(n * bpr <= 0x7fffffff, DGS_ERR_UNSUPPORTED, "gather: %lld rows of %lld B exceed one launch",

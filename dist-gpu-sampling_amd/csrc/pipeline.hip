@@ -51,12 +51,20 @@ constexpr uint32_t kBadRow = 0xffffffffu;      // row_cnt marker: degree >= 2^32
 constexpr int kMaxPicks = 64;
 constexpr int64_t kMaxPositions = int64_t(1) << 30;
 constexpr int64_t kInlineTiles = 2048;         // above this a separate scan launch is used
+// Launches are sized for the worst case, which can exceed the real work many times over (a hub
+// graph deduplicates heavily).  Grids are capped and blocks stride over the virtual block index,
+// so a mostly empty worst case costs a few loop trips instead of 10^5 empty blocks.
+constexpr int64_t kGridCap = 16384;
+inline uint32_t capped_grid(int64_t virtual_blocks) {
+  return uint32_t(virtual_blocks < 1 ? 1 : (virtual_blocks > kGridCap ? kGridCap : virtual_blocks));
+}
 
 struct Hop {
   const void* seeds;        // seed ids: caller's seeds (hop 0) or the frontier array
   const int64_t* n_seeds;   // device scalar (ignored when n_seeds_host >= 0)
   int64_t n_seeds_host;     // hop 0: the caller's count; later hops: -1
   int64_t* n_seeds_out;     // hop 0: where to publish n_seeds on the device
+  const int64_t* prev_nnz;  // device scalar: edges of the previous hop (NULL in hop 0)
   int64_t* n_unique;        // device scalar: frontier size after this hop
   int64_t* nnz;             // device scalar: edges of this hop
   int64_t* flags;           // device scalar: non-zero on a bad row
@@ -212,24 +220,14 @@ __device__ __forceinline__ void mark_lost(const Hop& h, uint32_t displaced) {
   if (displaced != kNoPosition) h.lost[displaced] = 1;
 }
 
+// One virtual block of the fill launch: 256 / G seed rows.
 template <typename IdT, typename PtrT, typename TableT, int G>
-__global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64_t fill_blocks,
-                                                          int64_t relabel_count, uint4* clear_begin,
-                                                          int64_t clear_n16, TableT table, TierView<PtrT> indptr,
-                                                          TierView<IdT> indices, bool replace, uint64_t rng_seed) {
-  if (int64_t(blockIdx.x) >= fill_blocks) {
-    const int64_t b = int64_t(blockIdx.x) - fill_blocks;
-    if (b < relabel_count) {  // surplus blocks: edge list of the previous hop
-      relabel_tile<IdT, TableT>(prev, table, b);
-    } else {                  // surplus blocks of hop 0: clear the lost marks of the later hops
-      const int64_t i = (b - relabel_count) * kBlock + threadIdx.x;
-      if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
-    }
-    return;
-  }
+__device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT& table,
+                                          const TierView<PtrT>& indptr, const TierView<IdT>& indices,
+                                          bool replace, uint64_t rng_seed) {
   const int64_t s = seeds_of(h);
-  if (h.n_seeds_out && blockIdx.x == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
-  const int64_t gid = int64_t(blockIdx.x) * kBlock + threadIdx.x;
+  if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
+  const int64_t gid = vb * kBlock + threadIdx.x;
   const int64_t i = gid / G;
   const int l = int(gid % G);
   if (i >= s) return;  // whole groups leave together
@@ -242,6 +240,15 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
   const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
   const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;
+  // Ids that repeat a lot (hub sources) are cheaper to insert with a look at the entry first;
+  // the previous hop tells: if more than a fifth of its picks were not new ids, look first.
+  // (hop 0 has no history: look first only when it is big enough for contention to matter)
+  bool look_first = s * k >= (int64_t(1) << 17);
+  if (h.prev_nnz) {
+    const int64_t picked = *h.prev_nnz;
+    const int64_t fresh = s - *(h.n_seeds - 1);  // ids the previous hop added to the frontier
+    look_first = fresh * 5 < picked * 4;
+  }
   if (l == 0) {
     h.row_cnt[i] = bad ? kBadRow : (replace ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
     if (h.index == 0) {  // the caller's seeds open the mapping list; flag() decides their first bits
@@ -259,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
       const IdT col = indices.at(b + pos);
       bool first;
       uint32_t displaced;
-      word = table.insert_min(col, uint32_t(p), &first, &displaced);
+      word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
       if (h.index != 0) {
         if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
         mark_lost(h, displaced);
@@ -269,36 +276,68 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
   }
 }
 
-template <typename IdT, typename TableT>
-__global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_blocks, TableT table) {
-  if (int64_t(blockIdx.x) >= flag_blocks) {  // surplus blocks: per-tile row offsets of this hop
-    offsets_tile(h, int(int64_t(blockIdx.x) - flag_blocks));
-    return;
+// Virtual blocks [0, fill_blocks): seed rows of this hop; then relabel_count blocks writing the
+// previous hop's edge list (off the critical path); then, in hop 0's launch, blocks clearing the
+// lost marks of the later hops.
+template <typename IdT, typename PtrT, typename TableT, int G>
+__global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64_t fill_blocks,
+                                                          int64_t relabel_count, uint4* clear_begin,
+                                                          int64_t clear_n16, TableT table, TierView<PtrT> indptr,
+                                                          TierView<IdT> indices, bool replace, uint64_t rng_seed) {
+  const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
+  const int64_t total = fill_blocks + relabel_count + clear_blocks;
+  for (int64_t vb = blockIdx.x; vb < total; vb += gridDim.x) {
+    if (vb < fill_blocks) {
+      fill_rows<IdT, PtrT, TableT, G>(h, vb, table, indptr, indices, replace, rng_seed);
+    } else if (vb < fill_blocks + relabel_count) {
+      relabel_tile<IdT, TableT>(prev, table, vb - fill_blocks);
+    } else {
+      const int64_t i = (vb - fill_blocks - relabel_count) * kBlock + threadIdx.x;
+      if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
   }
+}
+
+// One virtual block of the flag launch: 1024 padded positions.
+template <typename IdT, typename TableT>
+__device__ __forceinline__ void flag_tile(const Hop& h, int64_t tile, const TableT& table) {
   __shared__ int lds[kBlock / kWave];
   const int64_t s = seeds_of(h);
   const int64_t len = seed_part(h, s) + s * h.k;
-  const int64_t base = int64_t(blockIdx.x) * kPosTile + threadIdx.x * kPosItems;
+  const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
   int c = 0;
+  if (tile * kPosTile < len) {
 #pragma unroll
-  for (int j = 0; j < kPosItems; ++j) {
-    const int64_t rel = base + j;
-    if (rel < len) {
-      const int64_t p = h.pos_base + rel;
-      const uint32_t w = h.slot[p];
-      if (w == kInvalidSlot) continue;
-      if (h.index == 0) {
-        if (table.value(w) == uint32_t(p)) {
-          h.slot[p] = w | kFirstBit;
-          ++c;
+    for (int j = 0; j < kPosItems; ++j) {
+      const int64_t rel = base + j;
+      if (rel < len) {
+        const int64_t p = h.pos_base + rel;
+        const uint32_t w = h.slot[p];
+        if (w == kInvalidSlot) continue;
+        if (h.index == 0) {
+          if (table.value(w) == uint32_t(p)) {
+            h.slot[p] = w | kFirstBit;
+            ++c;
+          }
+        } else if (w & kFirstBit) {
+          if (h.lost[p]) h.slot[p] = w & ~kFirstBit; else ++c;
         }
-      } else if (w & kFirstBit) {
-        if (h.lost[p]) h.slot[p] = w & ~kFirstBit; else ++c;
       }
     }
+    c = block_sum<kBlock, int>(c, lds);
   }
-  c = block_sum<kBlock, int>(c, lds);
-  if (threadIdx.x == 0) h.pos_cnt[blockIdx.x] = c;
+  if (threadIdx.x == 0) h.pos_cnt[tile] = c;
+}
+
+// Virtual blocks [0, flag_blocks): position tiles; then row_tiles blocks scanning the rows' pick
+// counts per 256-row tile (for the packed edge list, off the critical path).
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_blocks, int64_t row_tiles,
+                                                          TableT table) {
+  for (int64_t vb = blockIdx.x; vb < flag_blocks + row_tiles; vb += gridDim.x) {
+    if (vb < flag_blocks) flag_tile<IdT, TableT>(h, vb, table);
+    else offsets_tile(h, int(vb - flag_blocks));
+  }
 }
 
 // Separate scans for very long tile lists (one block).
@@ -314,15 +353,15 @@ __global__ __launch_bounds__(1024) void tile_scan_kernel(Hop h) {
   single_block_scan<1024, int, int64_t>(h.tile_sum, h.tile_off, tiles, &sum);
 }
 
+// One virtual block of the compact launch: the first occurrences of one 1024-position tile.
 template <typename IdT, typename TableT>
-__global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, TableT table) {
+__device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, const TableT& table) {
   __shared__ int64_t lds64[kBlock / kWave];
   __shared__ int lds[kBlock / kWave];
   const int64_t s = seeds_of(h);
   const int64_t len = seed_part(h, s) + s * h.k;
   const int64_t tiles = (len + kPosTile - 1) / kPosTile;
   const int64_t rank0 = first_rank(h, s);
-  const int64_t tile = blockIdx.x;
   if (tile >= tiles && tile != 0) return;
   // first occurrences in the tiles before this one (block 0 also needs the grand total)
   int64_t before = 0, all = 0;
@@ -382,13 +421,18 @@ __global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, TableT table
 }
 
 template <typename IdT, typename TableT>
-__global__ __launch_bounds__(kBlock) void hop_relabel_kernel(Hop h, TableT table) {
-  relabel_tile<IdT, TableT>(h, table, int64_t(blockIdx.x));
+__global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, int64_t pos_tiles, TableT table) {
+  for (int64_t vb = blockIdx.x; vb < pos_tiles; vb += gridDim.x) compact_tile<IdT, TableT>(h, vb, table);
+}
+
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kBlock) void hop_relabel_kernel(Hop h, int64_t blocks, TableT table) {
+  for (int64_t vb = blockIdx.x; vb < blocks; vb += gridDim.x) relabel_tile<IdT, TableT>(h, table, vb);
 }
 
 __global__ __launch_bounds__(kBlock) void clear_kernel(uint4* __restrict__ p, int64_t n16) {
-  const int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x;
-  if (i < n16) p[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+  for (int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x; i < n16; i += int64_t(gridDim.x) * kBlock)
+    p[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
 }
 
 // ---- host side -------------------------------------------------------------------------------
@@ -479,7 +523,7 @@ void launch_fill(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* 
   const int64_t fill_blocks = (cur.s_max * G + kBlock - 1) / kBlock;
   const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
   hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G>),
-                     dim3(uint32_t(fill_blocks + relabel_count + clear_blocks)), dim3(kBlock), 0, st, cur, prev,
+                     dim3(capped_grid(fill_blocks + relabel_count + clear_blocks)), dim3(kBlock), 0, st, cur, prev,
                      fill_blocks, relabel_count, clear_begin, clear_n16, table, TierView<PtrT>(indptr),
                      TierView<IdT>(indices), replace, rng_seed);
 }
@@ -511,8 +555,8 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
     const int64_t len_max = (h == 0 ? cur.s_max : 0) + cur.s_max * cur.k;
     const int64_t pos_tiles = (len_max + kPosTile - 1) / kPosTile;
     const int64_t row_tiles = (cur.s_max + kRowTile - 1) / kRowTile;
-    hipLaunchKernelGGL((hop_flag_kernel<IdT, TableT>), dim3(uint32_t(pos_tiles + row_tiles)), dim3(kBlock), 0, st,
-                       cur, pos_tiles, table);
+    hipLaunchKernelGGL((hop_flag_kernel<IdT, TableT>), dim3(capped_grid(pos_tiles + row_tiles)), dim3(kBlock), 0,
+                       st, cur, pos_tiles, row_tiles, table);
     DGS_LAUNCH_CHECK();
     if (cur.pos_off) {
       hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
@@ -522,8 +566,9 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
       hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
       DGS_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT>), dim3(uint32_t(pos_tiles > 0 ? pos_tiles : 1)),
-                       dim3(kBlock), 0, st, cur, table);
+    const int64_t compact_blocks = pos_tiles > 0 ? pos_tiles : 1;  // block 0 always writes the lengths
+    hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT>), dim3(capped_grid(compact_blocks)), dim3(kBlock), 0, st,
+                       cur, compact_blocks, table);
     DGS_LAUNCH_CHECK();
   }
   // every length is final here: mark the point the caller may wait for
@@ -532,9 +577,10 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
     if (ts != DGS_OK) return ts;
   }
   const Hop& last = hops[p.n_hops - 1];
-  if (relabel_blocks(last.s_max, last.k) > 0) {
-    hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT>), dim3(uint32_t(relabel_blocks(last.s_max, last.k))),
-                       dim3(kBlock), 0, st, last, table);
+  const int64_t last_blocks = relabel_blocks(last.s_max, last.k);
+  if (last_blocks > 0) {
+    hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT>), dim3(capped_grid(last_blocks)), dim3(kBlock), 0, st, last,
+                       last_blocks, table);
     DGS_LAUNCH_CHECK();
   }
   return DGS_OK;
@@ -548,7 +594,7 @@ dgs_status run_blocks_table(const Plan& p, Hop* hops, void* hash_table, void* no
     return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch), indptr, indices,
                                                    replace, rng_seed, sizes_ticket, st);
   const int64_t n16 = int64_t(p.table_bytes / 16);
-  hipLaunchKernelGGL(clear_kernel, dim3(uint32_t((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
+  hipLaunchKernelGGL(clear_kernel, dim3(capped_grid((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                      static_cast<uint4*>(hash_table), n16);
   DGS_LAUNCH_CHECK();
   if (p.kind == TableKind::kPacked)
@@ -632,6 +678,7 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
     t.n_seeds = sizes_dev + h;
     t.n_seeds_host = h == 0 ? n_seeds : -1;
     t.n_seeds_out = h == 0 ? sizes_dev : nullptr;
+    t.prev_nnz = h == 0 ? nullptr : sizes_dev + n_hops + h;  // edges of hop h - 1
     t.n_unique = sizes_dev + h + 1;
     t.nnz = sizes_dev + n_hops + 1 + h;
     t.flags = sizes_dev + 2 * n_hops + 1 + h;

@@ -60,7 +60,8 @@ struct Table<IdT, true> {
   }
   // Same, reporting whether idx became the smallest position of its key (*first) and, if it
   // replaced a larger one, which (*displaced, else kNoPosition).
-  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced) const {
+  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced,
+                                                 bool /*look_first*/ = true) const {
     const unsigned long long packed = (static_cast<unsigned long long>(uint32_t(key)) << 32) | idx;
     uint32_t pos = hash_id(uint32_t(key)) & mask;
     *displaced = kNoPosition;
@@ -121,7 +122,8 @@ struct Table<IdT, false> {
     atomicMin(vals + pos, idx);
     return pos;
   }
-  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced) const {
+  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced,
+                                                 bool /*look_first*/ = true) const {
     using W = typename AtomicWord<IdT>::type;
     uint32_t pos = hash_id(uint64_t(int64_t(key))) & mask;
     for (;;) {
@@ -163,9 +165,16 @@ struct DirectTable {
   __host__ __device__ DirectTable(void* base, uint32_t epoch)
       : entries(static_cast<unsigned long long*>(base)), tag(~epoch) {}
 
-  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced) const {
+  // `look_first`: read the entry before the atomic.  A value already below v (a stale read can
+  // only be larger than the truth) settles the matter without an atomic, which is what keeps
+  // popular ids from serialising thousands of atomics on one address; on ids that are mostly
+  // new the extra read is pure cost.  The result is the same either way.
+  __device__ __forceinline__ uint32_t insert_min(IdT key, uint32_t idx, bool* first, uint32_t* displaced,
+                                                 bool look_first = true) const {
     const unsigned long long v = (static_cast<unsigned long long>(tag) << 32) | idx;
-    const unsigned long long old = atomicMin(entries + uint32_t(key), v);
+    unsigned long long* e = entries + uint32_t(key);
+    if (look_first && *e < v) { *first = false; *displaced = kNoPosition; return uint32_t(key); }
+    const unsigned long long old = atomicMin(e, v);
     *first = old > v;
     // an entry of this use that was larger: that position is no longer its id's smallest
     *displaced = (*first && uint32_t(old >> 32) == tag) ? uint32_t(old) : kNoPosition;
