@@ -58,6 +58,11 @@ constexpr int64_t kGridCap = 16384;
 inline uint32_t capped_grid(int64_t virtual_blocks) {
   return uint32_t(virtual_blocks < 1 ? 1 : (virtual_blocks > kGridCap ? kGridCap : virtual_blocks));
 }
+inline bool is_capped(int64_t virtual_blocks) { return virtual_blocks > kGridCap; }
+// Kernels come in two flavours: STRIDE = false runs exactly one virtual block per block (the
+// common, uncapped launch, with no loop in the instruction stream), STRIDE = true strides.
+#define DGS_FOR_VIRTUAL_BLOCKS(vb, total)                                                       \
+  for (int64_t vb = blockIdx.x; vb < (total); vb += STRIDE ? int64_t(gridDim.x) : (total))
 
 struct Hop {
   const void* seeds;        // seed ids: caller's seeds (hop 0) or the frontier array
@@ -279,14 +284,14 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
 // Virtual blocks [0, fill_blocks): seed rows of this hop; then relabel_count blocks writing the
 // previous hop's edge list (off the critical path); then, in hop 0's launch, blocks clearing the
 // lost marks of the later hops.
-template <typename IdT, typename PtrT, typename TableT, int G>
+template <typename IdT, typename PtrT, typename TableT, int G, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64_t fill_blocks,
                                                           int64_t relabel_count, uint4* clear_begin,
                                                           int64_t clear_n16, TableT table, TierView<PtrT> indptr,
                                                           TierView<IdT> indices, bool replace, uint64_t rng_seed) {
   const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
   const int64_t total = fill_blocks + relabel_count + clear_blocks;
-  for (int64_t vb = blockIdx.x; vb < total; vb += gridDim.x) {
+  DGS_FOR_VIRTUAL_BLOCKS(vb, total) {
     if (vb < fill_blocks) {
       fill_rows<IdT, PtrT, TableT, G>(h, vb, table, indptr, indices, replace, rng_seed);
     } else if (vb < fill_blocks + relabel_count) {
@@ -331,10 +336,10 @@ __device__ __forceinline__ void flag_tile(const Hop& h, int64_t tile, const Tabl
 
 // Virtual blocks [0, flag_blocks): position tiles; then row_tiles blocks scanning the rows' pick
 // counts per 256-row tile (for the packed edge list, off the critical path).
-template <typename IdT, typename TableT>
+template <typename IdT, typename TableT, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_blocks, int64_t row_tiles,
                                                           TableT table) {
-  for (int64_t vb = blockIdx.x; vb < flag_blocks + row_tiles; vb += gridDim.x) {
+  DGS_FOR_VIRTUAL_BLOCKS(vb, flag_blocks + row_tiles) {
     if (vb < flag_blocks) flag_tile<IdT, TableT>(h, vb, table);
     else offsets_tile(h, int(vb - flag_blocks));
   }
@@ -420,14 +425,14 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, const T
   }
 }
 
-template <typename IdT, typename TableT>
+template <typename IdT, typename TableT, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, int64_t pos_tiles, TableT table) {
-  for (int64_t vb = blockIdx.x; vb < pos_tiles; vb += gridDim.x) compact_tile<IdT, TableT>(h, vb, table);
+  DGS_FOR_VIRTUAL_BLOCKS(vb, pos_tiles) compact_tile<IdT, TableT>(h, vb, table);
 }
 
-template <typename IdT, typename TableT>
+template <typename IdT, typename TableT, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_relabel_kernel(Hop h, int64_t blocks, TableT table) {
-  for (int64_t vb = blockIdx.x; vb < blocks; vb += gridDim.x) relabel_tile<IdT, TableT>(h, table, vb);
+  DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) relabel_tile<IdT, TableT>(h, table, vb);
 }
 
 __global__ __launch_bounds__(kBlock) void clear_kernel(uint4* __restrict__ p, int64_t n16) {
@@ -522,10 +527,15 @@ void launch_fill(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* 
                  uint64_t rng_seed, hipStream_t st) {
   const int64_t fill_blocks = (cur.s_max * G + kBlock - 1) / kBlock;
   const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G>),
-                     dim3(capped_grid(fill_blocks + relabel_count + clear_blocks)), dim3(kBlock), 0, st, cur, prev,
-                     fill_blocks, relabel_count, clear_begin, clear_n16, table, TierView<PtrT>(indptr),
-                     TierView<IdT>(indices), replace, rng_seed);
+  const int64_t total = fill_blocks + relabel_count + clear_blocks;
+  if (is_capped(total))
+    hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G, true>), dim3(capped_grid(total)), dim3(kBlock), 0, st,
+                       cur, prev, fill_blocks, relabel_count, clear_begin, clear_n16, table,
+                       TierView<PtrT>(indptr), TierView<IdT>(indices), replace, rng_seed);
+  else
+    hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G, false>), dim3(capped_grid(total)), dim3(kBlock), 0, st,
+                       cur, prev, fill_blocks, relabel_count, clear_begin, clear_n16, table,
+                       TierView<PtrT>(indptr), TierView<IdT>(indices), replace, rng_seed);
 }
 
 template <typename IdT, typename PtrT, typename TableT>
@@ -555,8 +565,12 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
     const int64_t len_max = (h == 0 ? cur.s_max : 0) + cur.s_max * cur.k;
     const int64_t pos_tiles = (len_max + kPosTile - 1) / kPosTile;
     const int64_t row_tiles = (cur.s_max + kRowTile - 1) / kRowTile;
-    hipLaunchKernelGGL((hop_flag_kernel<IdT, TableT>), dim3(capped_grid(pos_tiles + row_tiles)), dim3(kBlock), 0,
-                       st, cur, pos_tiles, row_tiles, table);
+    if (is_capped(pos_tiles + row_tiles))
+      hipLaunchKernelGGL((hop_flag_kernel<IdT, TableT, true>), dim3(capped_grid(pos_tiles + row_tiles)),
+                         dim3(kBlock), 0, st, cur, pos_tiles, row_tiles, table);
+    else
+      hipLaunchKernelGGL((hop_flag_kernel<IdT, TableT, false>), dim3(capped_grid(pos_tiles + row_tiles)),
+                         dim3(kBlock), 0, st, cur, pos_tiles, row_tiles, table);
     DGS_LAUNCH_CHECK();
     if (cur.pos_off) {
       hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
@@ -567,8 +581,12 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
       DGS_LAUNCH_CHECK();
     }
     const int64_t compact_blocks = pos_tiles > 0 ? pos_tiles : 1;  // block 0 always writes the lengths
-    hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT>), dim3(capped_grid(compact_blocks)), dim3(kBlock), 0, st,
-                       cur, compact_blocks, table);
+    if (is_capped(compact_blocks))
+      hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT, true>), dim3(capped_grid(compact_blocks)), dim3(kBlock),
+                         0, st, cur, compact_blocks, table);
+    else
+      hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT, false>), dim3(capped_grid(compact_blocks)), dim3(kBlock),
+                         0, st, cur, compact_blocks, table);
     DGS_LAUNCH_CHECK();
   }
   // every length is final here: mark the point the caller may wait for
@@ -579,8 +597,12 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
   const Hop& last = hops[p.n_hops - 1];
   const int64_t last_blocks = relabel_blocks(last.s_max, last.k);
   if (last_blocks > 0) {
-    hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT>), dim3(capped_grid(last_blocks)), dim3(kBlock), 0, st, last,
-                       last_blocks, table);
+    if (is_capped(last_blocks))
+      hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT, true>), dim3(capped_grid(last_blocks)), dim3(kBlock), 0,
+                         st, last, last_blocks, table);
+    else
+      hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT, false>), dim3(capped_grid(last_blocks)), dim3(kBlock), 0,
+                         st, last, last_blocks, table);
     DGS_LAUNCH_CHECK();
   }
   return DGS_OK;
