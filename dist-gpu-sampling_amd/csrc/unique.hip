@@ -1,13 +1,14 @@
 // First-occurrence unique + relabel of node ids.
 //
-// A linear-probing table in HBM (capacity = power of two >= 2n, multiplicative
-// hash) maps each id to the smallest position at which it occurs; a position is
+// A linear-probing table in HBM (table.h: packed 64-bit slots for 4-byte ids, id array +
+// value array for 8-byte ids) maps each id to the smallest position at which it occurs; a position is
 // a "first occurrence" when the table holds exactly that position.  Flags are
 // scanned tile by tile, first occurrences are compacted in input order (which is
 // what makes the result independent of the table layout) and the table value
 // becomes the id's rank.  Every key remembers its slot, so only ids that were
 // not part of the mapping list are probed a second time.
 #include "common.h"
+#include "table.h"
 
 namespace dgs {
 namespace {
@@ -17,14 +18,6 @@ constexpr int kItems = 4;
 constexpr int kTileIds = kThreads * kItems;   // ids per block in flag / compact
 constexpr uint32_t kFirstBit = 0x80000000u;   // marks a first occurrence in slot[]
 constexpr int64_t kMaxMappingIds = int64_t(1) << 30;
-
-__device__ __forceinline__ uint32_t hash_id(uint64_t k) {
-  uint32_t h = uint32_t(k) ^ (uint32_t(k >> 32) * 0x9E3779B1u);
-  h ^= h >> 16; h *= 0x85EBCA6Bu;
-  h ^= h >> 13; h *= 0xC2B2AE35u;
-  h ^= h >> 16;
-  return h;
-}
 
 // Element i of the logical concatenation, or of a single array when count == 1.
 template <typename IdT>
@@ -66,32 +59,16 @@ __global__ __launch_bounds__(kThreads) void fill_ones_kernel(uint4* __restrict__
   if (i < n16) p[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
 }
 
-template <typename IdT> struct AtomicWord;
-template <> struct AtomicWord<int64_t> { using type = unsigned long long; };
-template <> struct AtomicWord<int32_t> { using type = unsigned int; };
-
-template <typename IdT>
-__global__ __launch_bounds__(kThreads) void insert_kernel(dgs_segments mapping, int64_t n,
-                                                          IdT* __restrict__ keys,
-                                                          uint32_t* __restrict__ vals, uint32_t mask,
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kThreads) void insert_kernel(dgs_segments mapping, int64_t n, TableT table,
                                                           uint32_t* __restrict__ slot) {
-  using W = typename AtomicWord<IdT>::type;
   const int64_t i = int64_t(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= n) return;
-  const IdT key = seg_load<IdT>(mapping, i);
-  uint32_t pos = hash_id(uint64_t(int64_t(key))) & mask;
-  for (;;) {
-    IdT cur = keys[pos];
-    if (cur == IdT(-1)) cur = IdT(atomicCAS(reinterpret_cast<W*>(keys + pos), W(IdT(-1)), W(key)));
-    if (cur == IdT(-1) || cur == key) break;
-    pos = (pos + 1) & mask;
-  }
-  atomicMin(vals + pos, uint32_t(i));
-  slot[i] = pos;
+  slot[i] = table.insert(seg_load<IdT>(mapping, i), uint32_t(i));
 }
 
-__global__ __launch_bounds__(kThreads) void flag_kernel(int64_t n, const uint32_t* __restrict__ vals,
-                                                        uint32_t* __restrict__ slot,
+template <typename TableT>
+__global__ __launch_bounds__(kThreads) void flag_kernel(int64_t n, TableT table, uint32_t* __restrict__ slot,
                                                         int* __restrict__ tile_cnt) {
   __shared__ int lds[kThreads / kWave];
   const int64_t base = int64_t(blockIdx.x) * kTileIds + threadIdx.x * kItems;
@@ -101,7 +78,7 @@ __global__ __launch_bounds__(kThreads) void flag_kernel(int64_t n, const uint32_
     const int64_t i = base + j;
     if (i < n) {
       const uint32_t s = slot[i];
-      if (vals[s] == uint32_t(i)) {
+      if (table.value(s) == uint32_t(i)) {
         slot[i] = s | kFirstBit;
         ++c;
       }
@@ -120,11 +97,10 @@ __global__ __launch_bounds__(1024) void unique_scan_kernel(const int* __restrict
   if (threadIdx.x == 0) *num_unique_dev = sum;
 }
 
-template <typename IdT>
+template <typename IdT, typename TableT>
 __global__ __launch_bounds__(kThreads) void compact_kernel(dgs_segments mapping, int64_t n,
                                                            const uint32_t* __restrict__ slot,
-                                                           const int* __restrict__ tile_off,
-                                                           uint32_t* __restrict__ vals,
+                                                           const int* __restrict__ tile_off, TableT table,
                                                            IdT* __restrict__ unique_out) {
   __shared__ int lds[kThreads / kWave];
   const int64_t base = int64_t(blockIdx.x) * kTileIds + threadIdx.x * kItems;
@@ -141,60 +117,43 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(dgs_segments mapping,
   for (int j = 0; j < kItems; ++j) {
     if (s[j] & kFirstBit) {
       unique_out[rank] = seg_load<IdT>(mapping, base + j);
-      vals[s[j] & ~kFirstBit] = uint32_t(rank);
+      table.set_value(s[j] & ~kFirstBit, uint32_t(rank));
       ++rank;
     }
   }
 }
 
 // out[j] = rank of requiring[j], -1 when the id is not in the table.
-template <typename IdT>
-__global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring, int64_t m,
-                                                          const IdT* __restrict__ keys,
-                                                          const uint32_t* __restrict__ vals,
-                                                          uint32_t mask, dgs_segments out) {
+template <typename IdT, typename TableT>
+__global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring, int64_t m, TableT table,
+                                                          dgs_segments out) {
   const int64_t j = int64_t(blockIdx.x) * kThreads + threadIdx.x;
   if (j >= m) return;
-  const IdT key = seg_load<IdT>(requiring, j);
-  uint32_t pos = hash_id(uint64_t(int64_t(key))) & mask;
-  IdT r = IdT(-1);
-  for (;;) {
-    const IdT cur = keys[pos];
-    if (cur == key) { r = IdT(vals[pos]); break; }
-    if (cur == IdT(-1)) break;
-    pos = (pos + 1) & mask;
-  }
-  seg_store<IdT>(out, j, r);
+  const uint32_t s = table.find(seg_load<IdT>(requiring, j));
+  seg_store<IdT>(out, j, s > table.mask ? IdT(-1) : IdT(table.value(s)));
 }
 
 struct UniqueWorkspace {
-  void* keys;       // IdT[capacity]
-  uint32_t* vals;   // [capacity], directly after keys
-  uint32_t* slot;   // [n]
+  void* table;       // capacity slots of the table layout in use
+  uint32_t* slot;    // [n]
   int* tile_cnt;
   int* tile_off;
   uint32_t capacity;
-  size_t table_bytes;  // keys + vals, multiple of 16
+  size_t table_bytes;  // multiple of 16
 };
 
-uint32_t table_capacity(int64_t n) {
-  uint64_t c = 1024;
-  while (c < uint64_t(n) * 2) c <<= 1;
-  return uint32_t(c);
-}
+// 4-byte ids always fit the packed 64-bit slot; 8-byte ids get the id array + value array.
+size_t slot_bytes(int32_t id_bytes) { return id_bytes == 4 ? 8 : size_t(id_bytes) + 4; }
 
 size_t unique_workspace_layout(int64_t n, int32_t id_bytes, void* base, UniqueWorkspace* w) {
   if (n < 0) n = 0;
   if (n > kMaxMappingIds) n = kMaxMappingIds;
-  const uint32_t cap = table_capacity(n);
   const size_t tiles = size_t((n + kTileIds - 1) / kTileIds);
   Carver c(base);
   UniqueWorkspace t;
-  t.capacity = cap;
-  t.table_bytes = size_t(cap) * size_t(id_bytes) + size_t(cap) * sizeof(uint32_t);
-  char* table = c.take<char>(t.table_bytes);
-  t.keys = table;
-  t.vals = reinterpret_cast<uint32_t*>(table + size_t(cap) * size_t(id_bytes));
+  t.capacity = table_capacity(n);
+  t.table_bytes = size_t(t.capacity) * slot_bytes(id_bytes);
+  t.table = c.take<char>(t.table_bytes);
   t.slot = c.take<uint32_t>(size_t(n));
   t.tile_cnt = c.take<int>(tiles);
   t.tile_off = c.take<int>(tiles);
@@ -208,34 +167,34 @@ int64_t seg_total(const dgs_segments& s) {
   return t;
 }
 
-template <typename IdT>
+template <typename IdT, typename TableT>
 dgs_status run_unique_relabel(const dgs_segments& mapping, int64_t n, const dgs_segments& requiring,
                               int64_t m, void* unique_out, int64_t* num_unique_dev,
                               const dgs_segments& out, const UniqueWorkspace& w, hipStream_t st) {
-  IdT* keys = static_cast<IdT*>(w.keys);
-  const uint32_t mask = w.capacity - 1;
+  const TableT table(w.table, w.capacity);
   const int64_t n16 = int64_t(w.table_bytes / 16);
   hipLaunchKernelGGL(fill_ones_kernel, dim3(uint32_t((n16 + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
-                     static_cast<uint4*>(w.keys), n16);
+                     static_cast<uint4*>(w.table), n16);
   DGS_LAUNCH_CHECK();
   const int64_t tiles = (n + kTileIds - 1) / kTileIds;
   if (n > 0) {
-    hipLaunchKernelGGL(insert_kernel<IdT>, dim3(uint32_t((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
-                       mapping, n, keys, w.vals, mask, w.slot);
+    hipLaunchKernelGGL((insert_kernel<IdT, TableT>), dim3(uint32_t((n + kThreads - 1) / kThreads)), dim3(kThreads),
+                       0, st, mapping, n, table, w.slot);
     DGS_LAUNCH_CHECK();
-    hipLaunchKernelGGL(flag_kernel, dim3(uint32_t(tiles)), dim3(kThreads), 0, st, n, w.vals, w.slot, w.tile_cnt);
+    hipLaunchKernelGGL(flag_kernel<TableT>, dim3(uint32_t(tiles)), dim3(kThreads), 0, st, n, table, w.slot,
+                       w.tile_cnt);
     DGS_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL(unique_scan_kernel, dim3(1), dim3(1024), 0, st, w.tile_cnt, w.tile_off, tiles, num_unique_dev);
   DGS_LAUNCH_CHECK();
   if (n > 0) {
-    hipLaunchKernelGGL(compact_kernel<IdT>, dim3(uint32_t(tiles)), dim3(kThreads), 0, st, mapping, n, w.slot,
-                       w.tile_off, w.vals, static_cast<IdT*>(unique_out));
+    hipLaunchKernelGGL((compact_kernel<IdT, TableT>), dim3(uint32_t(tiles)), dim3(kThreads), 0, st, mapping, n,
+                       w.slot, w.tile_off, table, static_cast<IdT*>(unique_out));
     DGS_LAUNCH_CHECK();
   }
   if (m > 0) {
-    hipLaunchKernelGGL(lookup_kernel<IdT>, dim3(uint32_t((m + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
-                       requiring, m, keys, w.vals, mask, out);
+    hipLaunchKernelGGL((lookup_kernel<IdT, TableT>), dim3(uint32_t((m + kThreads - 1) / kThreads)), dim3(kThreads),
+                       0, st, requiring, m, table, out);
     DGS_LAUNCH_CHECK();
   }
   return DGS_OK;
@@ -280,7 +239,8 @@ DGS_API dgs_status dgs_unique_relabel(dgs_segments mapping, dgs_segments requiri
   UniqueWorkspace w;
   unique_workspace_layout(n, id_bytes, workspace, &w);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8
-             ? run_unique_relabel<int64_t>(mapping, n, requiring, m, unique_out, num_unique_dev, out, w, st)
-             : run_unique_relabel<int32_t>(mapping, n, requiring, m, unique_out, num_unique_dev, out, w, st);
+  return id_bytes == 8 ? run_unique_relabel<int64_t, Table<int64_t, false>>(mapping, n, requiring, m, unique_out,
+                                                                           num_unique_dev, out, w, st)
+                       : run_unique_relabel<int32_t, Table<int32_t, true>>(mapping, n, requiring, m, unique_out,
+                                                                          num_unique_dev, out, w, st);
 }
