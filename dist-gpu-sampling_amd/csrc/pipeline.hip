@@ -36,6 +36,7 @@
 #include <cstdlib>
 
 #include "common.h"
+#include "picks.h"
 #include "table.h"
 
 namespace dgs {
@@ -122,37 +123,6 @@ __device__ __forceinline__ T block_sum(T v, T* lds /* NT/64 */) {
   for (int w = 0; w < NT / kWave; ++w) s += lds[w];
   __syncthreads();
   return s;
-}
-
-// Position inside the row for output slot l of a row of degree deg (all G lanes of the
-// group call this together); returns false when the slot is empty.
-template <int G>
-__device__ __forceinline__ bool pick_position(uint32_t deg, int k, bool replace, int l, int group_lane0,
-                                              uint64_t rng_seed, uint32_t rng_stream, int64_t row,
-                                              uint32_t* pos) {
-  if (replace) {
-    if (deg == 0 || l >= k) return false;
-    *pos = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), deg);
-    return true;
-  }
-  if (deg <= uint32_t(k)) {
-    *pos = uint32_t(l);
-    return uint32_t(l) < deg;
-  }
-  // Floyd: slot s draws from [0, deg-k+s]; a value already kept by a lower slot is replaced
-  // by deg-k+s, which no lower slot can hold.
-  constexpr uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << (G & 63)) - 1);
-  const uint32_t top = deg - uint32_t(k) + uint32_t(l);
-  uint32_t cand = 0xffffffffu;
-  if (l < k) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), top + 1u);
-  uint32_t kept = cand;
-  for (int s = 1; s < k; ++s) {
-    const uint32_t c = __shfl(cand, s, G);
-    const uint64_t hit = (__ballot(kept == c && l < s) >> group_lane0) & group_mask;
-    if (l == s && hit) kept = top;
-  }
-  *pos = kept;
-  return l < k;
 }
 
 // ---- packed edge list of one hop (off the critical path) -----------------------------

@@ -1,15 +1,17 @@
-// Row-wise uniform neighbour sampling over CSC held in two-tier views.
+// Row-wise uniform neighbour sampling over CSC held in two-tier views: the per-hop operator
+// (exact-size outputs, any fanout).
 //
-// Three launches per hop, no host round trip:
-//   count : one thread per seed reads its indptr pair, keeps (start, degree) and
-//           reduces the pick counts of a 256-seed tile;
+// Three launches per hop, no host round trip in between:
+//   count : one thread per seed reads its indptr pair, keeps (start, degree), scans the pick
+//           counts of a 256-seed tile (offset inside the tile + tile total);
 //   scan  : one block turns the tile totals into tile offsets and the edge count;
-//   fill  : one block per tile rebuilds the per-row offsets with an in-block scan
-//           and hands each row to a group of G lanes (G = 8..64, the smallest
-//           power of two holding num_picks), so a wave64 serves 64/G rows at once.
-// Random picks follow the "dgs-philox-1" contract: every (seed, stream, row,
-// draw) names one Philox block, so results do not depend on the launch shape.
+//   fill  : num_picks <= 64: a group of G lanes per seed row over the whole grid (G = 8..64,
+//           the smallest power of two holding num_picks), so a wave64 serves 64/G rows;
+//           larger num_picks: one wave per row, Floyd's kept set in LDS.
+// Random picks follow the "dgs-philox-1" contract: every (seed, stream, row, draw) names one
+// Philox block, so results do not depend on the launch shape.
 #include "common.h"
+#include "picks.h"
 
 namespace dgs {
 namespace {
@@ -20,16 +22,11 @@ constexpr int kMaxLdsPicks = 2048;   // fill_wave_kernel keeps Floyd's set in LD
 constexpr int kFlagDegree = 1;       // some row has degree >= 2^32
 constexpr int kFlagPicks = 2;        // deg > num_picks > kMaxLdsPicks without replacement
 
-__host__ __device__ inline int64_t pick_count(int64_t deg, int64_t k, bool replace) {
-  if (replace) return deg == 0 ? 0 : k;
-  return deg < k ? deg : k;
-}
-
 template <typename IdT, typename PtrT>
 __global__ __launch_bounds__(kTile) void sample_count_kernel(
     const IdT* __restrict__ seeds, int64_t n_seeds, TierView<PtrT> indptr, int64_t k, bool replace,
-    int64_t* __restrict__ row_start, uint32_t* __restrict__ row_deg, int64_t* __restrict__ tile_sum,
-    int* __restrict__ tile_flag) {
+    int64_t* __restrict__ row_start, uint32_t* __restrict__ row_deg, int64_t* __restrict__ row_off,
+    int64_t* __restrict__ tile_sum, int* __restrict__ tile_flag) {
   __shared__ int64_t lds[kTile / kWave];
   __shared__ int flag;
   if (threadIdx.x == 0) flag = 0;
@@ -50,7 +47,8 @@ __global__ __launch_bounds__(kTile) void sample_count_kernel(
     c = pick_count(deg, k, replace);
   }
   int64_t total;
-  block_exclusive_scan<kTile, int64_t>(c, &total, lds);
+  const int64_t ex = block_exclusive_scan<kTile, int64_t>(c, &total, lds);
+  if (i < n_seeds) row_off[i] = ex;
   if (threadIdx.x == 0) {
     tile_sum[blockIdx.x] = total;
     tile_flag[blockIdx.x] = flag;
@@ -76,150 +74,81 @@ __global__ __launch_bounds__(1024) void sample_scan_kernel(const int64_t* __rest
   }
 }
 
-// Loads the tile's rows into LDS and scans their pick counts.
-struct TileRows {
-  int64_t start[kTile];
-  int64_t off[kTile];
-  int64_t id[kTile];
-  uint32_t deg[kTile];
-};
-
-template <typename IdT>
-__device__ __forceinline__ int load_tile(TileRows& t, int64_t* scan_lds, const IdT* __restrict__ seeds,
-                                         int64_t n_seeds, const int64_t* __restrict__ row_start,
-                                         const uint32_t* __restrict__ row_deg,
-                                         const int64_t* __restrict__ tile_off, int64_t k, bool replace) {
-  const int64_t base = int64_t(blockIdx.x) * kTile;
-  const int64_t i = base + threadIdx.x;
-  int64_t c = 0;
-  if (i < n_seeds) {
-    const uint32_t d = row_deg[i];
-    t.start[threadIdx.x] = row_start[i];
-    t.deg[threadIdx.x] = d;
-    t.id[threadIdx.x] = int64_t(seeds[i]);
-    c = pick_count(d, k, replace);
-  }
-  int64_t total;
-  const int64_t ex = block_exclusive_scan<kTile, int64_t>(c, &total, scan_lds);
-  t.off[threadIdx.x] = tile_off[blockIdx.x] + ex;
-  __syncthreads();
-  const int64_t left = n_seeds - base;
-  return left < kTile ? int(left) : kTile;
-}
-
-// num_picks <= 64: G lanes per row, lane l owns output slot l.
+// num_picks <= 64: G lanes per row over the whole grid, lane l owns output slot l.
 template <typename IdT, int G>
 __global__ __launch_bounds__(kTile) void fill_group_kernel(
     const IdT* __restrict__ seeds, int64_t n_seeds, const int64_t* __restrict__ row_start,
-    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ tile_off, TierView<IdT> indices,
-    int k, bool replace, uint64_t rng_seed, uint32_t rng_stream, IdT* __restrict__ out_rows,
-    IdT* __restrict__ out_cols) {
-  __shared__ TileRows t;
-  __shared__ int64_t scan_lds[kTile / kWave];
-  const int rows = load_tile<IdT>(t, scan_lds, seeds, n_seeds, row_start, row_deg, tile_off, k, replace);
-
-  constexpr int kGroups = kTile / G;
-  const int g = threadIdx.x / G;
-  const int l = threadIdx.x % G;
-  const int group_lane0 = (threadIdx.x & (kWave - 1)) - l;  // first lane of this group in its wave
-  const uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << G) - 1);
-
-  for (int r = g; r < rows; r += kGroups) {
-    const int64_t start = t.start[r];
-    const int64_t off = t.off[r];
-    const int64_t row = t.id[r];
-    const uint32_t deg = t.deg[r];
-    if (replace) {
-      if (deg > 0 && l < k) {
-        const uint32_t p = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), deg);
-        out_rows[off + l] = IdT(row);
-        out_cols[off + l] = indices.at(start + p);
-      }
-    } else if (deg <= uint32_t(k)) {
-      if (uint32_t(l) < deg) {
-        out_rows[off + l] = IdT(row);
-        out_cols[off + l] = indices.at(start + l);
-      }
-    } else {
-      // Floyd: slot s draws from [0, deg-k+s]; a value already kept by a lower slot is
-      // replaced by deg-k+s (which no lower slot can hold).
-      const uint32_t top = deg - uint32_t(k) + uint32_t(l);
-      uint32_t cand = 0xffffffffu;
-      if (l < k) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), top + 1u);
-      uint32_t kept = cand;
-      for (int s = 1; s < k; ++s) {
-        const uint32_t c = __shfl(cand, s, G);
-        const uint64_t hit = (__ballot(kept == c && l < s) >> group_lane0) & group_mask;
-        if (l == s && hit) kept = top;
-      }
-      if (l < k) {
-        out_rows[off + l] = IdT(row);
-        out_cols[off + l] = indices.at(start + kept);
-      }
-    }
-  }
+    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ row_off,
+    const int64_t* __restrict__ tile_off, TierView<IdT> indices, int k, bool replace, uint64_t rng_seed,
+    uint32_t rng_stream, IdT* __restrict__ out_rows, IdT* __restrict__ out_cols) {
+  const int64_t gid = int64_t(blockIdx.x) * kTile + threadIdx.x;
+  const int64_t i = gid / G;
+  const int l = int(gid % G);
+  if (i >= n_seeds) return;  // whole groups leave together
+  const int group_lane0 = (threadIdx.x & (kWave - 1)) - l;
+  const int64_t row = int64_t(seeds[i]);
+  uint32_t pos;
+  if (!pick_position<G>(row_deg[i], k, replace, l, group_lane0, rng_seed, rng_stream, row, &pos)) return;
+  const int64_t o = tile_off[i / kTile] + row_off[i] + l;
+  out_rows[o] = IdT(row);
+  out_cols[o] = indices.at(row_start[i] + pos);
 }
 
-// Any num_picks: one wave per row, lanes stride over the slots; Floyd's kept set
-// lives in LDS (num_picks <= kMaxLdsPicks when it is needed at all).
+// Any num_picks: one wave per row, lanes stride over the slots; Floyd's kept set lives in LDS
+// (num_picks <= kMaxLdsPicks whenever it is needed: larger requests were zeroed by the count pass).
 template <typename IdT>
 __global__ __launch_bounds__(kTile) void fill_wave_kernel(
     const IdT* __restrict__ seeds, int64_t n_seeds, const int64_t* __restrict__ row_start,
-    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ tile_off, TierView<IdT> indices,
-    int64_t k, bool replace, uint64_t rng_seed, uint32_t rng_stream, IdT* __restrict__ out_rows,
-    IdT* __restrict__ out_cols) {
+    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ row_off,
+    const int64_t* __restrict__ tile_off, TierView<IdT> indices, int64_t k, bool replace, uint64_t rng_seed,
+    uint32_t rng_stream, IdT* __restrict__ out_rows, IdT* __restrict__ out_cols) {
   extern __shared__ uint32_t kept_lds[];  // (kTile / kWave) * min(k, kMaxLdsPicks) entries
-  __shared__ TileRows t;
-  __shared__ int64_t scan_lds[kTile / kWave];
-  const int rows = load_tile<IdT>(t, scan_lds, seeds, n_seeds, row_start, row_deg, tile_off, k, replace);
-
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
+  const int64_t i = int64_t(blockIdx.x) * (kTile / kWave) + wave;
+  if (i >= n_seeds) return;  // whole waves leave together
   const int64_t kk = k < kMaxLdsPicks ? k : kMaxLdsPicks;
   uint32_t* kept = kept_lds + int64_t(wave) * kk;
-
-  for (int r = wave; r < rows; r += kTile / kWave) {
-    const int64_t start = t.start[r];
-    const int64_t off = t.off[r];
-    const int64_t row = t.id[r];
-    const uint32_t deg = t.deg[r];
-    if (replace) {
-      if (deg > 0) {
-        for (int64_t s = lane; s < k; s += kWave) {
-          const uint32_t p = philox_bounded(rng_seed, rng_stream, row, uint32_t(s), deg);
-          out_rows[off + s] = IdT(row);
-          out_cols[off + s] = indices.at(start + p);
-        }
-      }
-    } else if (int64_t(deg) <= k) {
-      for (uint32_t s = lane; s < deg; s += kWave) {
-        out_rows[off + s] = IdT(row);
-        out_cols[off + s] = indices.at(start + s);
-      }
-    } else {
-      // here k <= kMaxLdsPicks (larger requests were zeroed by the count pass)
-      const uint32_t base_top = deg - uint32_t(k);
-      for (int s0 = 0; s0 < int(k); s0 += kWave) {
-        const int s = s0 + lane;
-        uint32_t cand = 0xffffffffu;
-        if (s < k) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(s), base_top + s + 1u);
-        const int batch = int(k) - s0 < kWave ? int(k) - s0 : kWave;
-        for (int b = 0; b < batch; ++b) {
-          const uint32_t c = __shfl(cand, b, kWave);
-          const int slot = s0 + b;
-          bool hit = false;
-          for (int q = lane; q < slot; q += kWave) hit |= kept[q] == c;
-          const bool any = __ballot(hit) != 0;
-          if (lane == 0) kept[slot] = any ? base_top + uint32_t(slot) : c;
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
-      }
+  const int64_t start = row_start[i];
+  const int64_t off = tile_off[i / kTile] + row_off[i];
+  const int64_t row = int64_t(seeds[i]);
+  const uint32_t deg = row_deg[i];
+  if (replace) {
+    if (deg > 0) {
       for (int64_t s = lane; s < k; s += kWave) {
+        const uint32_t p = philox_bounded(rng_seed, rng_stream, row, uint32_t(s), deg);
         out_rows[off + s] = IdT(row);
-        out_cols[off + s] = indices.at(start + kept[s]);
+        out_cols[off + s] = indices.at(start + p);
       }
+    }
+  } else if (int64_t(deg) <= k) {
+    for (uint32_t s = lane; s < deg; s += kWave) {
+      out_rows[off + s] = IdT(row);
+      out_cols[off + s] = indices.at(start + s);
+    }
+  } else {
+    // Floyd, 64 candidates at a time; each is checked against everything kept so far
+    const uint32_t base_top = deg - uint32_t(k);
+    for (int s0 = 0; s0 < int(k); s0 += kWave) {
+      const int s = s0 + lane;
+      uint32_t cand = 0xffffffffu;
+      if (s < k) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(s), base_top + s + 1u);
+      const int batch = int(k) - s0 < kWave ? int(k) - s0 : kWave;
+      for (int b = 0; b < batch; ++b) {
+        const uint32_t c = __shfl(cand, b, kWave);
+        const int slot = s0 + b;
+        bool hit = false;
+        for (int q = lane; q < slot; q += kWave) hit |= kept[q] == c;
+        const bool any = __ballot(hit) != 0;
+        if (lane == 0) kept[slot] = any ? base_top + uint32_t(slot) : c;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+    }
+    for (int64_t s = lane; s < k; s += kWave) {
+      out_rows[off + s] = IdT(row);
+      out_cols[off + s] = indices.at(start + kept[s]);
     }
   }
 }
@@ -227,6 +156,7 @@ __global__ __launch_bounds__(kTile) void fill_wave_kernel(
 struct SampleWorkspace {
   int64_t* row_start;
   uint32_t* row_deg;
+  int64_t* row_off;
   int64_t* tile_sum;
   int64_t* tile_off;
   int* tile_flag;
@@ -239,6 +169,7 @@ size_t sample_workspace_layout(int64_t n_seeds, void* base, SampleWorkspace* w) 
   SampleWorkspace tmp;
   tmp.row_start = c.take<int64_t>(n);
   tmp.row_deg = c.take<uint32_t>(n);
+  tmp.row_off = c.take<int64_t>(n);
   tmp.tile_sum = c.take<int64_t>(tiles);
   tmp.tile_off = c.take<int64_t>(tiles);
   tmp.tile_flag = c.take<int>(tiles);
@@ -253,7 +184,7 @@ dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr,
   if (tiles > 0) {
     hipLaunchKernelGGL((sample_count_kernel<IdT, PtrT>), dim3(uint32_t(tiles)), dim3(kTile), 0, st,
                        static_cast<const IdT*>(seeds), n_seeds, TierView<PtrT>(indptr), k, replace,
-                       w.row_start, w.row_deg, w.tile_sum, w.tile_flag);
+                       w.row_start, w.row_deg, w.row_off, w.tile_sum, w.tile_flag);
     DGS_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL(sample_scan_kernel, dim3(1), dim3(1024), 0, st, w.tile_sum, w.tile_off, w.tile_flag,
@@ -263,11 +194,12 @@ dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr,
 }
 
 template <typename IdT, int G>
-void launch_group(int64_t tiles, const void* seeds, int64_t n_seeds, const SampleWorkspace& w,
+void launch_group(const void* seeds, int64_t n_seeds, const SampleWorkspace& w,
                   const dgs_view& indices, int k, bool replace, uint64_t rng_seed, uint32_t rng_stream,
                   void* out_rows, void* out_cols, hipStream_t st) {
-  hipLaunchKernelGGL((fill_group_kernel<IdT, G>), dim3(uint32_t(tiles)), dim3(kTile), 0, st,
-                     static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.tile_off,
+  const int64_t blocks = (n_seeds * G + kTile - 1) / kTile;
+  hipLaunchKernelGGL((fill_group_kernel<IdT, G>), dim3(uint32_t(blocks)), dim3(kTile), 0, st,
+                     static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.row_off, w.tile_off,
                      TierView<IdT>(indices), k, replace, rng_seed, rng_stream, static_cast<IdT*>(out_rows),
                      static_cast<IdT*>(out_cols));
 }
@@ -280,15 +212,16 @@ dgs_status run_fill(const void* seeds, int64_t n_seeds, const dgs_view& indices,
   if (tiles == 0 || k <= 0) return DGS_OK;
   if (k <= kMaxGroupPicks) {
     const int kk = int(k);
-    if (kk <= 8) launch_group<IdT, 8>(tiles, seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
-    else if (kk <= 16) launch_group<IdT, 16>(tiles, seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
-    else if (kk <= 32) launch_group<IdT, 32>(tiles, seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
-    else launch_group<IdT, 64>(tiles, seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
+    if (kk <= 8) launch_group<IdT, 8>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
+    else if (kk <= 16) launch_group<IdT, 16>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
+    else if (kk <= 32) launch_group<IdT, 32>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
+    else launch_group<IdT, 64>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
   } else {
     const int64_t kk = k < kMaxLdsPicks ? k : kMaxLdsPicks;
     const size_t lds = replace ? 0 : size_t(kTile / kWave) * size_t(kk) * sizeof(uint32_t);
-    hipLaunchKernelGGL((fill_wave_kernel<IdT>), dim3(uint32_t(tiles)), dim3(kTile), lds, st,
-                       static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.tile_off,
+    const int64_t blocks = (n_seeds + kTile / kWave - 1) / (kTile / kWave);
+    hipLaunchKernelGGL((fill_wave_kernel<IdT>), dim3(uint32_t(blocks)), dim3(kTile), lds, st,
+                       static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.row_off, w.tile_off,
                        TierView<IdT>(indices), k, replace, rng_seed, rng_stream, static_cast<IdT*>(out_rows),
                        static_cast<IdT*>(out_cols));
   }
@@ -310,7 +243,8 @@ dgs_status check_common(const char* who, const void* seeds, int32_t id_bytes, in
   DGS_REQUIRE(width_ok(id_bytes), DGS_ERR_INVALID, "%s: id width %d is not 4 or 8", who, id_bytes);
   DGS_REQUIRE(n_seeds >= 0 && num_picks >= 0, DGS_ERR_INVALID, "%s: n_seeds=%lld num_picks=%lld", who,
               (long long)n_seeds, (long long)num_picks);
-  DGS_REQUIRE((n_seeds + kTile - 1) / kTile <= 0x7fffffff, DGS_ERR_UNSUPPORTED, "%s: too many seeds", who);
+  // the widest fill launch spends one wave on a row: kTile / kWave rows a block, 31-bit grids
+  DGS_REQUIRE(n_seeds <= int64_t(0x7fffffff) * (kTile / kWave), DGS_ERR_UNSUPPORTED, "%s: too many seeds", who);
   DGS_REQUIRE(workspace != nullptr && workspace_bytes >= dgs_sample_workspace_bytes(n_seeds),
               DGS_ERR_WORKSPACE, "%s: workspace of %zu B, need %zu", who, workspace_bytes,
               dgs_sample_workspace_bytes(n_seeds));
