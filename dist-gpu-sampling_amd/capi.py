@@ -60,6 +60,10 @@ SIGNATURES = {
                                        c_vp, c_sz, c_vp]),
     "dgs_sample_neighbors": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32,
                                             c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_fill_weighted": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32, c_vp,
+                                                c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_neighbors_weighted": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, View, c_i64, c_i32, c_u64,
+                                                     c_u32, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_unique_relabel_workspace_bytes": (c_sz, [c_i64, c_i32]),
     "dgs_unique_relabel": (ctypes.c_int, [Segments, Segments, c_i32, c_vp, c_vp, Segments, c_vp, c_sz, c_vp]),
     "dgs_sample_blocks_plan": (ctypes.c_int, [c_i64, ctypes.POINTER(c_i64), c_i32, ctypes.POINTER(c_i64),
@@ -197,6 +201,33 @@ def sample_neighbors(seeds, indptr_view, indices_view, num_picks, replace, rng_s
     check(lib.dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr_view, indices_view, num_picks, int(replace),
                                    rng_seed, rng_stream, rows.data_ptr(), cols.data_ptr(), nnz.data_ptr(),
                                    ws.data_ptr(), nb, stream_ptr()))
+    cnt, flags = read_i64(nnz, 2)
+    return rows[:cnt], cols[:cnt], flags
+
+
+def sample_neighbors_weighted(seeds, indptr_view, indices_view, probs_view, num_picks, replace, rng_seed,
+                              rng_stream, two_step=False):
+    """Returns (coo_row, coo_col, flags)."""
+    n = seeds.numel()
+    nb = lib.dgs_sample_workspace_bytes(n)
+    ws = _ws(nb, seeds.device)
+    nnz = torch.empty(2, dtype=torch.int64, device=seeds.device)
+    w = seeds.element_size()
+    if two_step:
+        check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
+                                   ws.data_ptr(), nb, stream_ptr()))
+        cnt, flags = read_i64(nnz, 2)
+        rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
+        cols = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
+        check(lib.dgs_sample_fill_weighted(seeds.data_ptr(), w, n, indices_view, probs_view, num_picks,
+                                           int(replace), rng_seed, rng_stream, rows.data_ptr(), cols.data_ptr(),
+                                           ws.data_ptr(), nb, stream_ptr()))
+        return rows, cols, flags
+    rows = torch.empty(n * num_picks, dtype=seeds.dtype, device=seeds.device)
+    cols = torch.empty(n * num_picks, dtype=seeds.dtype, device=seeds.device)
+    check(lib.dgs_sample_neighbors_weighted(seeds.data_ptr(), w, n, indptr_view, indices_view, probs_view,
+                                            num_picks, int(replace), rng_seed, rng_stream, rows.data_ptr(),
+                                            cols.data_ptr(), nnz.data_ptr(), ws.data_ptr(), nb, stream_ptr()))
     cnt, flags = read_i64(nnz, 2)
     return rows[:cnt], cols[:cnt], flags
 

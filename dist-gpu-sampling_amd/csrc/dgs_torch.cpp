@@ -241,16 +241,23 @@ dgs_view tensor_view(const torch::Tensor& t) {
   return v;
 }
 
-// Shared body of the two sampling operators.
+// Shared body of the sampling operators; `probs` is null for the uniform ones.
 std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_in, const dgs_view& indptr,
                                                      const dgs_view& indices, torch::ScalarType indices_dtype,
-                                                     int64_t num_picks, bool replace) {
+                                                     int64_t num_picks, bool replace,
+                                                     const dgs_view* probs = nullptr) {
   DGS_CHECK_GPU(seeds_in);
   const int32_t w = id_width(seeds_in, "seeds");
   TORCH_CHECK(seeds_in.scalar_type() == indices_dtype, "seeds (", seeds_in.scalar_type(), ") and indices (",
               indices_dtype, ") must have the same dtype");
   TORCH_CHECK(indptr.elem_bytes == 4 || indptr.elem_bytes == 8, "indptr must be int32 or int64");
   TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0, got ", num_picks);
+  if (probs != nullptr) {
+    TORCH_CHECK(probs->total == indices.total, "probs holds ", probs->total, " weights for ", indices.total,
+                " edges");
+    TORCH_CHECK(replace || num_picks <= 64,
+                "weighted sampling without replacement supports num_picks <= 64, got ", num_picks);
+  }
   torch::Tensor seeds = seeds_in.contiguous().view({-1});
   const int64_t n = seeds.numel();
   const auto rng = next_rng();
@@ -268,9 +275,14 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
   if (one_shot) {
     rows = torch::empty({n * num_picks}, seeds.options());
     cols = torch::empty({n * num_picks}, seeds.options());
-    check(dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr, indices, num_picks, replace, rng.first, rng.second,
-                               rows.data_ptr(), cols.data_ptr(), nnz_dev.data_ptr<int64_t>(), ws.data_ptr(),
-                               ws_bytes, st));
+    if (probs != nullptr)
+      check(dgs_sample_neighbors_weighted(seeds.data_ptr(), w, n, indptr, indices, *probs, num_picks, replace,
+                                          rng.first, rng.second, rows.data_ptr(), cols.data_ptr(),
+                                          nnz_dev.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
+    else
+      check(dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr, indices, num_picks, replace, rng.first,
+                                 rng.second, rows.data_ptr(), cols.data_ptr(), nnz_dev.data_ptr<int64_t>(),
+                                 ws.data_ptr(), ws_bytes, st));
     len = read_back(nnz_dev, 2);
   } else {
     check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(),
@@ -278,8 +290,12 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
     len = read_back(nnz_dev, 2);
     rows = torch::empty({len[0]}, seeds.options());
     cols = torch::empty({len[0]}, seeds.options());
-    check(dgs_sample_fill(seeds.data_ptr(), w, n, indices, num_picks, replace, rng.first, rng.second,
-                          rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st));
+    if (probs != nullptr)
+      check(dgs_sample_fill_weighted(seeds.data_ptr(), w, n, indices, *probs, num_picks, replace, rng.first,
+                                     rng.second, rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st));
+    else
+      check(dgs_sample_fill(seeds.data_ptr(), w, n, indices, num_picks, replace, rng.first, rng.second,
+                            rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st));
   }
   TORCH_CHECK((len[1] & 1) == 0, "sample_neighbors: a seed row has a degree of 2^32 or more");
   TORCH_CHECK((len[1] & 2) == 0,
@@ -309,6 +325,35 @@ std::tuple<torch::Tensor, torch::Tensor> SampleNeighborsWithChunkTensor(torch::T
   TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
               "indptr store must be int32 or int64");
   return sample_impl(seeds, indptr->view(), indices->view(), indices->dtype(), num_picks, replace);
+}
+
+// upstream RowWiseSamplingProbCUDA (src/cuda/rowwise_sampling_probs.cu:265-279)
+std::tuple<torch::Tensor, torch::Tensor> SampleNeighborsWithProbs(torch::Tensor seeds, torch::Tensor indptr,
+                                                                  torch::Tensor indices, torch::Tensor probs,
+                                                                  int64_t num_picks, bool replace) {
+  DGS_CHECK_GPU(indptr);
+  DGS_CHECK_GPU(indices);
+  DGS_CHECK_GPU(probs);
+  id_width(indptr, "indptr");
+  id_width(indices, "indices");
+  TORCH_CHECK(probs.scalar_type() == torch::kFloat32, "probs must be float32, got ", probs.scalar_type());
+  torch::Tensor ip = indptr.contiguous();
+  torch::Tensor ix = indices.contiguous();
+  torch::Tensor pr = probs.contiguous().view({-1});
+  const dgs_view pv = tensor_view(pr);
+  return sample_impl(seeds, tensor_view(ip), tensor_view(ix), ix.scalar_type(), num_picks, replace, &pv);
+}
+
+// upstream RowWiseSamplingProbWithChunkTensorCUDA
+// (src/cuda/rowwise_sampling_probs_with_chunk_tensor.cu:281-293)
+std::tuple<torch::Tensor, torch::Tensor> SampleNeighborsWithProbsWithChunkTensor(
+    torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr, c10::intrusive_ptr<ChunkTensor> indices,
+    c10::intrusive_ptr<ChunkTensor> probs, int64_t num_picks, bool replace) {
+  TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
+              "indptr store must be int32 or int64");
+  TORCH_CHECK(probs->dtype() == torch::kFloat32, "probs store must be float32, got ", probs->dtype());
+  const dgs_view pv = probs->view();
+  return sample_impl(seeds, indptr->view(), indices->view(), indices->dtype(), num_picks, replace, &pv);
 }
 
 // Packs up to DGS_MAX_SEGMENTS tensors; more are concatenated first.
@@ -519,6 +564,8 @@ TORCH_LIBRARY(dgs_ops, m) {
   m.def("_CAPI_tensor_relabel", &dgs::TensorRelabel)
       .def("_CAPI_sample_neighbors", &dgs::SampleNeighbors)
       .def("_CAPI_sample_neighbors_with_chunk_tensor", &dgs::SampleNeighborsWithChunkTensor)
+      .def("_CAPI_sample_neighbors_with_probs", &dgs::SampleNeighborsWithProbs)
+      .def("_CAPI_sample_neighbors_with_probs_with_chunk_tensor", &dgs::SampleNeighborsWithProbsWithChunkTensor)
       .def("_CAPI_get_unique_id", &dgs::GetUniqueId)
       .def("_CAPI_set_nccl", &dgs::SetNCCL)
       .def("_CAPI_get_current_allocated", &dgs::GetCurrentAllocated)

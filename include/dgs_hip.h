@@ -215,6 +215,46 @@ dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes,
                                 void* workspace, size_t workspace_bytes,
                                 void* stream);
 
+/*
+ * One weighted hop: like dgs_sample_neighbors with a float32 weight per edge
+ * (`probs`, a view of E floats laid out like `indices`).  Replaces
+ * RowWiseSamplingProbCUDA and RowWiseSamplingProbWithChunkTensorCUDA
+ * (src/cuda/rowwise_sampling_probs.cu:218-279,
+ * src/cuda/rowwise_sampling_probs_with_chunk_tensor.cu:181-293).  Pick counts are
+ * those of the uniform sampler, so dgs_sample_count is the shared first half.
+ *   - without replacement, deg <= num_picks: the whole row in CSC order;
+ *   - without replacement, deg > num_picks (num_picks <= 64; the reference
+ *     asserts <= 32): every position p races with the key E_p / w_p, E_p =
+ *     -ln((x + 0.5) / 2^32) for x = word p & 3 of the Philox block with counter
+ *     (0x80000000 | p >> 2, rng_stream, row), computed in float64 from exactly
+ *     rounded operations; weights that are not > 0 get the key +inf.  The
+ *     num_picks smallest (key, position) pairs win and are emitted in that order.
+ *     This is the reference's A-Res rule (largest u^(1/w)) in logarithms;
+ *   - with replacement, deg > 0: slot j picks position i with probability
+ *     q_i / sum(q), q_i = floor(2^32 * w_i / max(w)) (0 for weights not > 0):
+ *     the Philox block with counter (0x40000000 | j, rng_stream, row) is reduced to
+ *     [0, sum(q)) by Lemire's rule on its first 64 bits (second 64 bits accepted
+ *     unconditionally) and located by an upper bound on the inclusive sums of q;
+ *     a row with sum(q) == 0 picks its last position, like the reference's
+ *     clamped search (rowwise_sampling_probs.cu:203-204).
+ * Both rules are shared bit for bit with the CPU oracle.
+ */
+dgs_status dgs_sample_fill_weighted(const void* seeds, int32_t id_bytes,
+                                    int64_t n_seeds, dgs_view indices,
+                                    dgs_view probs, int64_t num_picks,
+                                    int32_t replace, uint64_t rng_seed,
+                                    uint32_t rng_stream, void* out_rows,
+                                    void* out_cols, void* workspace,
+                                    size_t workspace_bytes, void* stream);
+dgs_status dgs_sample_neighbors_weighted(const void* seeds, int32_t id_bytes,
+                                         int64_t n_seeds, dgs_view indptr,
+                                         dgs_view indices, dgs_view probs,
+                                         int64_t num_picks, int32_t replace,
+                                         uint64_t rng_seed, uint32_t rng_stream,
+                                         void* out_rows, void* out_cols,
+                                         int64_t* nnz_dev, void* workspace,
+                                         size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Unique + relabel                                                          */
 /* ------------------------------------------------------------------------ */

@@ -21,6 +21,14 @@
  *                        literal picks of the reference's cuRAND stream and of
  *                        DGL's CPU sampler: PARITY UNPINNED (neither can run here)
  *   unique / relabel     independent numpy computation (np.unique + first index)
+ *   neg_log_u32          math.log on the same argument (<= 2 ulp), monotone
+ *   weighted (deg > k)   brute force on tiny rows against the closed form of
+ *                        successive sampling; equal weights -> uniform subsets;
+ *                        zero weights lose every race
+ *   weighted, replace    frequencies against w / sum(w); quanta and inclusive
+ *                        sums against an independent numpy computation
+ *                        (literal picks of the reference's cuRAND stream:
+ *                        PARITY UNPINNED, as for the uniform sampler)
  *
  * Build: see oracle/Makefile (gcc -O2 -fopenmp -shared).
  */
@@ -271,6 +279,168 @@ ORACLE_API void oracle_sample_fill(const void* seeds, int id_bytes,
       }
     }
     free(picks);
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* Row-wise weighted sampling                                                */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * -ln((x + 0.5) / 2^32) from IEEE-754 basic operations only (exact integer
+ * conversions, one division, explicitly fused multiply-adds), so that the HIP
+ * kernel's copy of this routine returns the same bits.
+ *   u = t / 2^33 with t = 2x + 1;  t = m * 2^e, m in [1, 2), folded to
+ *   (sqrt(1/2), sqrt(2)];  ln m = 2 atanh(s), s = (m - 1) / (m + 1);
+ *   atanh series to s^21 (|s| <= 0.1716: the next term is below 2^-60).
+ */
+ORACLE_API double oracle_neg_log_u32(uint32_t x) {
+  static const double c[11] = {
+      0x1.0000000000000p+0, 0x1.5555555555555p-2, 0x1.999999999999ap-3,
+      0x1.2492492492492p-3, 0x1.c71c71c71c71cp-4, 0x1.745d1745d1746p-4,
+      0x1.3b13b13b13b14p-4, 0x1.1111111111111p-4, 0x1.e1e1e1e1e1e1ep-5,
+      0x1.af286bca1af28p-5, 0x1.8618618618618p-5};
+  const double ln2 = 0x1.62e42fefa39efp-1, sqrt2 = 0x1.6a09e667f3bcdp+0;
+  const uint64_t t = 2ull * x + 1ull;
+  int e = 63 - __builtin_clzll(t);
+  union { uint64_t u; double d; } scale;
+  scale.u = (uint64_t)(1023 - e) << 52; /* 2^-e */
+  double m = (double)t * scale.d;       /* exact */
+  if (m > sqrt2) { m *= 0.5; ++e; }
+  const double f = m - 1.0;             /* exact */
+  const double s = f / (2.0 + f);
+  const double z = s * s;
+  double p = c[10];
+  for (int i = 9; i >= 0; --i) p = __builtin_fma(p, z, c[i]);
+  const double r = s * p;
+  return __builtin_fma((double)(33 - e), ln2, -2.0 * r);
+}
+
+/* the four words of the Philox block that (row, j) names */
+static inline void draw_words(uint64_t seed, uint32_t stream, int64_t row,
+                              uint32_t j, uint32_t w[4]) {
+  uint32_t ctr[4] = {j, stream, (uint32_t)((uint64_t)row & 0xffffffffu),
+                     (uint32_t)((uint64_t)row >> 32)};
+  uint32_t key[2] = {(uint32_t)(seed & 0xffffffffu), (uint32_t)(seed >> 32)};
+  oracle_philox4x32_10(ctr, key, w);
+}
+
+/*
+ * Race key of neighbour position p: E / w with E a unit exponential variate,
+ * +inf for weights that are not > 0.  Keeping the k smallest keys is the
+ * A-Res rule of the reference (k largest u^(1/w),
+ * src/cuda/rowwise_sampling_probs.cu:102-118) in logarithms.
+ * Position p uses word p & 3 of block 0x80000000 | (p >> 2).
+ */
+ORACLE_API double oracle_weighted_key(uint64_t seed, uint32_t stream, int64_t row,
+                                      uint32_t p, float weight) {
+  uint32_t w[4];
+  draw_words(seed, stream, row, 0x80000000u | (p >> 2), w);
+  const double e = oracle_neg_log_u32(w[p & 3]);
+  const double wd = (double)weight;
+  return wd > 0.0 ? e / wd : __builtin_inf();
+}
+
+/* 32.32 fixed-point share of a weight in its row's largest weight */
+ORACLE_API uint64_t oracle_weight_quantum(float weight, float row_max) {
+  if (!(weight > 0.0f)) return 0;
+  const double r = (double)weight / (double)row_max;
+  return r > 0.0 ? (uint64_t)(r * 4294967296.0) : 0;
+}
+
+/* uniform in [0, n) from 64-bit words: Lemire's rule on (w0,w1), then (w2,w3)
+ * accepted unconditionally */
+ORACLE_API uint64_t oracle_bounded64(const uint32_t w[4], uint64_t n) {
+  unsigned __int128 m = 0;
+  for (int i = 0; i < 2; ++i) {
+    const uint64_t x = (uint64_t)w[2 * i] | ((uint64_t)w[2 * i + 1] << 32);
+    m = (unsigned __int128)x * n;
+    const uint64_t lo = (uint64_t)m;
+    if (lo >= n) break;
+    if (lo >= (0ull - n) % n) break;
+  }
+  return (uint64_t)(m >> 64);
+}
+
+typedef struct { double key; uint32_t pos; } race_t;
+static int race_cmp(const void* a, const void* b) {
+  const race_t* x = (const race_t*)a; const race_t* y = (const race_t*)b;
+  if (x->key < y->key) return -1;
+  if (x->key > y->key) return 1;
+  return x->pos < y->pos ? -1 : (x->pos > y->pos ? 1 : 0);
+}
+
+/*
+ * Weighted COO fill (src/cuda/rowwise_sampling_probs.cu:54-216 and
+ * rowwise_sampling_probs_with_chunk_tensor.cu:15-179); probs are float32, one
+ * per edge, stored like `indices`.
+ *   deg <= k, no replacement: the row in CSC order (:125-134);
+ *   deg > k, no replacement: the k smallest race keys, ties by position, emitted
+ *     in that order (the reference keeps the k largest u^(1/w) on a cuRAND
+ *     stream: same distribution, different literal picks);
+ *   replacement, deg > 0: k independent picks with P(i) = q_i / sum q, q the
+ *     32.32 quantum of w_i / max w (the reference scans float32 weights into a
+ *     CDF and searches u * total, :176-206: same distribution up to 2^-32 of the
+ *     largest weight); draw j is block 0x40000000 | j reduced to [0, sum q) and
+ *     located with an upper bound on the inclusive sums; a row without any
+ *     positive finite share picks its last neighbour, as the reference's
+ *     clamped search does (:203-204).
+ */
+ORACLE_API void oracle_sample_fill_weighted(
+    const void* seeds, int id_bytes, int64_t n_seeds, const void* ip_dev,
+    const void* ip_host, int64_t ip_thr, int ptr_bytes, const void* ix_dev,
+    const void* ix_host, int64_t ix_thr, const float* pr_dev, const float* pr_host,
+    int64_t pr_thr, int64_t k, int replace, uint64_t rng_seed, uint32_t rng_stream,
+    const int64_t* sub_indptr, void* out_rows, void* out_cols) {
+#pragma omp parallel for schedule(dynamic, 16)
+  for (int64_t i = 0; i < n_seeds; ++i) {
+    int64_t row = load_int(seeds, i, id_bytes);
+    int64_t b = at_int(ip_dev, ip_host, ip_thr, ptr_bytes, row);
+    int64_t e = at_int(ip_dev, ip_host, ip_thr, ptr_bytes, row + 1);
+    int64_t deg = e - b;
+    int64_t off = sub_indptr[i];
+#define PROB_AT(p) ((b + (p)) >= pr_thr ? pr_host[b + (p) - pr_thr] : pr_dev[b + (p)])
+    if (replace) {
+      if (deg == 0) continue;
+      float wmax = 0.0f;
+      for (int64_t p = 0; p < deg; ++p) { float w = PROB_AT(p); if (w > wmax) wmax = w; }
+      uint64_t* cdf = (uint64_t*)malloc(sizeof(uint64_t) * (size_t)deg);
+      uint64_t acc = 0;
+      for (int64_t p = 0; p < deg; ++p) { acc += oracle_weight_quantum(PROB_AT(p), wmax); cdf[p] = acc; }
+      for (int64_t j = 0; j < k; ++j) {
+        int64_t pick = deg - 1;
+        if (acc > 0) {
+          uint32_t w[4];
+          draw_words(rng_seed, rng_stream, row, 0x40000000u | (uint32_t)j, w);
+          const uint64_t r = oracle_bounded64(w, acc);
+          int64_t lo = 0, hi = deg - 1; /* first p with cdf[p] > r */
+          while (lo < hi) { int64_t mid = (lo + hi) / 2; if (cdf[mid] > r) hi = mid; else lo = mid + 1; }
+          pick = lo;
+        }
+        store_int(out_rows, off + j, id_bytes, row);
+        store_int(out_cols, off + j, id_bytes, at_int(ix_dev, ix_host, ix_thr, id_bytes, b + pick));
+      }
+      free(cdf);
+    } else if (deg <= k) {
+      for (int64_t j = 0; j < deg; ++j) {
+        store_int(out_rows, off + j, id_bytes, row);
+        store_int(out_cols, off + j, id_bytes, at_int(ix_dev, ix_host, ix_thr, id_bytes, b + j));
+      }
+    } else {
+      race_t* race = (race_t*)malloc(sizeof(race_t) * (size_t)deg);
+      for (int64_t p = 0; p < deg; ++p) {
+        race[p].key = oracle_weighted_key(rng_seed, rng_stream, row, (uint32_t)p, PROB_AT(p));
+        race[p].pos = (uint32_t)p;
+      }
+      qsort(race, (size_t)deg, sizeof(race_t), race_cmp);
+      for (int64_t j = 0; j < k; ++j) {
+        store_int(out_rows, off + j, id_bytes, row);
+        store_int(out_cols, off + j, id_bytes,
+                  at_int(ix_dev, ix_host, ix_thr, id_bytes, b + race[j].pos));
+      }
+      free(race);
+    }
+#undef PROB_AT
   }
 }
 

@@ -20,8 +20,10 @@ _lib = None
 
 def build(force=False):
     """Compile liboracle.so with the Makefile next to this file."""
-    if force or not os.path.exists(_LIB_PATH):
-        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "liboracle.so"])
+    stale = not os.path.exists(_LIB_PATH) or any(
+        os.path.getmtime(os.path.join(_HERE, f)) > os.path.getmtime(_LIB_PATH) for f in ("dgs_oracle.c", "Makefile"))
+    if force or stale:
+        subprocess.check_call(["make", "-C", _HERE, "-B", "-s", "liboracle.so"])
     return _LIB_PATH
 
 
@@ -34,6 +36,10 @@ def lib():
         _lib.oracle_draw.restype = ctypes.c_uint32
         _lib.oracle_sample_counts.restype = ctypes.c_int64
         _lib.oracle_unique_relabel.restype = ctypes.c_int64
+        _lib.oracle_neg_log_u32.restype = ctypes.c_double
+        _lib.oracle_weighted_key.restype = ctypes.c_double
+        _lib.oracle_weight_quantum.restype = ctypes.c_uint64
+        _lib.oracle_bounded64.restype = ctypes.c_uint64
     return _lib
 
 
@@ -148,6 +154,56 @@ def sample_neighbors(seeds, indptr, indices, num_picks, replace, rng_seed=0, rng
                              _p(ixh), _i64(ixt), _i64(num_picks), ctypes.c_int(int(replace)),
                              ctypes.c_uint64(rng_seed), ctypes.c_uint32(rng_stream), _p(sub),
                              _p(rows), _p(cols))
+    return rows, cols
+
+
+def neg_log_u32(x):
+    """-ln((x + 0.5) / 2^32) as the weighted sampler computes it."""
+    return lib().oracle_neg_log_u32(ctypes.c_uint32(x))
+
+
+def weighted_key(seed, stream, row, p, weight):
+    return lib().oracle_weighted_key(ctypes.c_uint64(seed), ctypes.c_uint32(stream), _i64(row),
+                                     ctypes.c_uint32(p), ctypes.c_float(weight))
+
+
+def weight_quantum(weight, row_max):
+    return lib().oracle_weight_quantum(ctypes.c_float(weight), ctypes.c_float(row_max))
+
+
+def bounded64(words, n):
+    w = (ctypes.c_uint32 * 4)(*words)
+    return lib().oracle_bounded64(w, ctypes.c_uint64(n))
+
+
+def sample_neighbors_weighted(seeds, indptr, indices, probs, num_picks, replace, rng_seed=0,
+                              rng_stream=0, indptr_threshold=None, indices_threshold=None,
+                              probs_threshold=None):
+    """One weighted hop; returns (coo_row, coo_col) like _CAPI_sample_neighbors_with_probs."""
+    seeds = _ids(seeds)
+    indptr = _ids(indptr)
+    indices = _ids(indices)
+    probs = np.ascontiguousarray(probs, dtype=np.float32)
+    assert seeds.dtype == indices.dtype and probs.size == indices.size
+    ipt = indptr.size if indptr_threshold is None else indptr_threshold
+    ixt = indices.size if indices_threshold is None else indices_threshold
+    prt = probs.size if probs_threshold is None else probs_threshold
+    ipd, iph = _tiers(indptr, ipt)
+    ixd, ixh = _tiers(indices, ixt)
+    prd, prh = _tiers(probs, prt)
+    n = seeds.size
+    sub = np.zeros(n + 1, dtype=np.int64)
+    idb = ctypes.c_int(seeds.dtype.itemsize)
+    pb = ctypes.c_int(indptr.dtype.itemsize)
+    nnz = lib().oracle_sample_counts(_p(seeds), idb, _i64(n), _p(ipd), _p(iph), _i64(ipt), pb,
+                                     _i64(num_picks), ctypes.c_int(int(replace)), _p(sub))
+    rows = np.empty(nnz, dtype=seeds.dtype)
+    cols = np.empty(nnz, dtype=indices.dtype)
+    lib().oracle_sample_fill_weighted(_p(seeds), idb, _i64(n), _p(ipd), _p(iph), _i64(ipt), pb,
+                                      _p(ixd), _p(ixh), _i64(ixt), _p(prd), _p(prh), _i64(prt),
+                                      _i64(num_picks), ctypes.c_int(int(replace)),
+                                      ctypes.c_uint64(rng_seed), ctypes.c_uint32(rng_stream),
+                                      _p(sub), _p(rows), _p(cols))
     return rows, cols
 
 

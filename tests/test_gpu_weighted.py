@@ -1,0 +1,152 @@
+"""GPU parity of weighted row-wise sampling against the CPU oracle.  The picks are bit-exact:
+race keys are float64 values built from exactly rounded operations on both sides, and the
+with-replacement rule works on integer quanta."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import load_pkg, powerlaw_graph
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    return load_pkg()
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _np(t):
+    return t.cpu().numpy()
+
+
+def _weights(rng, n):
+    """Spread over many binades, with zeros, negatives, NaN and exact ties."""
+    w = (rng.random(n) ** 6 * 100.0).astype(np.float32)
+    w[rng.random(n) < 0.05] = 0.0
+    w[rng.random(n) < 0.01] = -1.0
+    w[rng.random(n) < 0.005] = np.nan
+    ties = rng.random(n) < 0.2
+    w[ties] = np.float32(0.5)
+    return w
+
+
+@pytest.fixture(scope="module")
+def graph():
+    rng = np.random.default_rng(17)
+    indptr, indices = powerlaw_graph(rng, 20000, 20, 6000)
+    return indptr, indices, _weights(rng, indices.size)
+
+
+@pytest.mark.parametrize("k,replace", [(1, False), (5, False), (15, False), (32, False), (33, False), (63, False),
+                                       (64, False), (1, True), (10, True), (64, True), (65, True), (150, True)])
+def test_weighted_parity_c_abi(pkg, oracle, graph, k, replace):
+    capi = pkg.capi
+    indptr, indices, probs = graph
+    rng = np.random.default_rng(100 + k)
+    seeds = rng.integers(0, 20000, size=3001).astype(np.int64)
+    want_r, want_c = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, replace, 0x5eed5eed77, 6)
+    ip, ix, pr = _dev(indptr), _dev(indices), _dev(probs)
+    for two_step in (False, True):
+        r, c, flags = capi.sample_neighbors_weighted(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix),
+                                                     capi.tensor_view(pr), k, replace, 0x5eed5eed77, 6,
+                                                     two_step=two_step)
+        assert flags == 0
+        assert np.array_equal(_np(r), want_r), (k, replace, two_step)
+        assert np.array_equal(_np(c), want_c), (k, replace, two_step)
+
+
+def test_weighted_row_lengths_around_the_wave_width(pkg, oracle):
+    # degrees 0..200 and a few long rows: every residue of the 64-wide passes, the first-chunk
+    # sort with padding lanes, the insertion path, and rows shorter than num_picks
+    capi = pkg.capi
+    rng = np.random.default_rng(4)
+    deg = np.concatenate([np.arange(0, 201), [255, 256, 257, 1023, 1024, 1025, 5000, 20000]])
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, deg.size, size=int(indptr[-1])).astype(np.int64)
+    probs = rng.random(indices.size).astype(np.float32)
+    probs[indptr[150]:indptr[151]] = 0.0   # a row without any positive weight
+    probs[indptr[160]:indptr[161]] = 2.0   # a row of ties: positions decide
+    probs[indptr[-2]:indptr[-2] + 19000] = 0.0  # a long row with few positive weights
+    seeds = np.arange(deg.size, dtype=np.int64)
+    ip, ix, pr = _dev(indptr), _dev(indices), _dev(probs)
+    for k, replace in [(7, False), (64, False), (7, True), (100, True)]:
+        want_r, want_c = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, replace, 31, 1)
+        r, c, _ = capi.sample_neighbors_weighted(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix),
+                                                 capi.tensor_view(pr), k, replace, 31, 1)
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c), (k, replace)
+
+
+@pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int32, np.int32), (np.int32, np.int64), (np.int64, np.int32)])
+def test_weighted_mixed_widths(pkg, oracle, id_dtype, ptr_dtype):
+    capi = pkg.capi
+    rng = np.random.default_rng(3)
+    indptr, indices = powerlaw_graph(rng, 5000, 15, 500, id_dtype=id_dtype, ptr_dtype=ptr_dtype)
+    probs = _weights(rng, indices.size)
+    seeds = rng.integers(0, 5000, size=1500).astype(id_dtype)
+    ip, ix, pr = _dev(indptr), _dev(indices), _dev(probs)
+    for k, replace in [(10, False), (7, True)]:
+        want_r, want_c = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, replace, 42, 1)
+        r, c, _ = capi.sample_neighbors_weighted(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix),
+                                                 capi.tensor_view(pr), k, replace, 42, 1)
+        assert r.dtype == _dev(seeds).dtype
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+
+
+def test_weighted_operators_and_tiers(pkg, oracle, graph):
+    indptr, indices, probs = graph
+    rng = np.random.default_rng(8)
+    seeds = rng.permutation(20000)[:2048].astype(np.int64)
+    # all three arrays split across HBM and host memory
+    ip_ct = pkg.ChunkTensor([indptr.size], torch.int64, 8 * 7001)
+    ip_ct._CAPI_load_from_tensor(torch.from_numpy(indptr))
+    ix_ct = pkg.ChunkTensor([indices.size], torch.int64, 8 * (indices.size // 3))
+    ix_ct._CAPI_load_from_tensor(torch.from_numpy(indices))
+    pr_ct = pkg.ChunkTensor([probs.size], torch.float32, 4 * (probs.size // 2))
+    pr_ct._CAPI_load_from_tensor(torch.from_numpy(probs))
+    for k, replace in [(10, False), (10, True)]:
+        pkg.set_rng_state(777, 2)
+        r, c = pkg.ops._CAPI_sample_neighbors_with_probs_with_chunk_tensor(_dev(seeds), ip_ct, ix_ct, pr_ct, k,
+                                                                           replace)
+        want_r, want_c = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, replace, 777, 2)
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+        assert pkg.ops._CAPI_get_rng_state() == [777, 3]
+        pkg.set_rng_state(777, 2)
+        r, c = pkg.ops._CAPI_sample_neighbors_with_probs(_dev(seeds), _dev(indptr), _dev(indices), _dev(probs), k,
+                                                         replace)
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+
+
+def test_weighted_argument_errors(pkg, graph):
+    indptr, indices, probs = graph
+    seeds = _dev(np.arange(10, dtype=np.int64))
+    ops = pkg.ops
+    with pytest.raises(RuntimeError, match="num_picks <= 64"):
+        ops._CAPI_sample_neighbors_with_probs(seeds, _dev(indptr), _dev(indices), _dev(probs), 65, False)
+    with pytest.raises(RuntimeError, match="float32"):
+        ops._CAPI_sample_neighbors_with_probs(seeds, _dev(indptr), _dev(indices), _dev(probs.astype(np.float64)), 5,
+                                              False)
+    with pytest.raises(RuntimeError, match="weights for"):
+        ops._CAPI_sample_neighbors_with_probs(seeds, _dev(indptr), _dev(indices), _dev(probs[:-1]), 5, False)
+    r, c = ops._CAPI_sample_neighbors_with_probs(seeds[:0], _dev(indptr), _dev(indices), _dev(probs), 5, False)
+    assert r.numel() == 0 and c.numel() == 0
+
+
+def test_weighted_inclusion_frequencies(pkg):
+    # 20000 rows with the same 40 weights, k = 1: P(position i) = w_i / W exactly
+    rng = np.random.default_rng(9)
+    deg, trials = 80, 20000
+    w = (rng.random(deg) + 0.05).astype(np.float32)
+    indptr = np.arange(0, (trials + 1) * deg, deg, dtype=np.int64)
+    indices = np.tile(np.arange(deg, dtype=np.int64), trials)
+    probs = np.tile(w, trials)
+    seeds = _dev(np.arange(trials, dtype=np.int64))
+    exp = w.astype(np.float64) / w.astype(np.float64).sum() * trials
+    for replace in (False, True):
+        pkg.set_rng_state(12, 0)
+        _, c = pkg.ops._CAPI_sample_neighbors_with_probs(seeds, _dev(indptr), _dev(indices), _dev(probs), 1, replace)
+        cnt = np.bincount(_np(c), minlength=deg).astype(float)
+        assert ((cnt - exp) ** 2 / exp).sum() < 124.8  # chi-square 79 dof, p = 0.001

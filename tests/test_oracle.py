@@ -267,3 +267,159 @@ def test_sample_blocks_structure(oracle):
         # every edge (src -> dst) is an edge of the graph
         for s, d in zip(src_ids[src_l][:200], dst_ids[dst_l][:200]):
             assert s in indices[indptr[d]:indptr[d + 1]]
+
+
+# ---- weighted sampling ----------------------------------------------------
+def _tiled_rows(weights, trials):
+    """`trials` rows that all have the same weights; neighbour ids = positions."""
+    deg = len(weights)
+    indptr = np.arange(0, (trials + 1) * deg, deg, dtype=np.int64)
+    indices = np.tile(np.arange(deg, dtype=np.int64), trials)
+    probs = np.tile(np.asarray(weights, dtype=np.float32), trials)
+    return indptr, indices, probs, np.arange(trials, dtype=np.int64)
+
+
+def test_neg_log_matches_libm(oracle):
+    rng = np.random.default_rng(5)
+    fold = int(2 ** 32 / math.sqrt(2))  # where the mantissa is folded from above sqrt(2) to below 1
+    xs = [0, 1, 2, 3, 2 ** 31 - 1, 2 ** 31, 2 ** 32 - 2, 2 ** 32 - 1] + list(range(fold - 50, fold + 50))
+    xs += [int(x) for x in rng.integers(0, 2 ** 32, size=20000)]
+    xs += [int(x) for x in 2 ** 32 - 1 - rng.integers(0, 4096, size=2000)]  # u close to 1: heavy cancellation
+    for x in xs:
+        got = oracle.neg_log_u32(x)
+        want = -math.log((x + 0.5) / 4294967296.0)  # the argument is exact in float64
+        assert abs(got - want) <= 2 * np.spacing(want), (x, got, want)
+    # monotone where neighbouring arguments straddle a power of two or the fold
+    for x0 in (fold - 200, 2 ** 31 - 200, 2 ** 30 - 200):
+        vals = [oracle.neg_log_u32(x) for x in range(x0, x0 + 400)]
+        assert all(a >= b for a, b in zip(vals, vals[1:]))
+
+
+def test_weighted_key_layout(oracle):
+    seed, stream, row = 0xfeedface12345678, 11, (3 << 32) | 77
+    for p, wgt in [(0, 1.0), (1, 0.25), (2, 3.5), (3, 1e-3), (4, 2.0), (1022, 7.0), (1023, 0.5)]:
+        w = oracle.philox((0x80000000 | (p >> 2), stream, row & 0xffffffff, row >> 32),
+                          (seed & 0xffffffff, seed >> 32))
+        want = -math.log((int(w[p & 3]) + 0.5) / 4294967296.0) / float(np.float32(wgt))
+        got = oracle.weighted_key(seed, stream, row, p, wgt)
+        assert abs(got - want) <= 4 * np.spacing(want), (p, got, want)
+    for bad in (0.0, -1.0, float("nan"), -float("inf")):
+        assert oracle.weighted_key(seed, stream, row, 5, bad) == float("inf")
+    assert oracle.weighted_key(seed, stream, row, 5, float("inf")) == 0.0
+
+
+def test_weighted_matches_successive_sampling(oracle):
+    # order of the race = order of successive draws without replacement:
+    # P(a then b) = w_a / W * w_b / (W - w_a)
+    weights, k, trials = [1.0, 2.0, 3.0, 4.0], 2, 120000
+    indptr, indices, probs, seeds = _tiled_rows(weights, trials)
+    rows, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, False, 2024, 3)
+    assert np.array_equal(rows, np.repeat(seeds, k))
+    pairs = cols.reshape(trials, k)
+    assert (pairs[:, 0] != pairs[:, 1]).all()
+    total = sum(weights)
+    chi2 = 0.0
+    for a, b in itertools.permutations(range(4), 2):
+        exp = trials * weights[a] / total * weights[b] / (total - weights[a])
+        cnt = int(((pairs[:, 0] == a) & (pairs[:, 1] == b)).sum())
+        chi2 += (cnt - exp) ** 2 / exp
+    assert chi2 < 31.26  # chi-square 11 dof, p = 0.001
+
+
+def test_weighted_equal_weights_give_uniform_subsets(oracle):
+    deg, k, trials = 5, 3, 50000
+    indptr, indices, probs, seeds = _tiled_rows([0.7] * deg, trials)
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, False, 7, 0)
+    picks = np.sort(cols.reshape(trials, k), axis=1)
+    assert (picks[:, 1:] != picks[:, :-1]).all()
+    codes = picks[:, 0] * 25 + picks[:, 1] * 5 + picks[:, 2]
+    cnt = np.array([(codes == a * 25 + b * 5 + c).sum() for a, b, c in itertools.combinations(range(deg), k)], float)
+    assert cnt.sum() == trials
+    exp = trials / len(cnt)
+    assert ((cnt - exp) ** 2 / exp).sum() < 27.88  # chi-square 9 dof, p = 0.001
+
+
+def test_weighted_non_positive_weights_lose(oracle):
+    weights = [0.0, 1.0, 0.0, 2.0, -1.0, float("nan"), 0.0]
+    indptr, indices, probs, seeds = _tiled_rows(weights, 500)
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 2, False, 1, 1)
+    assert (np.sort(cols.reshape(500, 2), axis=1) == [1, 3]).all()
+    # more picks than positive weights: still num_picks picks (as upstream), the rest by position
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 4, False, 1, 1)
+    got = cols.reshape(500, 4)
+    assert (np.sort(got[:, :2], axis=1) == [1, 3]).all() and (got[:, 2:] == [0, 2]).all()
+
+
+def test_weighted_full_row_and_counts(oracle):
+    rng = np.random.default_rng(8)
+    deg = rng.integers(0, 9, size=60)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, 60, size=int(indptr[-1])).astype(np.int64)
+    probs = rng.random(indices.size).astype(np.float32)
+    seeds = rng.permutation(60).astype(np.int64)
+    rows, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 8, False, 5, 5)
+    assert np.array_equal(rows, np.concatenate([np.full(deg[s], s) for s in seeds]))
+    assert np.array_equal(cols, np.concatenate([indices[indptr[s]:indptr[s + 1]] for s in seeds]))
+    rows, _ = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 3, True, 5, 5)
+    assert np.array_equal(rows, np.concatenate([np.full(3 if deg[s] else 0, s) for s in seeds]))
+
+
+def test_weighted_replace_frequencies(oracle):
+    weights, k, trials = [1.0, 2.0, 0.0, 3.0, 4.0], 8, 40000
+    indptr, indices, probs, seeds = _tiled_rows(weights, trials)
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, True, 99, 2)
+    cnt = np.bincount(cols, minlength=5).astype(float)
+    assert cnt[2] == 0
+    exp = np.array(weights) / sum(weights) * trials * k
+    keep = exp > 0
+    assert ((cnt[keep] - exp[keep]) ** 2 / exp[keep]).sum() < 16.27  # chi-square 3 dof, p = 0.001
+    # slots are independent draws: the pair (slot 0, slot 1) has product probabilities
+    two = cols.reshape(trials, k)[:, :2]
+    chi2 = 0.0
+    for a in (0, 1, 3, 4):
+        for b in (0, 1, 3, 4):
+            e = trials * weights[a] * weights[b] / 100.0
+            chi2 += (int(((two[:, 0] == a) & (two[:, 1] == b)).sum()) - e) ** 2 / e
+    assert chi2 < 37.70  # chi-square 15 dof, p = 0.001
+    # no positive weight at all: the last neighbour, as upstream's clamped search returns
+    indptr, indices, probs, seeds = _tiled_rows([0.0, -2.0, 0.0], 10)
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 4, True, 99, 2)
+    assert (cols == 2).all()
+
+
+def test_weighted_replace_against_numpy_cdf(oracle):
+    # quanta, inclusive sums and the upper-bound search recomputed with numpy and Python integers
+    rng = np.random.default_rng(21)
+    deg, k, seed, stream = 300, 70, 0x1122334455, 4
+    w = (rng.random(deg) ** 4).astype(np.float32)
+    w[rng.integers(0, deg, 20)] = 0.0
+    q = np.floor(w.astype(np.float64) / np.float64(w.max()) * 4294967296.0).astype(np.uint64)
+    assert [oracle.weight_quantum(float(x), float(w.max())) for x in w[:50]] == [int(x) for x in q[:50]]
+    cdf = np.cumsum(q)
+    total = int(cdf[-1])
+    indptr = np.array([0, 0, 0, deg], dtype=np.int64)  # the sampled row is id 2
+    _, cols = oracle.sample_neighbors_weighted(np.array([2]), indptr, np.arange(deg, dtype=np.int64), w, k,
+                                               True, seed, stream)
+    want = []
+    for j in range(k):
+        wd = [int(x) for x in oracle.philox((0x40000000 | j, stream, 2, 0), (seed & 0xffffffff, seed >> 32))]
+        x = wd[0] | (wd[1] << 32)
+        lo = (x * total) & (2 ** 64 - 1)
+        if lo < total and lo < (2 ** 64 - total) % total:
+            x = wd[2] | (wd[3] << 32)
+        r = (x * total) >> 64
+        want.append(int(np.searchsorted(cdf, np.uint64(r), side="right")))
+    assert list(cols) == want
+
+
+def test_bounded64_rejection_rule(oracle):
+    n = 2 ** 63 + 1  # 2^64 mod n = 2^63 - 1: x = 2 gives lo = 2 < threshold -> rejected
+    assert oracle.bounded64((2, 0, 0, 0x80000000), n) == ((0x80000000 << 32) * n) >> 64
+    assert oracle.bounded64((1, 0, 9, 9), n) == 0          # lo = n >= n: accepted at once
+    assert oracle.bounded64((0, 0x80000000, 9, 9), 3) == 1  # x = 2^63: lo = 2^63 >= 3
+    assert oracle.bounded64((0, 0, 5, 0), 3) == 0           # x = 0: lo = 0 < 2^64 mod 3 = 1 -> second pair
+    rng = np.random.default_rng(2)
+    cnt = np.zeros(7)
+    for _ in range(7000):
+        cnt[oracle.bounded64([int(x) for x in rng.integers(0, 2 ** 32, 4)], 7)] += 1
+    assert ((cnt - 1000) ** 2 / 1000).sum() < 22.46  # chi-square 6 dof, p = 0.001
