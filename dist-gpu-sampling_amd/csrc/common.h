@@ -148,11 +148,12 @@ __device__ __forceinline__ PhiloxWords philox4x32_10(uint32_t c0, uint32_t c1, u
                                                      uint32_t k0, uint32_t k1) {
 #pragma unroll
   for (int r = 0; r < 10; ++r) {
-    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
-    const uint32_t n0 = hi1 ^ c1 ^ k0;
-    const uint32_t n2 = hi0 ^ c3 ^ k1;
-    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+    // one 32x32->64 multiply each (v_mad_u64_u32) instead of separate high and low halves
+    const uint64_t p0 = uint64_t(0xD2511F53u) * c0;
+    const uint64_t p1 = uint64_t(0xCD9E8D57u) * c2;
+    const uint32_t n0 = uint32_t(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n2 = uint32_t(p0 >> 32) ^ c3 ^ k1;
+    c0 = n0; c1 = uint32_t(p1); c2 = n2; c3 = uint32_t(p0);
     k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
   }
   return PhiloxWords{{c0, c1, c2, c3}};

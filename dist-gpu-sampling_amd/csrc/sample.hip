@@ -12,12 +12,11 @@
 // Philox block, so results do not depend on the launch shape.
 #include "common.h"
 #include "picks.h"
-#include "weights.h"
+#include "sample_workspace.h"
 
 namespace dgs {
 namespace {
 
-constexpr int kTile = 256;           // seeds per block in count and fill
 constexpr int kMaxGroupPicks = 64;   // fill_group_kernel handles num_picks <= 64
 constexpr int kMaxLdsPicks = 2048;   // fill_wave_kernel keeps Floyd's set in LDS
 constexpr int kFlagDegree = 1;       // some row has degree >= 2^32
@@ -154,192 +153,6 @@ __global__ __launch_bounds__(kTile) void fill_wave_kernel(
   }
 }
 
-// ---- weighted rows (float32 weight per edge, stored like `indices`) ----
-
-constexpr uint64_t kNoKey = ~uint64_t(0);  // above every key, +inf included
-
-__device__ __forceinline__ bool race_less(uint64_t ka, uint32_t pa, uint64_t kb, uint32_t pb) {
-  return ka < kb || (ka == kb && pa < pb);
-}
-
-// Without replacement, num_picks <= 64: one wave per row keeps the num_picks smallest
-// (key, position) pairs in order, lane l holding the l-th; the first 64 positions are sorted by a
-// bitonic network, every later position that beats the current last one is inserted by a shift.
-template <typename IdT>
-__global__ __launch_bounds__(kTile) void fill_weighted_kernel(
-    const IdT* __restrict__ seeds, int64_t n_seeds, const int64_t* __restrict__ row_start,
-    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ row_off,
-    const int64_t* __restrict__ tile_off, TierView<IdT> indices, TierView<float> probs, int k,
-    uint64_t rng_seed, uint32_t rng_stream, IdT* __restrict__ out_rows, IdT* __restrict__ out_cols) {
-  const int wave = threadIdx.x / kWave;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t i = int64_t(blockIdx.x) * (kTile / kWave) + wave;
-  if (i >= n_seeds) return;  // whole waves leave together
-  const int64_t start = row_start[i];
-  const int64_t off = tile_off[i / kTile] + row_off[i];
-  const int64_t row = int64_t(seeds[i]);
-  const uint32_t deg = row_deg[i];
-  if (deg <= uint32_t(k)) {
-    if (uint32_t(lane) < deg) {
-      out_rows[off + lane] = IdT(row);
-      out_cols[off + lane] = indices.at(start + lane);
-    }
-    return;
-  }
-  uint64_t key = kNoKey;
-  uint32_t pos = 0xffffffffu;
-  if (uint32_t(lane) < deg) {
-    pos = uint32_t(lane);
-    key = weighted_key(rng_seed, rng_stream, row, pos, probs.at(start + pos));
-  }
-#pragma unroll
-  for (int size = 2; size <= kWave; size <<= 1) {
-#pragma unroll
-    for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      const uint64_t ok = __shfl_xor(key, stride, kWave);
-      const uint32_t op = __shfl_xor(pos, stride, kWave);
-      const bool take_min = ((lane & stride) == 0) == ((lane & size) == 0);
-      const bool swap = take_min ? race_less(ok, op, key, pos) : race_less(key, pos, ok, op);
-      if (swap) {
-        key = ok;
-        pos = op;
-      }
-    }
-  }
-  if (lane >= k) {
-    key = kNoKey;
-    pos = 0xffffffffu;
-  }
-  uint64_t last_key = __shfl(key, k - 1, kWave);
-  uint32_t last_pos = __shfl(pos, k - 1, kWave);
-  for (uint32_t base = kWave; base < deg; base += kWave) {  // base < 2^32 - 64: deg fits 32 bits
-    const uint32_t p = base + lane;
-    uint64_t ck = kNoKey;
-    if (p < deg) ck = weighted_key(rng_seed, rng_stream, row, p, probs.at(start + p));
-    uint64_t hits = __ballot(p < deg && race_less(ck, p, last_key, last_pos));
-    while (hits) {
-      const int b = __builtin_ctzll(hits);
-      hits &= hits - 1;
-      const uint64_t nk = __shfl(ck, b, kWave);
-      const uint32_t np = base + uint32_t(b);
-      if (!race_less(nk, np, last_key, last_pos)) continue;  // the bar moved since the ballot
-      const uint64_t pk = __shfl_up(key, 1, kWave);
-      const uint32_t pp = __shfl_up(pos, 1, kWave);
-      if (race_less(nk, np, key, pos)) {  // this lane's entry moves up one place or makes room
-        const bool shift = lane > 0 && race_less(nk, np, pk, pp);
-        key = shift ? pk : nk;
-        pos = shift ? pp : np;
-      }
-      if (lane >= k) {
-        key = kNoKey;
-        pos = 0xffffffffu;
-      }
-      last_key = __shfl(key, k - 1, kWave);
-      last_pos = __shfl(pos, k - 1, kWave);
-    }
-  }
-  if (lane < k) {
-    out_rows[off + lane] = IdT(row);
-    out_cols[off + lane] = indices.at(start + pos);
-  }
-}
-
-// With replacement: one wave per row makes three passes over the row's weights: largest weight,
-// sum of the 32.32 quanta, then a running inclusive sum against which up to 64 draws a time are
-// located (a draw r belongs to the first position whose inclusive sum exceeds r).
-template <typename IdT>
-__global__ __launch_bounds__(kTile) void fill_weighted_replace_kernel(
-    const IdT* __restrict__ seeds, int64_t n_seeds, const int64_t* __restrict__ row_start,
-    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ row_off,
-    const int64_t* __restrict__ tile_off, TierView<IdT> indices, TierView<float> probs, int64_t k,
-    uint64_t rng_seed, uint32_t rng_stream, IdT* __restrict__ out_rows, IdT* __restrict__ out_cols) {
-  const int wave = threadIdx.x / kWave;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t i = int64_t(blockIdx.x) * (kTile / kWave) + wave;
-  if (i >= n_seeds) return;  // whole waves leave together
-  const int64_t start = row_start[i];
-  const int64_t off = tile_off[i / kTile] + row_off[i];
-  const int64_t row = int64_t(seeds[i]);
-  const int64_t deg = int64_t(row_deg[i]);
-  if (deg == 0) return;
-
-  float wmax = 0.0f;
-  for (int64_t p = lane; p < deg; p += kWave) {
-    const float w = probs.at(start + p);
-    if (w > wmax) wmax = w;
-  }
-#pragma unroll
-  for (int d = kWave / 2; d > 0; d >>= 1) {
-    const float o = __shfl_xor(wmax, d, kWave);
-    if (o > wmax) wmax = o;
-  }
-  uint64_t total = 0;
-  for (int64_t p = lane; p < deg; p += kWave) total += weight_quantum(probs.at(start + p), wmax);
-#pragma unroll
-  for (int d = kWave / 2; d > 0; d >>= 1) total += __shfl_xor(total, d, kWave);
-
-  for (int64_t first = 0; first < k; first += kWave) {
-    const int64_t j = first + lane;
-    const bool active = j < k;
-    int64_t pick = deg - 1;  // a row without a positive finite share keeps its last neighbour
-    if (total > 0) {
-      uint64_t r = 0;
-      if (active) r = philox_bounded64(rng_seed, rng_stream, row, uint32_t(j), total);
-      uint64_t pending = __ballot(active);
-      uint64_t sum_before = 0;
-      for (int64_t cb = 0; cb < deg && pending; cb += kWave) {
-        const int64_t p = cb + lane;
-        uint64_t incl = p < deg ? weight_quantum(probs.at(start + p), wmax) : 0;
-#pragma unroll
-        for (int d = 1; d < kWave; d <<= 1) {
-          const uint64_t t = __shfl_up(incl, d, kWave);
-          if (lane >= d) incl += t;
-        }
-        incl += sum_before;
-        const uint64_t sum_after = __shfl(incl, kWave - 1, kWave);
-        uint64_t here = __ballot(active && r >= sum_before && r < sum_after);
-        pending &= ~here;
-        while (here) {
-          const int b = __builtin_ctzll(here);
-          here &= here - 1;
-          const uint64_t rb = __shfl(r, b, kWave);
-          const int item = __builtin_ctzll(__ballot(incl > rb));
-          if (lane == b) pick = cb + item;
-        }
-        sum_before = sum_after;
-      }
-    }
-    if (active) {
-      out_rows[off + j] = IdT(row);
-      out_cols[off + j] = indices.at(start + pick);
-    }
-  }
-}
-
-struct SampleWorkspace {
-  int64_t* row_start;
-  uint32_t* row_deg;
-  int64_t* row_off;
-  int64_t* tile_sum;
-  int64_t* tile_off;
-  int* tile_flag;
-};
-
-size_t sample_workspace_layout(int64_t n_seeds, void* base, SampleWorkspace* w) {
-  const size_t n = size_t(n_seeds < 0 ? 0 : n_seeds);
-  const size_t tiles = (n + kTile - 1) / kTile;
-  Carver c(base);
-  SampleWorkspace tmp;
-  tmp.row_start = c.take<int64_t>(n);
-  tmp.row_deg = c.take<uint32_t>(n);
-  tmp.row_off = c.take<int64_t>(n);
-  tmp.tile_sum = c.take<int64_t>(tiles);
-  tmp.tile_off = c.take<int64_t>(tiles);
-  tmp.tile_flag = c.take<int>(tiles);
-  if (w) *w = tmp;
-  return c.used + 256;
-}
-
 template <typename IdT, typename PtrT>
 dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr, int64_t k, bool replace,
                      const SampleWorkspace& w, int64_t* nnz_dev, hipStream_t st) {
@@ -392,27 +205,6 @@ dgs_status run_fill(const void* seeds, int64_t n_seeds, const dgs_view& indices,
   return DGS_OK;
 }
 
-template <typename IdT>
-dgs_status run_fill_weighted(const void* seeds, int64_t n_seeds, const dgs_view& indices, const dgs_view& probs,
-                             int64_t k, bool replace, uint64_t rng_seed, uint32_t rng_stream,
-                             const SampleWorkspace& w, void* out_rows, void* out_cols, hipStream_t st) {
-  if (n_seeds == 0 || k <= 0) return DGS_OK;
-  const int64_t blocks = (n_seeds + kTile / kWave - 1) / (kTile / kWave);
-  if (replace) {
-    hipLaunchKernelGGL((fill_weighted_replace_kernel<IdT>), dim3(uint32_t(blocks)), dim3(kTile), 0, st,
-                       static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.row_off, w.tile_off,
-                       TierView<IdT>(indices), TierView<float>(probs), k, rng_seed, rng_stream,
-                       static_cast<IdT*>(out_rows), static_cast<IdT*>(out_cols));
-  } else {
-    hipLaunchKernelGGL((fill_weighted_kernel<IdT>), dim3(uint32_t(blocks)), dim3(kTile), 0, st,
-                       static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.row_off, w.tile_off,
-                       TierView<IdT>(indices), TierView<float>(probs), int(k), rng_seed, rng_stream,
-                       static_cast<IdT*>(out_rows), static_cast<IdT*>(out_cols));
-  }
-  DGS_LAUNCH_CHECK();
-  return DGS_OK;
-}
-
 }  // namespace
 }  // namespace dgs
 
@@ -420,30 +212,11 @@ DGS_API size_t dgs_sample_workspace_bytes(int64_t n_seeds) {
   return dgs::sample_workspace_layout(n_seeds, nullptr, nullptr);
 }
 
-namespace {
-dgs_status check_common(const char* who, const void* seeds, int32_t id_bytes, int64_t n_seeds,
-                        int64_t num_picks, const void* workspace, size_t workspace_bytes) {
-  using namespace dgs;
-  DGS_REQUIRE(width_ok(id_bytes), DGS_ERR_INVALID, "%s: id width %d is not 4 or 8", who, id_bytes);
-  DGS_REQUIRE(n_seeds >= 0 && num_picks >= 0, DGS_ERR_INVALID, "%s: n_seeds=%lld num_picks=%lld", who,
-              (long long)n_seeds, (long long)num_picks);
-  // the widest fill launch spends one wave on a row: kTile / kWave rows a block, 31-bit grids
-  DGS_REQUIRE(n_seeds <= int64_t(0x7fffffff) * (kTile / kWave), DGS_ERR_UNSUPPORTED, "%s: too many seeds", who);
-  DGS_REQUIRE(workspace != nullptr && workspace_bytes >= dgs_sample_workspace_bytes(n_seeds),
-              DGS_ERR_WORKSPACE, "%s: workspace of %zu B, need %zu", who, workspace_bytes,
-              dgs_sample_workspace_bytes(n_seeds));
-  DGS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, DGS_ERR_WORKSPACE,
-              "%s: workspace must be 256-byte aligned", who);
-  DGS_REQUIRE(n_seeds == 0 || seeds != nullptr, DGS_ERR_INVALID, "%s: null seeds", who);
-  return DGS_OK;
-}
-}  // namespace
-
 DGS_API dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
                                     int64_t num_picks, int32_t replace, int64_t* nnz_dev, void* workspace,
                                     size_t workspace_bytes, void* stream) {
   using namespace dgs;
-  dgs_status s = check_common("sample_count", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
+  dgs_status s = check_sample_args("sample_count", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
   if (s != DGS_OK) return s;
   DGS_REQUIRE(width_ok(indptr.elem_bytes), DGS_ERR_INVALID, "sample_count: indptr width %d is not 4 or 8",
               indptr.elem_bytes);
@@ -464,7 +237,7 @@ DGS_API dgs_status dgs_sample_fill(const void* seeds, int32_t id_bytes, int64_t 
                                    void* out_rows, void* out_cols, void* workspace, size_t workspace_bytes,
                                    void* stream) {
   using namespace dgs;
-  dgs_status s = check_common("sample_fill", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
+  dgs_status s = check_sample_args("sample_fill", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
   if (s != DGS_OK) return s;
   DGS_REQUIRE(indices.elem_bytes == id_bytes, DGS_ERR_INVALID,
               "sample_fill: indices width %d differs from the seed width %d", indices.elem_bytes, id_bytes);
@@ -489,50 +262,4 @@ DGS_API dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes, int
   if (s != DGS_OK) return s;
   return dgs_sample_fill(seeds, id_bytes, n_seeds, indices, num_picks, replace, rng_seed, rng_stream, out_rows,
                          out_cols, workspace, workspace_bytes, stream);
-}
-
-DGS_API dgs_status dgs_sample_fill_weighted(const void* seeds, int32_t id_bytes, int64_t n_seeds,
-                                            dgs_view indices, dgs_view probs, int64_t num_picks, int32_t replace,
-                                            uint64_t rng_seed, uint32_t rng_stream, void* out_rows,
-                                            void* out_cols, void* workspace, size_t workspace_bytes,
-                                            void* stream) {
-  using namespace dgs;
-  dgs_status s = check_common("sample_fill_weighted", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
-  if (s != DGS_OK) return s;
-  DGS_REQUIRE(indices.elem_bytes == id_bytes, DGS_ERR_INVALID,
-              "sample_fill_weighted: indices width %d differs from the seed width %d", indices.elem_bytes, id_bytes);
-  DGS_REQUIRE(probs.elem_bytes == 4, DGS_ERR_INVALID, "sample_fill_weighted: weights must be float32 (width %d)",
-              probs.elem_bytes);
-  DGS_REQUIRE(probs.total == indices.total, DGS_ERR_INVALID,
-              "sample_fill_weighted: %lld weights for %lld edges", (long long)probs.total, (long long)indices.total);
-  DGS_REQUIRE(replace != 0 || num_picks <= kMaxGroupPicks, DGS_ERR_UNSUPPORTED,
-              "sample_fill_weighted: num_picks %lld above %d without replacement", (long long)num_picks,
-              kMaxGroupPicks);
-  DGS_REQUIRE(num_picks < (int64_t(1) << 30), DGS_ERR_UNSUPPORTED, "sample_fill_weighted: num_picks %lld too large",
-              (long long)num_picks);
-  DGS_REQUIRE(n_seeds == 0 || num_picks == 0 || (out_rows != nullptr && out_cols != nullptr), DGS_ERR_INVALID,
-              "sample_fill_weighted: null output");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  SampleWorkspace w;
-  sample_workspace_layout(n_seeds, workspace, &w);
-  const bool rep = replace != 0;
-  return id_bytes == 8 ? run_fill_weighted<int64_t>(seeds, n_seeds, indices, probs, num_picks, rep, rng_seed,
-                                                    rng_stream, w, out_rows, out_cols, st)
-                       : run_fill_weighted<int32_t>(seeds, n_seeds, indices, probs, num_picks, rep, rng_seed,
-                                                    rng_stream, w, out_rows, out_cols, st);
-}
-
-DGS_API dgs_status dgs_sample_neighbors_weighted(const void* seeds, int32_t id_bytes, int64_t n_seeds,
-                                                 dgs_view indptr, dgs_view indices, dgs_view probs,
-                                                 int64_t num_picks, int32_t replace, uint64_t rng_seed,
-                                                 uint32_t rng_stream, void* out_rows, void* out_cols,
-                                                 int64_t* nnz_dev, void* workspace, size_t workspace_bytes,
-                                                 void* stream) {
-  DGS_REQUIRE(replace != 0 || num_picks <= 64, DGS_ERR_UNSUPPORTED,
-              "sample_neighbors_weighted: num_picks %lld above 64 without replacement", (long long)num_picks);
-  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, num_picks, replace, nnz_dev, workspace,
-                                  workspace_bytes, stream);
-  if (s != DGS_OK) return s;
-  return dgs_sample_fill_weighted(seeds, id_bytes, n_seeds, indices, probs, num_picks, replace, rng_seed,
-                                  rng_stream, out_rows, out_cols, workspace, workspace_bytes, stream);
 }

@@ -37,29 +37,49 @@ __device__ __forceinline__ double neg_log_u32(uint32_t x) {
   return __builtin_fma(double(33 - e), 0x1.62e42fefa39efp-1, -2.0 * r);
 }
 
-// Race key of neighbour position p of `row`: a unit exponential variate over the weight, as the
-// bits of a non-negative double (they order like the values); +inf for weights that are not > 0.
-// Position p takes word p & 3 of the Philox block 0x80000000 | (p >> 2).
-__device__ __forceinline__ uint64_t weighted_key(uint64_t seed, uint32_t stream, int64_t row, uint32_t p,
-                                                 float weight) {
+// Race key of neighbour position p: a unit exponential variate (from the position's Philox word
+// x) over the weight, as the bits of a non-negative double (they order like the values).  A
+// weight that is not > 0 gets +inf with p in the low bits, so such keys are distinct and order by
+// position.  Position p of a row owns word p & 3 of the row's Philox block with counter word
+// 0x80000000 | (p >> 2).
+__device__ __forceinline__ uint64_t race_key(uint32_t x, float weight, uint32_t p) {
 #pragma clang fp contract(off)
-  const PhiloxWords b = philox4x32_10(0x80000000u | (p >> 2), stream, uint32_t(uint64_t(row)),
-                                      uint32_t(uint64_t(row) >> 32), uint32_t(seed), uint32_t(seed >> 32));
-  const uint32_t lo = (p & 1) ? b.w[1] : b.w[0];
-  const uint32_t hi = (p & 1) ? b.w[3] : b.w[2];
-  const double e = neg_log_u32((p & 2) ? hi : lo);
   const double w = double(weight);
-  const double key = w > 0.0 ? e / w : __builtin_inf();
-  return uint64_t(__double_as_longlong(key));
+  if (!(w > 0.0)) return 0x7ff0000000000000ull | p;
+  return uint64_t(__double_as_longlong(neg_log_u32(x) / w));
 }
 
-// 32.32 fixed-point share of a weight in its row's largest weight; sums of these are exact in
-// any order, which is what lets a parallel scan and a sequential one agree.
-__device__ __forceinline__ uint64_t weight_quantum(float weight, float row_max) {
-#pragma clang fp contract(off)
+// Scale of a row's integer shares: 32 - E with 2^(E-1) <= row_max < 2^E; row_max finite and > 0.
+__device__ __forceinline__ int quantum_shift(float row_max) {
+  const uint64_t bits = uint64_t(__double_as_longlong(double(row_max)));  // normal as a double
+  return 32 - (int((bits >> 52) & 0x7ff) - 1022);
+}
+
+// Integer share of a weight in its row: floor(w * 2^shift) < 2^32, exact because the scale is a
+// power of two; sums of shares are exact in any order, which is what lets a parallel scan and a
+// sequential one agree.  0 for weights that are not > 0.
+__device__ __forceinline__ uint64_t weight_quantum(float weight, int shift) {
   if (!(weight > 0.0f)) return 0;
-  const double r = double(weight) / double(row_max);
-  return r > 0.0 ? uint64_t(r * 4294967296.0) : 0;
+  return uint64_t(__double2uint_rz(ldexp(double(weight), shift)));
+}
+
+// What a row's shares are measured against: `shift` when the largest weight is finite and > 0.
+struct QuantumScale {
+  int shift;
+  bool none;      // no weight > 0: the row has no shares at all
+  bool infinite;  // the largest weight is +inf: infinite weights share 1, finite ones 0
+};
+__device__ __forceinline__ QuantumScale quantum_scale(float row_max) {
+  QuantumScale s;
+  s.none = !(row_max > 0.0f);
+  s.infinite = row_max > 3.4028234663852886e38f;
+  s.shift = (s.none || s.infinite) ? 0 : quantum_shift(row_max);
+  return s;
+}
+__device__ __forceinline__ uint64_t weight_quantum(float weight, const QuantumScale& s) {
+  if (s.none) return 0;
+  if (s.infinite) return weight > 3.4028234663852886e38f ? 1 : 0;
+  return weight_quantum(weight, s.shift);
 }
 
 // Draw j of `row` (block 0x40000000 | j) reduced to [0, n): multiply-shift with rejection on the

@@ -231,7 +231,8 @@ dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes,
  *     num_picks smallest (key, position) pairs win and are emitted in that order.
  *     This is the reference's A-Res rule (largest u^(1/w)) in logarithms;
  *   - with replacement, deg > 0: slot j picks position i with probability
- *     q_i / sum(q), q_i = floor(2^32 * w_i / max(w)) (0 for weights not > 0):
+ *     q_i / sum(q), q_i = floor(w_i * 2^(32-E)) with 2^(E-1) <= max(w) < 2^E
+ *     (an exact power-of-two scaling; 0 for weights not > 0):
  *     the Philox block with counter (0x40000000 | j, rng_stream, row) is reduced to
  *     [0, sum(q)) by Lemire's rule on its first 64 bits (second 64 bits accepted
  *     unconditionally) and located by an upper bound on the inclusive sums of q;

@@ -32,6 +32,7 @@
  *
  * Build: see oracle/Makefile (gcc -O2 -fopenmp -shared).
  */
+#include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -341,11 +342,19 @@ ORACLE_API double oracle_weighted_key(uint64_t seed, uint32_t stream, int64_t ro
   return wd > 0.0 ? e / wd : __builtin_inf();
 }
 
-/* 32.32 fixed-point share of a weight in its row's largest weight */
+/*
+ * Integer share of a weight: floor(w * 2^(32 - E)) with 2^(E-1) <= row_max < 2^E,
+ * so the largest weight of the row maps into [2^31, 2^32).  Scaling by a power
+ * of two is exact: the shares, and with them every partial sum, are integers
+ * that do not depend on the order of summation.  Weights that are not > 0 get
+ * no share; when the largest weight is +inf only infinite weights get one.
+ */
 ORACLE_API uint64_t oracle_weight_quantum(float weight, float row_max) {
-  if (!(weight > 0.0f)) return 0;
-  const double r = (double)weight / (double)row_max;
-  return r > 0.0 ? (uint64_t)(r * 4294967296.0) : 0;
+  if (!(weight > 0.0f) || !(row_max > 0.0f)) return 0;
+  if (row_max > 3.4028234663852886e38f) return weight > 3.4028234663852886e38f ? 1 : 0;
+  int e;
+  (void)frexp((double)row_max, &e); /* row_max = f * 2^e, 0.5 <= f < 1 */
+  return (uint64_t)ldexp((double)weight, 32 - e);
 }
 
 /* uniform in [0, n) from 64-bit words: Lemire's rule on (w0,w1), then (w2,w3)
@@ -378,10 +387,10 @@ static int race_cmp(const void* a, const void* b) {
  *   deg > k, no replacement: the k smallest race keys, ties by position, emitted
  *     in that order (the reference keeps the k largest u^(1/w) on a cuRAND
  *     stream: same distribution, different literal picks);
- *   replacement, deg > 0: k independent picks with P(i) = q_i / sum q, q the
- *     32.32 quantum of w_i / max w (the reference scans float32 weights into a
- *     CDF and searches u * total, :176-206: same distribution up to 2^-32 of the
- *     largest weight); draw j is block 0x40000000 | j reduced to [0, sum q) and
+ *   replacement, deg > 0: k independent picks with P(i) = q_i / sum q, q_i the
+ *     integer share floor(w_i * 2^(32-E)) for 2^(E-1) <= max w < 2^E (the
+ *     reference scans float32 weights into a CDF and searches u * total,
+ *     :176-206: same distribution up to 2^-31 of the largest weight); draw j is block 0x40000000 | j reduced to [0, sum q) and
  *     located with an upper bound on the inclusive sums; a row without any
  *     positive finite share picks its last neighbour, as the reference's
  *     clamped search does (:203-204).

@@ -71,6 +71,8 @@ def test_weighted_row_lengths_around_the_wave_width(pkg, oracle):
     probs[indptr[150]:indptr[151]] = 0.0   # a row without any positive weight
     probs[indptr[160]:indptr[161]] = 2.0   # a row of ties: positions decide
     probs[indptr[-2]:indptr[-2] + 19000] = 0.0  # a long row with few positive weights
+    for row in (170, 190, 205, 207):                # infinite weights: race keys tie at 0, positions decide;
+        probs[indptr[row]:indptr[row + 1]:3] = np.inf  # with replacement only they hold a share
     seeds = np.arange(deg.size, dtype=np.int64)
     ip, ix, pr = _dev(indptr), _dev(indices), _dev(probs)
     for k, replace in [(7, False), (64, False), (7, True), (100, True)]:
@@ -78,6 +80,23 @@ def test_weighted_row_lengths_around_the_wave_width(pkg, oracle):
         r, c, _ = capi.sample_neighbors_weighted(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix),
                                                  capi.tensor_view(pr), k, replace, 31, 1)
         assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c), (k, replace)
+
+
+@pytest.mark.parametrize("group", ["16", "32", "64"])
+def test_weighted_every_group_width(pkg, oracle, graph, group, monkeypatch):
+    # the library picks the lanes-per-row from num_picks; the hook forces each width (and with it
+    # each long-row threshold) over the same inputs
+    monkeypatch.setenv("DGS_WEIGHTED_GROUP", group)
+    capi = pkg.capi
+    indptr, indices, probs = graph
+    rng = np.random.default_rng(int(group))
+    seeds = rng.integers(0, 20000, size=4000).astype(np.int64)
+    ip, ix, pr = _dev(indptr), _dev(indices), _dev(probs)
+    for k, replace in [(3, False), (12, False), (16, False), (5, True), (40, True)]:
+        want_r, want_c = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, replace, 77, 9)
+        r, c, _ = capi.sample_neighbors_weighted(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix),
+                                                 capi.tensor_view(pr), k, replace, 77, 9)
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c), (group, k, replace)
 
 
 @pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int32, np.int32), (np.int32, np.int64), (np.int64, np.int32)])

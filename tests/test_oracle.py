@@ -387,13 +387,29 @@ def test_weighted_replace_frequencies(oracle):
     assert (cols == 2).all()
 
 
+def test_weighted_infinite_weights(oracle):
+    weights = [1.0, float("inf"), 5.0, float("inf"), 2.0, float("inf")]
+    indptr, indices, probs, seeds = _tiled_rows(weights, 3000)
+    # without replacement: keys 0 for the infinite weights, taken first and in position order
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 4, False, 6, 0)
+    got = cols.reshape(3000, 4)
+    assert (got[:, :3] == [1, 3, 5]).all() and np.isin(got[:, 3], [0, 2, 4]).all()
+    # with replacement: only they hold a share, equally
+    _, cols = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, 6, True, 6, 0)
+    cnt = np.bincount(cols, minlength=6).astype(float)
+    assert cnt[[0, 2, 4]].sum() == 0
+    assert ((cnt[[1, 3, 5]] - 6000) ** 2 / 6000).sum() < 13.82  # chi-square 2 dof, p = 0.001
+
+
 def test_weighted_replace_against_numpy_cdf(oracle):
     # quanta, inclusive sums and the upper-bound search recomputed with numpy and Python integers
     rng = np.random.default_rng(21)
     deg, k, seed, stream = 300, 70, 0x1122334455, 4
     w = (rng.random(deg) ** 4).astype(np.float32)
     w[rng.integers(0, deg, 20)] = 0.0
-    q = np.floor(w.astype(np.float64) / np.float64(w.max()) * 4294967296.0).astype(np.uint64)
+    shift = 32 - math.frexp(float(w.max()))[1]  # 2^(E-1) <= max w < 2^E, shares = floor(w * 2^(32-E))
+    q = np.floor(np.ldexp(w.astype(np.float64), shift)).astype(np.uint64)
+    assert 2 ** 31 <= int(q.max()) < 2 ** 32
     assert [oracle.weight_quantum(float(x), float(w.max())) for x in w[:50]] == [int(x) for x in q[:50]]
     cdf = np.cumsum(q)
     total = int(cdf[-1])
