@@ -32,6 +32,11 @@ WORKLOADS = {
     # BASELINE.json configs[1]: the configuration the metric is quoted on
     "c1": dict(nodes=2_449_029, edges=123_718_280, max_deg=17_000, deg1_frac=0.05, feat_dim=100,
                feat_dtype="float32", batch=1024, fanouts=[15, 10, 5], replace=False, graph_seed=20240602),
+    # c1 with a float32 weight per edge: every hop uses the weighted operator
+    # (upstream ChunkTensorSampler with chunk_probs), per-hop path, then the same gather
+    "c1w": dict(nodes=2_449_029, edges=123_718_280, max_deg=17_000, deg1_frac=0.05, feat_dim=100,
+                feat_dtype="float32", batch=1024, fanouts=[15, 10, 5], replace=False, graph_seed=20240602,
+                weighted=True),
     # BASELINE.json configs[0] (CPU-runnable plumbing case), used by --workload c0
     "c0": dict(nodes=10_000, edges=200_000, max_deg=1_000, deg1_frac=0.0, feat_dim=128,
                feat_dtype="float32", batch=1024, fanouts=[10, 5], replace=False, graph_seed=20240601),
@@ -92,7 +97,13 @@ def algorithmic_bytes(stats, feat_dim, feat_bytes, w_id=8, w_ptr=8):
     return b_s, b_u, b_g
 
 
-def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0):
+def make_weights(cfg, n_edges):
+    """Edge weights of the weighted workload: uniform in (0.01, 1.01)."""
+    g = torch.Generator().manual_seed(cfg["graph_seed"] + 4)
+    return torch.rand(n_edges, generator=g, dtype=torch.float32) + 0.01
+
+
+def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0, probs=None):
     """The CPU oracle (a port of the reference algorithm, OpenMP over seed rows) plus
     torch.index_select, timed on this machine's host cores on a bounded sample of the
     same batches."""
@@ -102,6 +113,7 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0):
     os.environ["OMP_NUM_THREADS"] = str(threads)
     torch.set_num_threads(threads)
     ip, ix = indptr.numpy(), indices.numpy()
+    pr = None if probs is None else probs.numpy()
     edges = rows = 0
     t_sample = t_gather = 0.0
     done = 0
@@ -113,7 +125,7 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0):
             yield torch.randint(0, cfg["nodes"], (cfg["batch"],), generator=extra, dtype=torch.int64)
     for b in more():
         t0 = time.perf_counter()
-        frontier, _, blocks = oracle.sample_blocks(b.numpy(), ip, ix, cfg["fanouts"], cfg["replace"], 1, 0)
+        frontier, _, blocks = oracle.sample_blocks(b.numpy(), ip, ix, cfg["fanouts"], cfg["replace"], 1, 0, probs=pr)
         t1 = time.perf_counter()
         x = torch.index_select(feats, 0, torch.from_numpy(frontier))
         t2 = time.perf_counter()
@@ -363,7 +375,11 @@ def main():
     ct_indptr = dgs.create_chunktensor(indptr, 1, big)
     ct_indices = dgs.create_chunktensor(indices, 1, big)
     ct_feats = dgs.create_chunktensor(feats, 1, big)
-    sampler = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, replace=cfg["replace"])
+    probs = ct_probs = None
+    if cfg.get("weighted"):
+        probs = make_weights(cfg, indices.numel())
+        ct_probs = dgs.create_chunktensor(probs, 1, big)
+    sampler = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, ct_probs, replace=cfg["replace"])
 
     n_batches = args.steps + args.warmup
     batches_cpu = make_batches(cfg, n_batches)
@@ -445,7 +461,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {cfg['nodes']} nodes / {cfg['edges']} edges CSC int64, "
                                f"features {cfg['feat_dtype']} x{cfg['feat_dim']}, all in HBM, batch {cfg['batch']} "
-                               f"uniform seeds, fanouts {cfg['fanouts']} without replacement, then gather",
+                               f"uniform seeds, fanouts {cfg['fanouts']} without replacement"
+                               f"{', weighted by a float32 weight per edge' if cfg.get('weighted') else ''}, then gather",
                    "fanouts": cfg["fanouts"], "batch": cfg["batch"]},
         "sample_edges_per_s": edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
@@ -458,12 +475,26 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gather_flat_kernel (ChunkTensor._CAPI_index)",
                      "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gather_gbps / HBM_PEAK_GBPS,
-                     "traffic": (C1_GATHER_TRAFFIC_BYTES_PER_ROW * rows / args.steps) if args.workload == "c1" else None,
+                     "traffic": (C1_GATHER_TRAFFIC_BYTES_PER_ROW * rows / args.steps) if args.workload in ("c1", "c1w") else None,
                      "algorithmic_bytes": bg / args.steps, "avg_launch_us": 1e3 * ms_gather},
         "graph_gen_s": t_gen,
     }
+    if cfg.get("weighted"):
+        # the weighted fill of the widest hop alone: its input is every weight of every sampled row
+        ops = torch.ops.dgs_ops
+        seeds = blocks[0].dst_ids
+        k = cfg["fanouts"][0]
+        ip_dev = ct_indptr._CAPI_get_sub_device_tensor()
+        degs = ip_dev[seeds + 1] - ip_dev[seeds]
+        scanned = int(degs[degs > k].sum().item())
+        t = time_call(lambda: ops._CAPI_sample_neighbors_with_probs_with_chunk_tensor(
+            seeds, ct_indptr, ct_indices, ct_probs, k, cfg["replace"]), 10)
+        out["weighted_hop"] = {"seeds": seeds.numel(), "num_picks": k, "weights_scanned": scanned,
+                               "us_per_call": 1e6 * t, "weights_per_s": scanned / t,
+                               "weights_GBps": 4 * scanned / t / 1e9,
+                               "hbm_frac_of_weight_bytes": 4 * scanned / t / 1e9 / HBM_PEAK_GBPS}
     if not args.no_cpu_baseline:
-        cb = cpu_baseline(cfg, indptr, indices, feats, batches_cpu[args.warmup:], args.cpu_budget_s)
+        cb = cpu_baseline(cfg, indptr, indices, feats, batches_cpu[args.warmup:], args.cpu_budget_s, probs)
         out["cpu_baseline"] = cb
         out["gpu_over_cpu"] = out["value"] / cb["value"]
     print(json.dumps(out), flush=True)

@@ -1,15 +1,15 @@
 // Row-wise weighted neighbour sampling: a float32 weight per edge, stored like `indices`.
 //
 // The count pass is the uniform sampler's (same pick counts).  The fill hands every seed row to a
-// group of G lanes (G = 16, 32 or 64, the smallest that holds num_picks, so a wave64 serves up to
-// four rows); rows of more than 32 G neighbours are queued and then split over the 16 waves of a
-// 1024-thread block, so a hub row costs about as much as sixteen ordinary ones.
+// group of G lanes (G = 16, 32 or 64, so a wave64 serves up to four rows; chosen on the host from
+// num_picks); rows of more than 32 G neighbours are queued and then split over the 16 waves of a
+// 1024-thread block.
 //   without replacement: every position races with the key E / w (E a unit exponential variate
 //     from the row's Philox stream); a group keeps the num_picks smallest (key, position) pairs
 //     in order, lane l holding the l-th;
-//   with replacement: weights become 32.32 fixed-point shares of the row's largest weight, whose
-//     sums are exact in any order; draws in [0, sum) are located against the running inclusive
-//     sum.
+//   with replacement: weights become integer shares floor(w * 2^(32-E)), 2^E the power of two
+//     above the row's largest weight; their sums are exact in any order, and draws in [0, sum)
+//     are located against the running inclusive sum.
 // Both rules are evaluated from exactly rounded operations only (see weights.h), so the picks
 // equal the CPU oracle's bit for bit whatever the launch shape.  Loops that contain cross-lane
 // operations run a wave-uniform number of times: a group that has run out of work keeps
@@ -25,7 +25,7 @@ namespace {
 
 constexpr int kLongBlock = 1024;
 constexpr int kLongWaves = kLongBlock / kWave;
-constexpr int kMaxLongGrid = 2048;
+constexpr int kMaxLongGrid = 512;  // two 1024-thread blocks fit a CU: one round over 256 CUs
 constexpr int kMaxWeightedPicks = 64;      // without replacement: one lane per kept pair
 constexpr uint64_t kNoKey = ~uint64_t(0);  // above every key, +inf included
 constexpr uint32_t kNoPos = 0xffffffffu;
@@ -212,6 +212,11 @@ __device__ __forceinline__ uint64_t lowest_bar(uint64_t* bars, int lane) {
   return v;
 }
 
+__device__ __forceinline__ uint64_t lowest_bar_after_sync(uint64_t* bars, int lane) {
+  __syncthreads();  // every wave of the block has published its final bar
+  return lowest_bar(bars, lane);
+}
+
 // Runs positions [begin, end) of the group's row, in steps of `stride`, through its race.  begin
 // and stride are multiples of 4 G: one Philox block per lane covers 4 G positions (four words
 // each), and the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the group.
@@ -306,8 +311,8 @@ __global__ __launch_bounds__(kTile) void fill_weighted_kernel(const IdT* __restr
   }
 }
 
-// Without replacement, queued long rows: each wave races an interleaved share of the row, wave 0
-// then runs the other waves' winners through its own race.
+// Without replacement, queued long rows: each wave races an interleaved share of the row, then
+// the waves' winners are merged pairwise.
 template <typename IdT>
 __global__ __launch_bounds__(kLongBlock) void fill_weighted_long_kernel(const IdT* __restrict__ seeds, RowArgs a,
                                                                         TierView<IdT> indices,
@@ -332,21 +337,23 @@ __global__ __launch_bounds__(kLongBlock) void fill_weighted_long_kernel(const Id
     Race r;
     race_reset(r);
     race_scan<kWave>(r, g, probs, start, 256u * wave, deg, 256u * kLongWaves, k, rng_seed, rng_stream, row, bars);
-    lds_key[threadIdx.x] = r.key;
-    lds_pos[threadIdx.x] = r.pos;
-    __syncthreads();
-    if (wave == 0) {
-      const uint64_t bar = lowest_bar(bars, g.l);
-      for (int w = 1; w < kLongWaves; ++w) {
-        const uint64_t ck = lds_key[w * kWave + g.l];
-        race_offer<kWave>(r, g, ck > bar ? kNoKey : ck, lds_pos[w * kWave + g.l], k);
+    // pairwise rounds: wave w takes over the entries of wave w + step, 16 lists become one in four
+    // rounds; entries beyond the lowest published bar cannot be among the row's best
+    const uint64_t bar = lowest_bar_after_sync(bars, g.l);
+    for (int step = 1; step < kLongWaves; step <<= 1) {
+      lds_key[threadIdx.x] = r.key;
+      lds_pos[threadIdx.x] = r.pos;
+      __syncthreads();
+      if ((wave & (2 * step - 1)) == 0) {
+        const uint64_t ck = lds_key[(wave + step) * kWave + g.l];
+        race_offer<kWave>(r, g, ck > bar ? kNoKey : ck, lds_pos[(wave + step) * kWave + g.l], k);
       }
-      if (g.l < k && r.pos < deg) {  // deg > k: every entry is filled
-        out_rows[off + g.l] = IdT(row);
-        out_cols[off + g.l] = indices.at(start + r.pos);
-      }
+      __syncthreads();  // the arrays are rewritten by the next round and by the block's next row
     }
-    __syncthreads();  // the arrays are reused by the block's next row
+    if (wave == 0 && g.l < k && r.pos < deg) {  // deg > k: every entry is filled
+      out_rows[off + g.l] = IdT(row);
+      out_cols[off + g.l] = indices.at(start + r.pos);
+    }
   }
 }
 

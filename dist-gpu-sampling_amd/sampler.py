@@ -43,21 +43,26 @@ def create_chunktensor(tensor, num_gpus, available_mem, cache_rate=1.0, root_ran
 
 
 class ChunkTensorSampler:
-    """chunktensor_sampler.py:63-118 (uniform sampling only).
+    """chunktensor_sampler.py:62-118, same positional arguments (the DGL prefetch options of
+    BlockSampler have no counterpart here).
 
     sample_blocks runs the upstream loop -- per hop one sampling call and one relabel call,
-    over reversed(fanouts) -- through the single fused operator when every fanout is at
-    most 64 (`fused=False` forces the per-hop operators; both give identical results).
+    over reversed(fanouts).  Uniform sampling goes through the single fused operator when
+    every fanout is at most 64 (`fused=False` forces the per-hop operators; both give
+    identical results); with `chunk_probs` (a float32 ChunkTensor of edge weights) every hop
+    calls the weighted operator, as upstream does (:97-100).
     """
 
     FUSED_MAX_FANOUT = 64
 
-    def __init__(self, fanouts, chunk_indptr, chunk_indices, replace=False, fused=True):
+    def __init__(self, fanouts, chunk_indptr, chunk_indices, chunk_probs=None, replace=False, fused=True):
         self.chunk_indptr = chunk_indptr
         self.chunk_indices = chunk_indices
+        self.chunk_probs = chunk_probs
         self.fanouts = list(fanouts)
         self.replace = replace
-        self.fused = fused and all(0 <= f <= self.FUSED_MAX_FANOUT for f in self.fanouts)
+        self.fused = (fused and chunk_probs is None
+                      and all(0 <= f <= self.FUSED_MAX_FANOUT for f in self.fanouts))
 
     @staticmethod
     def _blocks(seeds, frontiers, srcs, dsts):
@@ -78,8 +83,12 @@ class ChunkTensorSampler:
         blocks = []
         frontier = seeds
         for fan_out in reversed(self.fanouts):
-            coo_row, coo_col = torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor(
-                seeds, self.chunk_indptr, self.chunk_indices, fan_out, self.replace)
+            if self.chunk_probs is not None:
+                coo_row, coo_col = torch.ops.dgs_ops._CAPI_sample_neighbors_with_probs_with_chunk_tensor(
+                    seeds, self.chunk_indptr, self.chunk_indices, self.chunk_probs, fan_out, self.replace)
+            else:
+                coo_row, coo_col = torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor(
+                    seeds, self.chunk_indptr, self.chunk_indices, fan_out, self.replace)
             frontier, (coo_row, coo_col) = torch.ops.dgs_ops._CAPI_tensor_relabel(
                 [seeds, coo_col], [coo_row, coo_col])
             blocks.insert(0, Block(coo_col, coo_row, frontier.numel(), seeds.numel(), frontier, seeds))

@@ -237,7 +237,7 @@ def unique_relabel(mapping, requiring):
 
 # --------------------------------------------------- multi-layer driver -----
 def sample_blocks(seed_nodes, indptr, indices, fanouts, replace=False, rng_seed=0,
-                  first_stream=0):
+                  first_stream=0, probs=None):
     """ChunkTensorSampler.sample_blocks
     (oppo_bench/single_node/utils/chunktensor_sampler.py:93-118) with the DGL
     block replaced by the tuple (src_local, dst_local, n_src, n_dst, src_ids,
@@ -248,8 +248,12 @@ def sample_blocks(seed_nodes, indptr, indices, fanouts, replace=False, rng_seed=
     blocks = []
     frontier = seeds
     for hop, fan_out in enumerate(reversed(list(fanouts))):
-        coo_row, coo_col = sample_neighbors(seeds, indptr, indices, fan_out, replace, rng_seed,
-                                            first_stream + hop)
+        if probs is not None:  # chunktensor_sampler.py:97-100
+            coo_row, coo_col = sample_neighbors_weighted(seeds, indptr, indices, probs, fan_out,
+                                                         replace, rng_seed, first_stream + hop)
+        else:
+            coo_row, coo_col = sample_neighbors(seeds, indptr, indices, fan_out, replace, rng_seed,
+                                                first_stream + hop)
         frontier, (row_l, col_l) = unique_relabel([seeds, coo_col], [coo_row, coo_col])
         blocks.insert(0, (col_l, row_l, frontier.size, seeds.size, frontier, seeds))
         seeds = frontier

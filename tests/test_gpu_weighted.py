@@ -169,3 +169,25 @@ def test_weighted_inclusion_frequencies(pkg):
         _, c = pkg.ops._CAPI_sample_neighbors_with_probs(seeds, _dev(indptr), _dev(indices), _dev(probs), 1, replace)
         cnt = np.bincount(_np(c), minlength=deg).astype(float)
         assert ((cnt - exp) ** 2 / exp).sum() < 124.8  # chi-square 79 dof, p = 0.001
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_weighted_sampler_loop(pkg, oracle, graph, replace):
+    # ChunkTensorSampler with chunk_probs: the upstream loop with the weighted operator per hop
+    indptr, indices, probs = graph
+    rng = np.random.default_rng(2)
+    seeds = rng.permutation(20000)[:512].astype(np.int64)
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    pr_ct = pkg.create_chunktensor(torch.from_numpy(probs), 1, big)
+    sampler = pkg.ChunkTensorSampler([6, 4, 3], ip_ct, ix_ct, pr_ct, replace)
+    pkg.set_rng_state(31337, 10)
+    frontier, seed_out, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
+    want_frontier, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, [6, 4, 3], replace, 31337, 10,
+                                                         probs=probs)
+    assert np.array_equal(_np(frontier), want_frontier)
+    assert len(blocks) == 3
+    for got, want in zip(blocks, want_blocks):
+        assert np.array_equal(_np(got.src_local), want[0]) and np.array_equal(_np(got.dst_local), want[1])
+        assert (got.num_src, got.num_dst) == (want[2], want[3])
