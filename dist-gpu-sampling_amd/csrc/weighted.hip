@@ -228,32 +228,44 @@ __device__ __forceinline__ void race_scan(Race& r, const Group<G>& g, const Tier
   bool first = true;
   uint64_t published = kNoKey;
   for (uint64_t sb = begin; __ballot(sb < end); sb += stride) {
+    // the four steps of this stretch are independent until they meet the race: their loads are
+    // issued together and their key arithmetic (long dependent float64 chains) interleaves
+    float wt[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
+      wt[c] = p < end ? probs.at(start + int64_t(p)) : 0.0f;
+    }
     PhiloxWords w{{0, 0, 0, 0}};
     if (sb + 4u * uint32_t(g.l) < end)
       w = philox4x32_10(0x80000000u | (uint32_t(sb >> 2) + uint32_t(g.l)), rng_stream, uint32_t(uint64_t(row)),
                         uint32_t(uint64_t(row) >> 32), uint32_t(rng_seed), uint32_t(rng_seed >> 32));
+    uint64_t ck[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const uint64_t cb = sb + uint64_t(G) * c;
-      if (!__ballot(cb < end)) break;
       const int src = (G / 4) * c + (g.l >> 2);
       const uint32_t a0 = __shfl(w.w[0], src, G), a1 = __shfl(w.w[1], src, G);
       const uint32_t a2 = __shfl(w.w[2], src, G), a3 = __shfl(w.w[3], src, G);
       const uint32_t x = (g.l & 2) ? ((g.l & 1) ? a3 : a2) : ((g.l & 1) ? a1 : a0);
-      const uint64_t p = cb + uint32_t(g.l);
-      uint64_t ck = kNoKey;
-      if (p < end) ck = race_key(x, probs.at(start + int64_t(p)), uint32_t(p));
+      const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
+      ck[c] = p < end ? race_key(x, wt[c], uint32_t(p)) : kNoKey;
+    }
+    const uint64_t bar = bars != nullptr ? lowest_bar(bars, g.l) : kNoKey;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint64_t cb = sb + uint64_t(G) * c;
+      if (!__ballot(cb < end)) break;
+      const uint32_t p = uint32_t(cb) + uint32_t(g.l);
       if (first) {
-        race_seed<G>(r, g, ck, uint32_t(p), k);
+        race_seed<G>(r, g, ck[c], p, k);
         first = false;
       } else {
-        if (bars != nullptr && ck > lowest_bar(bars, g.l)) ck = kNoKey;
-        race_offer<G>(r, g, ck, uint32_t(p), k);
+        race_offer<G>(r, g, ck[c] > bar ? kNoKey : ck[c], p, k);
       }
-      if (bars != nullptr && r.last_key < published) {
-        published = r.last_key;
-        if (g.l == 0) __atomic_store_n(&bars[threadIdx.x / kWave], published, __ATOMIC_RELAXED);
-      }
+    }
+    if (bars != nullptr && r.last_key < published) {
+      published = r.last_key;
+      if (g.l == 0) __atomic_store_n(&bars[threadIdx.x / kWave], published, __ATOMIC_RELAXED);
     }
   }
 }
