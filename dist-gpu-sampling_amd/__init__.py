@@ -1,6 +1,7 @@
 """MI355X-native implementation of the per-GPU hot path of Dist-GPU-sampling:
-row-wise uniform neighbour sampling over CSC, first-occurrence unique/relabel and
-the two-tier ChunkTensor row gather.
+row-wise neighbour sampling over CSC (uniform or weighted), first-occurrence
+unique/relabel, the two-tier ChunkTensor row gather, and the hottest-rows-first
+placement that feeds it.
 
 Importing the package loads the two in-tree shared libraries:
   libdgs_hip.so  HIP kernels behind a C ABI (include/dgs_hip.h), bound in `capi`;
@@ -35,8 +36,11 @@ from .sampler import (  # noqa: E402
     set_rng_state,
 )
 
+from . import placement  # noqa: E402
+from . import loading_factor  # noqa: E402
+
 ChunkTensor = torch.classes.dgs_classes.ChunkTensor
 ops = torch.ops.dgs_ops
 
-__all__ = ["capi", "ops", "ChunkTensor", "ChunkTensorSampler", "Block", "create_chunktensor",
+__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "Block", "create_chunktensor",
            "create_dgs_communicator", "get_available_memory", "set_rng_state", "HIP_LIB", "TORCH_LIB"]

@@ -73,6 +73,7 @@ SIGNATURES = {
     "dgs_sample_blocks": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, ctypes.POINTER(c_i64), c_i32, c_i32,
                                          c_u64, c_u32, c_vp, c_u32, c_vp, ctypes.POINTER(BlockOut), c_vp, c_vp,
                                          ctypes.POINTER(c_vp), c_vp, c_sz, c_vp]),
+    "dgs_renumber_csc": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp]),
     "dgs_read_back": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp]),
     "dgs_read_back_begin": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp, ctypes.POINTER(c_vp)]),
     "dgs_read_back_wait": (ctypes.c_int, [c_vp]),
@@ -230,6 +231,15 @@ def sample_neighbors_weighted(seeds, indptr_view, indices_view, probs_view, num_
                                             cols.data_ptr(), nnz.data_ptr(), ws.data_ptr(), nb, stream_ptr()))
     cnt, flags = read_i64(nnz, 2)
     return rows[:cnt], cols[:cnt], flags
+
+
+def renumber_csc(indptr, indices, order, rank, new_indptr):
+    """New edge array of the graph renumbered by order[new] = old / rank[old] = new."""
+    out = torch.empty_like(indices)
+    check(lib.dgs_renumber_csc(indptr.data_ptr(), indptr.element_size(), indices.data_ptr(), indices.element_size(),
+                               order.data_ptr(), rank.data_ptr(), new_indptr.data_ptr(), indptr.numel() - 1,
+                               indices.numel(), out.data_ptr(), stream_ptr()))
+    return out
 
 
 def unique_relabel(mapping, requiring):

@@ -356,6 +356,35 @@ std::tuple<torch::Tensor, torch::Tensor> SampleNeighborsWithProbsWithChunkTensor
   return sample_impl(seeds, indptr->view(), indices->view(), indices->dtype(), num_picks, replace, &pv);
 }
 
+// Not in upstream: the graph renumbered so that new id r is old id order[r] (stable, e.g. by
+// decreasing degree).  Returns (new_indptr, new_indices, rank) with rank[old] = new.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RenumberCSC(torch::Tensor indptr, torch::Tensor indices,
+                                                                    torch::Tensor order) {
+  DGS_CHECK_GPU(indptr);
+  DGS_CHECK_GPU(indices);
+  DGS_CHECK_GPU(order);
+  const int32_t pw = id_width(indptr, "indptr");
+  const int32_t iw = id_width(indices, "indices");
+  TORCH_CHECK(order.scalar_type() == torch::kInt64, "order must be int64, got ", order.scalar_type());
+  TORCH_CHECK(indptr.dim() == 1 && indptr.numel() >= 1, "indptr must be 1-D with n + 1 entries");
+  const int64_t n = indptr.numel() - 1;
+  TORCH_CHECK(order.dim() == 1 && order.numel() == n, "order holds ", order.numel(), " ids for ", n, " rows");
+  torch::Tensor ip = indptr.contiguous();
+  torch::Tensor ix = indices.contiguous().view({-1});
+  torch::Tensor ord = order.contiguous();
+  // rank = inverse permutation; it doubles as the check that order is one
+  torch::Tensor rank = torch::full({n}, -1, ix.options());
+  rank.index_put_({ord}, torch::arange(n, ix.options()));
+  TORCH_CHECK(n == 0 || rank.min().item<int64_t>() >= 0, "order is not a permutation of the row ids");
+  torch::Tensor deg = ip.slice(0, 1) - ip.slice(0, 0, n);
+  torch::Tensor new_ip = torch::zeros({n + 1}, ip.options());
+  if (n > 0) new_ip.slice(0, 1).copy_(deg.index_select(0, ord).cumsum(0));
+  torch::Tensor new_ix = torch::empty_like(ix);
+  check(dgs_renumber_csc(ip.data_ptr(), pw, ix.data_ptr(), iw, ord.data_ptr<int64_t>(), rank.data_ptr(),
+                         new_ip.data_ptr(), n, ix.numel(), new_ix.data_ptr(), current_stream()));
+  return std::make_tuple(new_ip, new_ix, rank);
+}
+
 // Packs up to DGS_MAX_SEGMENTS tensors; more are concatenated first.
 dgs_segments pack_segments(std::vector<torch::Tensor>& tensors, std::vector<torch::Tensor>& keep_alive) {
   dgs_segments s{};
@@ -572,6 +601,8 @@ TORCH_LIBRARY(dgs_ops, m) {
       // not in upstream: the whole sampler loop (and optionally the feature gather) in one call
       .def("_CAPI_sample_blocks", &dgs::SampleBlocks)
       .def("_CAPI_sample_blocks_and_index", &dgs::SampleBlocksAndIndex)
+      // not in upstream: node renumbering (hottest rows first) for the positional stores
+      .def("_CAPI_renumber_csc", &dgs::RenumberCSC)
       // not in upstream: the sampling generator's (seed, stream)
       .def("_CAPI_set_rng_state", &dgs::SetRngState)
       .def("_CAPI_get_rng_state", &dgs::GetRngState);

@@ -350,6 +350,30 @@ dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seed
                              size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
+/* Placement                                                                 */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Rewrites the edge array of a CSC graph for a renumbering of its nodes, so that the
+ * rows a positional store keeps in HBM (the first ones) are the hottest.  No counterpart
+ * in the reference's native code: its stores are positional too (src/chunk_tensor.h:33-42)
+ * and the harness caches "the first rows" (chunktensor_sampler.py:32-60), which only
+ * pays when the caller has ordered the nodes beforehand.
+ *   order      : device int64[n_rows], order[new] = old
+ *   rank       : device ids (id_bytes wide)[n_rows], rank[old] = new
+ *   new_indptr : device offsets (ptr_bytes wide)[n_rows + 1], the exclusive scan of the
+ *                old degrees taken in the new order
+ *   new_indices: device ids[n_edges]; new row r receives the edges of old row order[r]
+ *                in their old order, endpoints renamed through rank
+ * All arrays are plain device memory (a renumbering is done before the stores are filled).
+ */
+dgs_status dgs_renumber_csc(const void* old_indptr, int32_t ptr_bytes,
+                            const void* old_indices, int32_t id_bytes,
+                            const int64_t* order, const void* rank,
+                            const void* new_indptr, int64_t n_rows, int64_t n_edges,
+                            void* new_indices, void* stream);
+
+/* ------------------------------------------------------------------------ */
 /* Small utilities                                                           */
 /* ------------------------------------------------------------------------ */
 

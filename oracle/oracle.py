@@ -258,3 +258,30 @@ def sample_blocks(seed_nodes, indptr, indices, fanouts, replace=False, rng_seed=
         blocks.insert(0, (col_l, row_l, frontier.size, seeds.size, frontier, seeds))
         seeds = frontier
     return frontier, _ids(seed_nodes), blocks
+
+
+# ------------------------------------------------------------ placement -----
+def degree_order(indptr):
+    """order[new] = old by decreasing in-degree, ties by increasing old id."""
+    deg = np.diff(_ids(indptr))
+    return np.argsort(-deg, kind="stable").astype(np.int64)
+
+
+def renumber_csc(indptr, indices, order):
+    """The graph with node order[r] renamed r, row by row (plain Python loop over rows:
+    the definition itself).  Returns (new_indptr, new_indices, rank), rank[old] = new."""
+    indptr, indices = _ids(indptr), _ids(indices)
+    order = np.asarray(order, dtype=np.int64)
+    n = order.size
+    rank = np.empty(n, dtype=indices.dtype)
+    rank[order] = np.arange(n, dtype=indices.dtype)
+    new_indptr = np.zeros(n + 1, dtype=indptr.dtype)
+    new_indices = np.empty_like(indices)
+    at = 0
+    for r in range(n):
+        o = order[r]
+        seg = indices[indptr[o]:indptr[o + 1]]
+        new_indices[at:at + seg.size] = rank[seg]
+        at += seg.size
+        new_indptr[r + 1] = at
+    return new_indptr, new_indices, rank

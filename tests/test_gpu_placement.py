@@ -1,0 +1,108 @@
+"""Hottest-rows-first placement: the renumbering kernel against its row-by-row definition, and
+what the placement is for: a sampled-and-gathered batch is the same batch under new names."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import load_pkg, powerlaw_graph
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    return load_pkg()
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _np(t):
+    return t.cpu().numpy()
+
+
+@pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int64, np.int64), (np.int32, np.int64), (np.int32, np.int32),
+                                                (np.int64, np.int32)])
+def test_renumber_parity(pkg, oracle, id_dtype, ptr_dtype):
+    rng = np.random.default_rng(5)
+    indptr, indices = powerlaw_graph(rng, 30000, 12, 9000, zero_frac=0.1, id_dtype=id_dtype, ptr_dtype=ptr_dtype)
+    order = pkg.placement.degree_order(_dev(indptr))
+    want_order = oracle.degree_order(indptr)
+    assert np.array_equal(_np(order), want_order)
+    want_ip, want_ix, want_rank = oracle.renumber_csc(indptr, indices, want_order)
+    new_ip, new_ix, rank = pkg.placement.renumber_csc(_dev(indptr), _dev(indices), order)
+    assert new_ip.dtype == _dev(indptr).dtype and new_ix.dtype == _dev(indices).dtype
+    assert np.array_equal(_np(new_ip), want_ip) and np.array_equal(_np(new_ix), want_ix)
+    assert np.array_equal(_np(rank), want_rank)
+    # an arbitrary permutation (empty rows in the middle of the new order), through the C ABI
+    perm = rng.permutation(30000).astype(np.int64)
+    want_ip, want_ix, want_rank = oracle.renumber_csc(indptr, indices, perm)
+    got = pkg.capi.renumber_csc(_dev(indptr), _dev(indices), _dev(perm), _dev(want_rank), _dev(want_ip))
+    assert np.array_equal(_np(got), want_ix)
+
+
+def test_renumber_edge_cases(pkg):
+    ops = pkg.ops
+    empty_ip = torch.zeros(1, dtype=torch.int64, device="cuda")
+    ip, ix, rank = ops._CAPI_renumber_csc(empty_ip, empty_ip[:0], empty_ip[:0])
+    assert ip.tolist() == [0] and ix.numel() == 0 and rank.numel() == 0
+    ip = _dev(np.array([0, 0, 3, 3], dtype=np.int64))          # one row holds every edge
+    ix = _dev(np.array([2, 0, 1], dtype=np.int64))
+    new_ip, new_ix, rank = ops._CAPI_renumber_csc(ip, ix, _dev(np.array([1, 0, 2], dtype=np.int64)))
+    assert new_ip.tolist() == [0, 3, 3, 3] and new_ix.tolist() == [2, 1, 0] and rank.tolist() == [1, 0, 2]
+    with pytest.raises(RuntimeError, match="permutation"):
+        ops._CAPI_renumber_csc(ip, ix, _dev(np.array([1, 1, 2], dtype=np.int64)))
+    with pytest.raises(RuntimeError, match="rows"):
+        ops._CAPI_renumber_csc(ip, ix, _dev(np.array([1, 0], dtype=np.int64)))
+
+
+def test_placed_batch_is_the_same_batch(pkg):
+    # full-fanout sampling is deterministic, so the batch sampled on the renumbered graph from the
+    # renamed seeds, with the features permuted alike, must be the original batch under new names
+    rng = np.random.default_rng(9)
+    n = 20000
+    indptr, indices = powerlaw_graph(rng, n, 6, 40)
+    feats = rng.standard_normal((n, 24)).astype(np.float32)
+    pl = pkg.placement
+    order = pl.degree_order(_dev(indptr))
+    new_ip, new_ix, rank = pl.renumber_csc(_dev(indptr), _dev(indices), order)
+    new_feats = pl.permute_rows(torch.from_numpy(feats), order.cpu())
+    hot_rows = n // 4
+    cap = pl.capacity_for_rows(new_feats, rows=hot_rows)
+    assert pl.rows_in_hbm(new_feats, new_feats.dtype, cap) == hot_rows
+    big = 1 << 40
+    fanouts = [40, 40]
+    seeds = rng.permutation(n)[:300].astype(np.int64)
+
+    def batch(ip, ix, x, capacity, s):
+        ct_ip = pkg.create_chunktensor(ip.cpu(), 1, big)
+        ct_ix = pkg.create_chunktensor(ix.cpu(), 1, big)
+        ct_x = pkg.ChunkTensor(list(x.shape), x.dtype, capacity)
+        ct_x._CAPI_load_from_tensor(x)
+        sampler = pkg.ChunkTensorSampler(fanouts, ct_ip, ct_ix)
+        return sampler.sample_blocks_and_index(None, torch.from_numpy(s), ct_x)
+
+    f0, _, b0, x0 = batch(_dev(indptr), _dev(indices), torch.from_numpy(feats), big, seeds)
+    f1, _, b1, x1 = batch(new_ip, new_ix, new_feats, cap, _np(rank)[seeds])
+    assert np.array_equal(_np(order)[_np(f1)], _np(f0))          # same nodes, same order
+    assert np.array_equal(_np(x1), _np(x0))                      # same feature rows, from both tiers
+    for a, b in zip(b0, b1):
+        assert np.array_equal(_np(a.src_local), _np(b.src_local)) and np.array_equal(_np(a.dst_local), _np(b.dst_local))
+    # the hot prefix really is hot: a quarter of the rows draws well over a quarter of the picks
+    deg_new = (new_ip[1:] - new_ip[:-1])
+    assert pl.expected_hit_rate(deg_new, hot_rows) > 0.5
+
+
+def test_loading_factor_runs(pkg):
+    n, d = 2_000_000, 32
+    lines = []
+    for option, cap in (("local", n * d * 4), ("host", 0)):
+        ct = pkg.ChunkTensor([n, d], torch.float32, cap)
+        for part in (ct._CAPI_get_sub_device_tensor(), ct._CAPI_get_host_tensor()):
+            if part.numel():
+                part.fill_(1.0)
+        f = pkg.loading_factor.compute_loading_factor(ct, n, d, 4, option, 8000.0 if option == "local" else 64.0,
+                                                      valid_time_threshold_ms=0.02, valid_needed=2, log=lines.append)
+        assert f > 0.5 and np.isfinite(f)   # nothing moves faster than the stated bandwidth allows (with slack)
+    assert len(lines) == 4

@@ -439,3 +439,26 @@ def test_bounded64_rejection_rule(oracle):
     for _ in range(7000):
         cnt[oracle.bounded64([int(x) for x in rng.integers(0, 2 ** 32, 4)], 7)] += 1
     assert ((cnt - 1000) ** 2 / 1000).sum() < 22.46  # chi-square 6 dof, p = 0.001
+
+
+# ---- placement ------------------------------------------------------------
+def test_renumber_is_an_isomorphism(oracle):
+    rng = np.random.default_rng(12)
+    deg = rng.integers(0, 12, size=200)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, 200, size=int(indptr[-1])).astype(np.int64)
+    order = oracle.degree_order(indptr)
+    new_deg = deg[order]
+    assert (new_deg[:-1] >= new_deg[1:]).all()                       # hottest first
+    same = new_deg[:-1] == new_deg[1:]
+    assert (order[:-1][same] < order[1:][same]).all()                # ties keep the old order
+    new_indptr, new_indices, rank = oracle.renumber_csc(indptr, indices, order)
+    assert np.array_equal(rank[order], np.arange(200)) and np.array_equal(np.diff(new_indptr), new_deg)
+    # edge (u -> v) exists, at the same place in v's list, iff (rank[u] -> rank[v]) does
+    for v in range(200):
+        r = rank[v]
+        assert np.array_equal(order[new_indices[new_indptr[r]:new_indptr[r + 1]]],
+                              indices[indptr[v]:indptr[v + 1]])
+    # renumbering back with the inverse permutation restores the graph
+    back_indptr, back_indices, _ = oracle.renumber_csc(new_indptr, new_indices, rank.astype(np.int64))
+    assert np.array_equal(back_indptr, indptr) and np.array_equal(back_indices, indices)
