@@ -48,6 +48,21 @@ def main():
         out[f"block{i}_src"] = b[0]
         out[f"block{i}_dst"] = b[1]
     np.savez_compressed(os.path.join(HERE, "sample_small.npz"), **out)
+    # weighted sampling on the same graph: weights over many binades with zeros, a negative, ties
+    w = (rng.random(indices.size) ** 5 * 50.0).astype(np.float32)
+    w[rng.random(indices.size) < 0.08] = 0.0
+    w[rng.random(indices.size) < 0.15] = np.float32(0.25)
+    w[3] = -1.0
+    wout = {"probs": w}
+    for k, replace in [(5, False), (20, False), (64, False), (6, True), (80, True)]:
+        r, c = oracle.sample_neighbors_weighted(seeds, indptr, indices, w, k, replace, 0x5EED1234ABCD, 23)
+        tag = f"k{k}_{'rep' if replace else 'norep'}"
+        wout[f"rows_{tag}"] = r
+        wout[f"cols_{tag}"] = c
+    xs = np.array([0, 1, 2, 1000, 2 ** 31 - 1, 2 ** 31, 3037000499, 3037000500, 2 ** 32 - 2, 2 ** 32 - 1], dtype=np.uint64)
+    wout["neg_log_x"] = xs
+    wout["neg_log_bits"] = np.array([np.float64(oracle.neg_log_u32(int(x))).view(np.uint64) for x in xs], dtype=np.uint64)
+    np.savez_compressed(os.path.join(HERE, "weighted_small.npz"), **wout)
     draws = [[s, st, row, j, nn, oracle.draw(s, st, row, j, nn)]
              for s, st, row, j, nn in [(0, 0, 0, 0, 10), (1, 2, 3, 4, 5), (2 ** 63 + 5, 7, 2 ** 40 + 3, 63, 1000003),
                                        (7777, 0, 2449028, 14, 17000), (42, 4294967295, 1, 0, 4294967295)]]

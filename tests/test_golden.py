@@ -71,6 +71,39 @@ def test_kernels_reproduce_samples(gold):
         assert np.array_equal(b.dst_local.cpu().numpy(), gold[f"block{i}_dst"])
 
 
+WEIGHTED_CASES = [(5, False), (20, False), (64, False), (6, True), (80, True)]
+
+
+def test_oracle_reproduces_weighted_samples(oracle, gold):
+    wg = np.load(os.path.join(GOLD, "weighted_small.npz"))
+    seed = int(gold["rng_seed"][0])
+    for x, bits in zip(wg["neg_log_x"], wg["neg_log_bits"]):
+        assert np.float64(oracle.neg_log_u32(int(x))).view(np.uint64) == bits
+    for k, replace in WEIGHTED_CASES:
+        tag = f"k{k}_{'rep' if replace else 'norep'}"
+        r, c = oracle.sample_neighbors_weighted(gold["seeds"], gold["indptr"], gold["indices"], wg["probs"], k,
+                                                replace, seed, 23)
+        assert np.array_equal(r, wg[f"rows_{tag}"]) and np.array_equal(c, wg[f"cols_{tag}"])
+
+
+@pytest.mark.gpu
+def test_kernels_reproduce_weighted_samples(gold):
+    import torch
+    pkg = load_pkg()
+    capi = pkg.capi
+    wg = np.load(os.path.join(GOLD, "weighted_small.npz"))
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    seed = int(gold["rng_seed"][0])
+    ip, ix, pr, seeds = dev(gold["indptr"]), dev(gold["indices"]), dev(wg["probs"]), dev(gold["seeds"])
+    for k, replace in WEIGHTED_CASES:
+        tag = f"k{k}_{'rep' if replace else 'norep'}"
+        r, c, flags = capi.sample_neighbors_weighted(seeds, capi.tensor_view(ip), capi.tensor_view(ix),
+                                                     capi.tensor_view(pr), k, replace, seed, 23)
+        assert flags == 0
+        assert np.array_equal(r.cpu().numpy(), wg[f"rows_{tag}"])
+        assert np.array_equal(c.cpu().numpy(), wg[f"cols_{tag}"])
+
+
 @pytest.mark.gpu
 def test_kernels_reproduce_readme_demo():
     import torch
