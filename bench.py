@@ -194,6 +194,33 @@ def store_from_device(dgs, t, capacity_bytes):
     return ct
 
 
+def run_batches(sampler, seed_batches, features, inflight, consume=lambda r: None):
+    """The timed loop: every batch is submitted on one of `inflight` streams in turn and collected
+    once `inflight` batches are queued, so that many batches share the GPU at any time.
+    `consume` turns each result into what the caller keeps (the big buffers are dropped at once so
+    the allocator can hand them to the next batch).  The caller brackets the call with
+    synchronisations."""
+    if inflight <= 1 or not sampler.fused:
+        return [consume(sampler.sample_blocks_and_index(None, b, features)) for b in seed_batches]
+    if len(getattr(run_batches, "streams", [])) != inflight:
+        run_batches.streams = [torch.cuda.Stream() for _ in range(inflight)]
+    streams = run_batches.streams
+    start = torch.cuda.current_stream()
+    for st in streams:
+        st.wait_stream(start)
+    out, queue = [], []
+    for i, b in enumerate(seed_batches):
+        with torch.cuda.stream(streams[i % inflight]):
+            queue.append(sampler.submit(None, b, features))
+        if len(queue) >= inflight:
+            out.append(consume(queue.pop(0).result()))
+    while queue:
+        out.append(consume(queue.pop(0).result()))
+    for st in streams:
+        start.wait_stream(st)
+    return out
+
+
 def time_call(fn, reps):
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(reps)]
     fn()
@@ -293,21 +320,23 @@ def run_large(args, dgs):
         r = torch.randint(0, n if pool is None else pool.numel(), (batch,), generator=gen, device="cuda")
         seeds.append(r.to(torch.int32) if pool is None else pool[r])
     dgs.set_rng_state(cfg["seed"], 0)
-    for i in range(args.warmup):
-        sampler.sample_blocks_and_index(None, seeds[i], ct_x)
+    # the two-tier case gathers tens of GB per batch: one batch at a time
+    inflight = args.inflight if cfg["hbm_rows"] >= 1.0 else 1
+    run_batches(sampler, seeds[:args.warmup], ct_x, inflight)
     torch.cuda.synchronize()
     edges = rows = 0
     frontiers = []
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        frontier, _, blocks, x = sampler.sample_blocks_and_index(None, seeds[args.warmup + i], ct_x)
-        edges += sum(b.src_local.numel() for b in blocks)
+    results = run_batches(sampler, seeds[args.warmup:], ct_x, inflight,
+                          lambda r: (r[0], sum(b.src_local.numel() for b in r[2])))
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for frontier, n_edges in results:
+        edges += n_edges
         rows += frontier.numel()
         if len(frontiers) < 8:
             frontiers.append(frontier)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    del x
+    del results
     row_bytes = dim * eb
     # the gather alone, once per kept frontier (a repeat of the same rows would be served by the
     # 256 MB last-level cache), events on the launching stream, queued back to back
@@ -331,7 +360,8 @@ def run_large(args, dgs):
         "config": {"workload": f"{args.workload}: {cfg['graph']} graph, {n} nodes / {e} edges CSC int64+int32, "
                                f"features {str(cfg['feat_dtype']).split('.')[-1]} x{dim} ({n * row_bytes / 1e9:.1f} GB), "
                                f"{int(100 * cfg['hbm_rows'])}% of rows in HBM, batch {batch}, fanouts {fanouts}, "
-                               f"{'with' if cfg['replace'] else 'without'} replacement", "scale": scale},
+                               f"{'with' if cfg['replace'] else 'without'} replacement", "scale": scale,
+                   "batches_in_flight": inflight},
         "avg_frontier_rows": rows / args.steps, "avg_edges_per_batch": edges / args.steps,
         "gather_ms": 1e3 * t_mixed, "gather_GBps": gather_gbps, "graph_gen_s": t_gen,
     }
@@ -365,6 +395,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + sorted(LARGE))
     ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
+    ap.add_argument("--inflight", type=int, default=2,
+                    help="batches in flight on as many streams (1 = one blocking call per batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
@@ -402,13 +434,8 @@ def main():
     feat_bytes = feats.element_size()
     dgs.set_rng_state(20240602, 0)
 
-    def step(seeds):
-        # sampler loop + feature gather, one blocking length read at the very end
-        frontier, _, blocks, x = sampler.sample_blocks_and_index(None, seeds, ct_feats)
-        return frontier, blocks, x
-
-    for i in range(args.warmup):
-        step(batches[i])
+    inflight = args.inflight if sampler.fused else 1
+    run_batches(sampler, batches[:args.warmup], ct_feats, inflight)
     torch.cuda.synchronize()
     if args.calibrate_copy_mib > 0:
         src = torch.empty(args.calibrate_copy_mib << 18, dtype=torch.float32, device="cuda").normal_()
@@ -417,17 +444,26 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    stats = []
-    frontiers = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        frontier, blocks, x = step(batches[args.warmup + i])
-        stats.append({"frontier": frontier.numel(),
-                      "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(blocks)]})
-        frontiers.append(frontier)
+    def keep(r):  # sizes, the frontier ids (for the gather leg below) and the destination ids of the widest hop
+        return ({"frontier": r[0].numel(),
+                 "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]}, r[0], r[2][0].dst_ids)
+
+    results = run_batches(sampler, batches[args.warmup:], ct_feats, inflight, keep)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    stats = [r[0] for r in results]
+    frontiers = [r[1] for r in results]
+    widest_hop_seeds = results[-1][2]
+    del results
+    # one batch at a time on one stream: what a single batch takes from call to result
+    dgs.set_rng_state(20240602, 0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_batches(sampler, batches[args.warmup:], ct_feats, 1)
+    torch.cuda.synchronize()
+    ms_latency = 1e3 * (time.perf_counter() - t0) / args.steps
 
     # Stage split and the dominant kernel's duration, on the same batches: events on torch's
     # current stream (the one the C ABI launches on) around the sampler call and around the
@@ -478,7 +514,8 @@ def main():
                                f"features {cfg['feat_dtype']} x{cfg['feat_dim']}, all in HBM, batch {cfg['batch']} "
                                f"uniform seeds, fanouts {cfg['fanouts']} without replacement"
                                f"{', weighted by a float32 weight per edge' if cfg.get('weighted') else ''}, then gather",
-                   "fanouts": cfg["fanouts"], "batch": cfg["batch"]},
+                   "fanouts": cfg["fanouts"], "batch": cfg["batch"], "batches_in_flight": inflight},
+        "ms_per_batch_alone": ms_latency,
         "sample_edges_per_s": edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
         "ms_sample_relabel": ms_sample,
@@ -497,7 +534,7 @@ def main():
     if cfg.get("weighted"):
         # the weighted fill of the widest hop alone: its input is every weight of every sampled row
         ops = torch.ops.dgs_ops
-        seeds = blocks[0].dst_ids
+        seeds = widest_hop_seeds
         k = cfg["fanouts"][0]
         ip_dev = ct_indptr._CAPI_get_sub_device_tensor()
         degs = ip_dev[seeds + 1] - ip_dev[seeds]

@@ -23,6 +23,7 @@
 #include <torch/script.h>
 
 #include <atomic>
+#include <map>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -197,17 +198,25 @@ class ChunkTensor : public torch::CustomClassHolder {
 
   // Persistent direct-address table for sample_blocks when this store is a graph's indptr
   // (one entry per node).  Created on first use; returns (pointer, epoch for this call).
-  std::pair<void*, uint32_t> node_table() {
+  // Calls in flight on different streams must not share a table, so there is one per stream
+  // (up to kMaxNodeTables; further streams get none and the call uses a hash table instead).
+  std::pair<void*, uint32_t> node_table(void* stream) {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
     if (bytes == 0 || bytes > (size_t(8) << 30)) return {nullptr, 0u};
     std::lock_guard<std::mutex> lock(node_table_mutex_);
-    if (!node_table_.defined() || node_epoch_ >= 0xffffff00u) {
-      node_table_ = torch::full({static_cast<int64_t>(bytes / 8)}, int64_t(-1),
-                                torch::TensorOptions().dtype(torch::kInt64).device(device_));
-      node_epoch_ = 0;
+    auto it = node_tables_.find(stream);
+    if (it == node_tables_.end()) {
+      if (node_tables_.size() >= kMaxNodeTables) return {nullptr, 0u};
+      it = node_tables_.emplace(stream, NodeTable{}).first;
     }
-    return {node_table_.data_ptr(), ++node_epoch_};
+    NodeTable& t = it->second;
+    if (!t.entries.defined() || t.epoch >= 0xffffff00u) {
+      t.entries = torch::full({static_cast<int64_t>(bytes / 8)}, int64_t(-1),
+                              torch::TensorOptions().dtype(torch::kInt64).device(device_));
+      t.epoch = 0;
+    }
+    return {t.entries.data_ptr(), ++t.epoch};
   }
 
   const dgs_view& view() const { return view_; }
@@ -224,8 +233,12 @@ class ChunkTensor : public torch::CustomClassHolder {
   dgs_store* store_ = nullptr;
   dgs_view view_{};
   c10::Device device_{c10::DeviceType::CUDA, 0};
-  torch::Tensor node_table_;
-  uint32_t node_epoch_ = 0;
+  struct NodeTable {
+    torch::Tensor entries;
+    uint32_t epoch = 0;
+  };
+  static constexpr size_t kMaxNodeTables = 4;
+  std::map<void*, NodeTable> node_tables_;
   std::mutex node_table_mutex_;
 };
 
@@ -456,82 +469,115 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> TensorRelabel(std::vector<
   return std::make_tuple(unique.narrow(0, 0, u), relabelled.split_with_sizes(sizes, 0));
 }
 
-// All hops of the sampler loop (chunktensor_sampler.py:93-118) in one call with a single
-// blocking wait for the lengths.  `fanouts` is in hop order (the reversed model fanouts).
-// Returns per hop, nearest the seeds first: frontier (= the hop's source ids, seeds first;
-// all views of one array), src_local, dst_local -- and, when `features` is given, the
-// gathered feature rows of the last frontier, enqueued before the lengths are known.
-//
-// Seeds may also arrive on the host, as the upstream sampler receives them
-// (chunktensor_sampler.py:94); they are uploaded on the caller's stream.  (Running the
-// sampling half on a second stream so that it overlaps the previous call's gather was
-// measured and dropped: the cross-stream waits cost more than the overlap saved.)
-std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor,
-           torch::Tensor>
-sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<ChunkTensor>& indptr,
-                   const c10::intrusive_ptr<ChunkTensor>& indices, const std::vector<int64_t>& fanouts,
-                   bool replace, const c10::intrusive_ptr<ChunkTensor>& features) {
-  const int32_t w = id_width(seeds_in, "seeds");
-  TORCH_CHECK(seeds_in.scalar_type() == indices->dtype(), "seeds (", seeds_in.scalar_type(), ") and indices (",
-              indices->dtype(), ") must have the same dtype");
-  TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
-              "indptr store must be int32 or int64");
-  const int32_t hops = static_cast<int32_t>(fanouts.size());
-  TORCH_CHECK(hops >= 1 && hops <= DGS_MAX_HOPS, "sample_blocks: between 1 and ", DGS_MAX_HOPS, " fanouts");
-  const int64_t n = seeds_in.numel();
-  std::vector<int64_t> seeds_max(hops + 1), edges_max(hops);
-  check(dgs_sample_blocks_plan(n, fanouts.data(), hops, seeds_max.data(), edges_max.data()));
-  const int n_sizes = 3 * hops + 1;
-  TORCH_CHECK(n_sizes <= 32);
+using BlocksResult = std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::vector<torch::Tensor>,
+                                torch::Tensor, torch::Tensor>;
 
-  const c10::Device dev = indptr->device();
-  TORCH_CHECK(seeds_in.device().is_cpu() || seeds_in.device() == dev, "seeds must be on the host or on ", dev);
-  void* st = current_stream();
+}  // namespace
 
-  thread_local torch::Tensor pinned =
-      torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-  int64_t* sizes_host = pinned.data_ptr<int64_t>();
+// A sample_blocks call whose kernels are enqueued but whose lengths have not been read yet.
+// Finish() waits for the lengths (not for the relabel of the last hop or the gather, which stay
+// queued on the call's stream) and cuts the worst-case buffers to size.  Holding several of these
+// on different streams keeps one batch's gather and the next batch's sampling on the GPU together.
+class PendingBlocks : public torch::CustomClassHolder {
+ public:
+  PendingBlocks() = default;
+  ~PendingBlocks() override {
+    if (ticket_ != nullptr) dgs_ticket_wait(ticket_);  // never leave a ticket behind
+  }
 
-  torch::Tensor seeds = seeds_in.to(dev, /*non_blocking=*/true).contiguous().view({-1});
-  const auto opt = seeds.options();
-  std::vector<torch::Tensor> frontier(hops), src(hops), dst(hops);
-  std::vector<dgs_block_out> outs(hops);
-  torch::Tensor all = torch::empty({seeds_max[hops]}, opt);  // every hop's frontier is a prefix of it
-  for (int h = 0; h < hops; ++h) {
-    src[h] = torch::empty({edges_max[h]}, opt);
-    dst[h] = torch::empty({edges_max[h]}, opt);
-    outs[h] = dgs_block_out{src[h].data_ptr(), dst[h].data_ptr()};
+  BlocksResult Finish() {
+    TORCH_CHECK(ticket_ != nullptr, "PendingBlocks: already finished");
+    void* t = ticket_;
+    ticket_ = nullptr;
+    const dgs_status ws_status = dgs_ticket_wait(t);
+    check(gather_status_);
+    check(ws_status);
+    const int64_t* sizes_host = pinned_.data_ptr<int64_t>();
+    const int n_sizes = 3 * hops_ + 1;
+    const std::vector<int64_t> sz(sizes_host, sizes_host + n_sizes);
+    std::vector<torch::Tensor> frontier(hops_);
+    for (int h = 0; h < hops_; ++h) {
+      TORCH_CHECK(sz[2 * hops_ + 1 + h] == 0, "sample_blocks: a seed row of hop ", h,
+                  " has a degree of 2^32 or more");
+      frontier[h] = all_.narrow(0, 0, sz[h + 1]);
+      src_[h] = src_[h].narrow(0, 0, sz[hops_ + 1 + h]);
+      dst_[h] = dst_[h].narrow(0, 0, sz[hops_ + 1 + h]);
+    }
+    if (x_.defined()) x_ = x_.narrow(0, 0, sz[hops_]);
+    return std::make_tuple(frontier, src_, dst_, x_.defined() ? x_ : torch::empty({0}, seeds_.options()), seeds_);
   }
-  torch::Tensor sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
-  const size_t ws_bytes = dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
-  torch::Tensor ws = device_bytes(ws_bytes, dev);
-  const auto rng = next_rng(static_cast<uint32_t>(hops));
-  const auto table = indptr->node_table();
-  void* ticket = nullptr;
-  check(dgs_sample_blocks(seeds.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops, replace,
-                          rng.first, rng.second, table.first, table.second, all.data_ptr(), outs.data(),
-                          sizes_dev.data_ptr<int64_t>(), sizes_host, &ticket, ws.data_ptr(), ws_bytes, st));
-  // the lengths are final at the ticket; the gather is enqueued before the host waits for them
-  torch::Tensor x;
-  dgs_status gs = DGS_OK;
-  if (features) {
-    x = torch::empty({seeds_max[hops], features->elem_stride()},
-                     torch::TensorOptions().dtype(features->dtype()).device(dev));
-    gs = dgs_gather_rows_dyn(features->view(), features->elem_stride(), all.data_ptr(), w, seeds_max[hops],
-                             sizes_dev.data_ptr<int64_t>() + hops, x.data_ptr(), DGS_TIER_ANY, st);
+
+  static c10::intrusive_ptr<PendingBlocks> Begin(const torch::Tensor& seeds_in,
+                                                 const c10::intrusive_ptr<ChunkTensor>& indptr,
+                                                 const c10::intrusive_ptr<ChunkTensor>& indices,
+                                                 const std::vector<int64_t>& fanouts, bool replace,
+                                                 const c10::intrusive_ptr<ChunkTensor>& features) {
+    const int32_t w = id_width(seeds_in, "seeds");
+    TORCH_CHECK(seeds_in.scalar_type() == indices->dtype(), "seeds (", seeds_in.scalar_type(), ") and indices (",
+                indices->dtype(), ") must have the same dtype");
+    TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
+                "indptr store must be int32 or int64");
+    const int32_t hops = static_cast<int32_t>(fanouts.size());
+    TORCH_CHECK(hops >= 1 && hops <= DGS_MAX_HOPS, "sample_blocks: between 1 and ", DGS_MAX_HOPS, " fanouts");
+    const int64_t n = seeds_in.numel();
+    std::vector<int64_t> seeds_max(hops + 1), edges_max(hops);
+    check(dgs_sample_blocks_plan(n, fanouts.data(), hops, seeds_max.data(), edges_max.data()));
+    const int n_sizes = 3 * hops + 1;
+    TORCH_CHECK(n_sizes <= 32);
+
+    const c10::Device dev = indptr->device();
+    TORCH_CHECK(seeds_in.device().is_cpu() || seeds_in.device() == dev, "seeds must be on the host or on ", dev);
+    void* st = current_stream();
+
+    auto p = c10::make_intrusive<PendingBlocks>();
+    p->hops_ = hops;
+    // the kernels mirror the lengths into this call's own pinned words
+    p->pinned_ = torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    p->seeds_ = seeds_in.to(dev, /*non_blocking=*/true).contiguous().view({-1});
+    const auto opt = p->seeds_.options();
+    p->src_.resize(hops);
+    p->dst_.resize(hops);
+    std::vector<dgs_block_out> outs(hops);
+    p->all_ = torch::empty({seeds_max[hops]}, opt);  // every hop's frontier is a prefix of it
+    for (int h = 0; h < hops; ++h) {
+      p->src_[h] = torch::empty({edges_max[h]}, opt);
+      p->dst_[h] = torch::empty({edges_max[h]}, opt);
+      outs[h] = dgs_block_out{p->src_[h].data_ptr(), p->dst_[h].data_ptr()};
+    }
+    torch::Tensor sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
+    const size_t ws_bytes = dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
+    torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
+    const auto rng = next_rng(static_cast<uint32_t>(hops));
+    const auto table = indptr->node_table(st);
+    check(dgs_sample_blocks(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops,
+                            replace, rng.first, rng.second, table.first, table.second, p->all_.data_ptr(),
+                            outs.data(), sizes_dev.data_ptr<int64_t>(), p->pinned_.data_ptr<int64_t>(), &p->ticket_,
+                            ws.data_ptr(), ws_bytes, st));
+    // the lengths are final at the ticket; the gather is enqueued before anybody waits for them
+    if (features) {
+      p->x_ = torch::empty({seeds_max[hops], features->elem_stride()},
+                           torch::TensorOptions().dtype(features->dtype()).device(dev));
+      p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
+                                              seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops,
+                                              p->x_.data_ptr(), DGS_TIER_ANY, st);
+    }
+    return p;
   }
-  const dgs_status ws_status = dgs_ticket_wait(ticket);  // never leave a ticket behind
-  check(gs);
-  check(ws_status);
-  const std::vector<int64_t> sz(sizes_host, sizes_host + n_sizes);
-  for (int h = 0; h < hops; ++h) {
-    TORCH_CHECK(sz[2 * hops + 1 + h] == 0, "sample_blocks: a seed row of hop ", h, " has a degree of 2^32 or more");
-    frontier[h] = all.narrow(0, 0, sz[h + 1]);
-    src[h] = src[h].narrow(0, 0, sz[hops + 1 + h]);
-    dst[h] = dst[h].narrow(0, 0, sz[hops + 1 + h]);
-  }
-  if (features) x = x.narrow(0, 0, sz[hops]);
-  return std::make_tuple(frontier, src, dst, x, seeds);
+
+ private:
+  int hops_ = 0;
+  void* ticket_ = nullptr;
+  dgs_status gather_status_ = DGS_OK;
+  torch::Tensor pinned_, seeds_, all_, x_;
+  std::vector<torch::Tensor> src_, dst_;
+};
+
+namespace {
+
+BlocksResult sample_blocks_impl(const torch::Tensor& seeds_in, const c10::intrusive_ptr<ChunkTensor>& indptr,
+                                const c10::intrusive_ptr<ChunkTensor>& indices, const std::vector<int64_t>& fanouts,
+                                bool replace, const c10::intrusive_ptr<ChunkTensor>& features) {
+  return PendingBlocks::Begin(seeds_in, indptr, indices, fanouts, replace, features)->Finish();
 }
 
 // Both operators also return the seeds as a device tensor (the upload they did anyway).
@@ -549,6 +595,22 @@ SampleBlocksAndIndex(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr
                      c10::intrusive_ptr<ChunkTensor> features) {
   TORCH_CHECK(features, "sample_blocks_and_index: features store is null");
   return sample_blocks_impl(seeds, indptr, indices, fanouts, replace, features);
+}
+
+// The same two operators in two halves: *_begin enqueues everything on the current stream and
+// returns at once, PendingBlocks._CAPI_finish waits for the lengths and returns the results.
+c10::intrusive_ptr<PendingBlocks> SampleBlocksBegin(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr,
+                                                    c10::intrusive_ptr<ChunkTensor> indices,
+                                                    std::vector<int64_t> fanouts, bool replace) {
+  return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace, c10::intrusive_ptr<ChunkTensor>());
+}
+c10::intrusive_ptr<PendingBlocks> SampleBlocksAndIndexBegin(torch::Tensor seeds,
+                                                            c10::intrusive_ptr<ChunkTensor> indptr,
+                                                            c10::intrusive_ptr<ChunkTensor> indices,
+                                                            std::vector<int64_t> fanouts, bool replace,
+                                                            c10::intrusive_ptr<ChunkTensor> features) {
+  TORCH_CHECK(features, "sample_blocks_and_index: features store is null");
+  return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace, features);
 }
 
 int64_t GetCurrentAllocated() { return dgs_current_allocated(); }
@@ -575,6 +637,7 @@ std::vector<int64_t> GetRngState() {
 }  // namespace dgs
 
 using dgs::ChunkTensor;
+using dgs::PendingBlocks;
 
 TORCH_LIBRARY(dgs_classes, m) {
   m.class_<ChunkTensor>("ChunkTensor")
@@ -587,6 +650,8 @@ TORCH_LIBRARY(dgs_classes, m) {
       .def("_CAPI_remote_index", &ChunkTensor::RemoteIndex)
       .def("_CAPI_host_index", &ChunkTensor::HostIndex)
       .def("_CAPI_load_from_tensor", &ChunkTensor::LoadFromTensor);
+  // not in upstream: a sample_blocks call in flight
+  m.class_<PendingBlocks>("PendingBlocks").def("_CAPI_finish", &PendingBlocks::Finish);
 }
 
 TORCH_LIBRARY(dgs_ops, m) {
@@ -601,6 +666,8 @@ TORCH_LIBRARY(dgs_ops, m) {
       // not in upstream: the whole sampler loop (and optionally the feature gather) in one call
       .def("_CAPI_sample_blocks", &dgs::SampleBlocks)
       .def("_CAPI_sample_blocks_and_index", &dgs::SampleBlocksAndIndex)
+      .def("_CAPI_sample_blocks_begin", &dgs::SampleBlocksBegin)
+      .def("_CAPI_sample_blocks_and_index_begin", &dgs::SampleBlocksAndIndexBegin)
       // not in upstream: node renumbering (hottest rows first) for the positional stores
       .def("_CAPI_renumber_csc", &dgs::RenumberCSC)
       // not in upstream: the sampling generator's (seed, stream)

@@ -42,6 +42,26 @@ def create_chunktensor(tensor, num_gpus, available_mem, cache_rate=1.0, root_ran
     return chunk_tensor
 
 
+class PendingBatch:
+    """A batch whose kernels are enqueued (ChunkTensorSampler.submit).  result() waits until the
+    batch's sizes are known and returns what sample_blocks / sample_blocks_and_index return; the
+    last kernels of the batch may still be running on the stream it was submitted on, so a consumer
+    on another stream orders itself after that stream (`consumer.wait_stream(batch.stream)`)."""
+
+    def __init__(self, handle, seed_nodes, with_features, stream):
+        self._handle = handle
+        self._seed_nodes = seed_nodes
+        self._with_features = with_features
+        self.stream = stream
+
+    def result(self):
+        frontiers, srcs, dsts, x, seeds = self._handle._CAPI_finish()
+        blocks = ChunkTensorSampler._blocks(seeds, frontiers, srcs, dsts)
+        if self._with_features:
+            return frontiers[-1], self._seed_nodes, blocks, x
+        return frontiers[-1], self._seed_nodes, blocks
+
+
 class ChunkTensorSampler:
     """chunktensor_sampler.py:62-118, same positional arguments (the DGL prefetch options of
     BlockSampler have no counterpart here).
@@ -94,6 +114,22 @@ class ChunkTensorSampler:
             blocks.insert(0, Block(coo_col, coo_row, frontier.numel(), seeds.numel(), frontier, seeds))
             seeds = frontier
         return frontier, seed_nodes, blocks
+
+    def submit(self, g, seed_nodes, chunk_features=None):
+        """Enqueues a batch on the current stream and returns at once (fused path only).  Batches
+        submitted on different streams overlap on the GPU: one batch's gather is bound by HBM
+        bandwidth, the next batch's sampling by memory transactions, and they share the machine
+        well.  Results come from PendingBatch.result(), in any order."""
+        if not self.fused:
+            raise RuntimeError("submit() needs the fused path: uniform sampling with every fanout <= 64")
+        hop_fanouts = list(reversed(self.fanouts))
+        if chunk_features is None:
+            handle = torch.ops.dgs_ops._CAPI_sample_blocks_begin(
+                seed_nodes, self.chunk_indptr, self.chunk_indices, hop_fanouts, self.replace)
+        else:
+            handle = torch.ops.dgs_ops._CAPI_sample_blocks_and_index_begin(
+                seed_nodes, self.chunk_indptr, self.chunk_indices, hop_fanouts, self.replace, chunk_features)
+        return PendingBatch(handle, seed_nodes, chunk_features is not None, torch.cuda.current_stream())
 
     def sample_blocks_and_index(self, g, seed_nodes, chunk_features):
         """sample_blocks followed by chunk_features._CAPI_index(input_nodes)

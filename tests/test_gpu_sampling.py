@@ -292,3 +292,55 @@ def test_host_seeds_are_accepted(pkg, oracle, graph):
         assert out_seeds is s and np.array_equal(_np(frontier), o_frontier)
         _check_blocks(blocks, o_blocks)
         assert blocks[-1].dst_ids.is_cuda and torch.equal(x.cpu(), feats[frontier.cpu()])
+
+
+def test_batches_in_flight_on_two_streams(pkg, oracle, graph):
+    # submit() on alternating streams, results collected later and out of order: every batch must
+    # equal the oracle's for its own rng stream, and the synchronous call must still interleave
+    indptr, indices = graph
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    rng = np.random.default_rng(77)
+    feats = rng.standard_normal((20000, 20)).astype(np.float32)
+    x_ct = pkg.create_chunktensor(torch.from_numpy(feats), 1, big, cache_rate=0.5)
+    fanouts = [7, 5, 3]
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.current_stream()]
+    batches = [rng.integers(0, 20000, size=700).astype(np.int64) for _ in range(9)]
+    pkg.set_rng_state(4321, 50)
+    pending = []
+    for i, b in enumerate(batches):
+        with torch.cuda.stream(streams[i % 3]):
+            pending.append(sampler.submit(None, _dev(b), x_ct if i % 2 == 0 else None))
+        if i == 4:  # a blocking call in the middle takes its own three rng streams
+            f_sync, _, _ = sampler.sample_blocks(None, _dev(batches[0]))
+    order = [8, 0, 3, 1, 7, 2, 6, 5, 4]
+    results = {i: pending[i].result() for i in order}
+    torch.cuda.synchronize()
+    first_stream = 50
+    for i, b in enumerate(batches):
+        want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, fanouts, False, 4321, first_stream)
+        first_stream += 3
+        got = results[i]
+        assert np.array_equal(_np(got[0]), want_f), i
+        for gb, wb in zip(got[2], want_blocks):
+            assert np.array_equal(_np(gb.src_local), wb[0]) and np.array_equal(_np(gb.dst_local), wb[1])
+        if i % 2 == 0:
+            assert np.array_equal(_np(got[3]), feats[want_f])
+        if i == 4:
+            want_sync, _, _ = oracle.sample_blocks(batches[0], indptr, indices, fanouts, False, 4321, first_stream)
+            assert np.array_equal(_np(f_sync), want_sync)
+            first_stream += 3
+    with pytest.raises(RuntimeError, match="already finished"):
+        pending[0]._handle._CAPI_finish()
+    # a fifth stream finds the table pool full and runs on the hash table: same results
+    extra = [torch.cuda.Stream() for _ in range(3)]
+    pkg.set_rng_state(4321, 50)
+    for s_ in extra:
+        with torch.cuda.stream(s_):
+            f, _, _ = sampler.submit(None, _dev(batches[0])).result()
+        s_.synchronize()
+        want_f, _, _ = oracle.sample_blocks(batches[0], indptr, indices, fanouts, False, 4321, 50)
+        assert np.array_equal(_np(f), want_f)
+        pkg.set_rng_state(4321, 50)
