@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 C1_GATHER_TRAFFIC_BYTES_PER_ROW = (378.3e6 + 288.2e6) / 719002.0
 
 WORKLOADS = {
-    # BASELINE.json configs[1]: the configuration the metric is quoted on
+    # benchmark configuration 1: the one the headline metric is quoted on
     "c1": dict(nodes=2_449_029, edges=123_718_280, max_deg=17_000, deg1_frac=0.05, feat_dim=100,
                feat_dtype="float32", batch=1024, fanouts=[15, 10, 5], replace=False, graph_seed=20240602),
     # c1 with a float32 weight per edge: every hop uses the weighted operator
@@ -37,7 +37,7 @@ WORKLOADS = {
     "c1w": dict(nodes=2_449_029, edges=123_718_280, max_deg=17_000, deg1_frac=0.05, feat_dim=100,
                 feat_dtype="float32", batch=1024, fanouts=[15, 10, 5], replace=False, graph_seed=20240602,
                 weighted=True),
-    # BASELINE.json configs[0] (CPU-runnable plumbing case), used by --workload c0
+    # benchmark configuration 0 (CPU-runnable plumbing case), used by --workload c0
     "c0": dict(nodes=10_000, edges=200_000, max_deg=1_000, deg1_frac=0.0, feat_dim=128,
                feat_dtype="float32", batch=1024, fanouts=[10, 5], replace=False, graph_seed=20240601),
 }
@@ -265,20 +265,20 @@ def device_rmat_csc(scale_bits, e, gen):
 
 
 LARGE = {
-    # BASELINE.json configs[2]: large graph, all in HBM, bf16 x128, 4096 seeds from a 1% train subset
+    # benchmark configuration 2: large graph, all in HBM, bf16 x128, 4096 seeds from a 1% train subset
     "c2": dict(graph="powerlaw", nodes=111_059_956, edges=1_615_685_872, dim=128, feat_dtype=torch.bfloat16,
                hbm_rows=1.0, batch=4096, fanouts=[15, 10, 5], replace=False, train_frac=0.01, seed=20240603),
-    # configs[3]: same graph, f32 x256, top 40% of rows by in-degree in HBM, rest in pinned host memory
+    # configuration 3: same graph, f32 x256, top 40% of rows by in-degree in HBM, rest in pinned host memory
     "c3": dict(graph="powerlaw", nodes=111_059_956, edges=1_615_685_872, dim=256, feat_dtype=torch.float32,
                hbm_rows=0.4, batch=8192, fanouts=[20, 15, 10], replace=False, train_frac=1.0, seed=20240604),
-    # configs[4]: R-MAT scale 26, 2^30 edges, with replacement, fanouts [50, 50], 16384 seeds, f32 x64
+    # configuration 4: R-MAT scale 26, 2^30 edges, with replacement, fanouts [50, 50], 16384 seeds, f32 x64
     "c4": dict(graph="rmat", nodes=1 << 26, edges=1 << 30, dim=64, feat_dtype=torch.float32,
                hbm_rows=1.0, batch=16384, fanouts=[50, 50], replace=True, train_frac=1.0, seed=20240605),
 }
 
 
 def run_large(args, dgs):
-    """BASELINE.json configs[2..4], built on the device.  For the two-tier case (c3) the tiers
+    """Benchmark configurations 2 to 4, built on the device.  For the two-tier case (c3) the tiers
     are also timed separately: device tier against HBM, host tier against PCIe Gen5 x16."""
     cfg = LARGE[args.workload]
     scale = args.scale
