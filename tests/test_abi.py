@@ -98,3 +98,30 @@ def test_sampler_cache_size_formula():
     with pytest.raises(ValueError):
         import torch
         pkg.create_chunktensor(torch.zeros(4), 2, 100)
+
+
+def test_placement_host_arithmetic(oracle):
+    # the parts of the placement helpers that need no GPU: degree order, capacity <-> rows, hit rate
+    import numpy as np
+    import torch
+    pl = load_pkg().placement
+    rng = np.random.default_rng(3)
+    deg = rng.integers(0, 9, size=500)
+    indptr = torch.from_numpy(np.concatenate([[0], np.cumsum(deg)]).astype(np.int64))
+    order = pl.degree_order(indptr)
+    assert np.array_equal(order.numpy(), oracle.degree_order(indptr.numpy()))
+    indices = torch.from_numpy(rng.integers(0, 500, size=int(indptr[-1])).astype(np.int64))
+    by_out = pl.degree_order(indptr, indices, by="out")
+    out_deg = np.bincount(indices.numpy(), minlength=500)
+    assert (np.diff(out_deg[by_out.numpy()]) <= 0).all()
+    feats = torch.arange(500 * 6, dtype=torch.float32).reshape(500, 6)
+    assert torch.equal(pl.permute_rows(feats, order, chunk_rows=64), feats[order])
+    # capacity for a prefix of rows and back; upstream's split is in elements, a partial row counts for neither tier
+    cap = pl.capacity_for_rows(feats, rows=123)
+    assert cap == 123 * 6 * 4 and pl.rows_in_hbm(feats, feats.dtype, cap) == 123
+    assert pl.rows_in_hbm(feats, feats.dtype, cap + 5) == 123 and pl.rows_in_hbm(feats, feats.dtype, 10 ** 9) == 500
+    assert pl.capacity_for_rows([500, 6], torch.float32, fraction=0.4) == 200 * 24
+    d = torch.tensor([5.0, 3.0, 1.0, 1.0])
+    assert pl.expected_hit_rate(d, 2) == 0.8 and pl.expected_hit_rate(torch.zeros(3), 1) == 0.0
+    with pytest.raises(ValueError):
+        pl.degree_order(indptr, by="sideways")
