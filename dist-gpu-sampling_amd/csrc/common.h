@@ -125,23 +125,6 @@ __device__ __forceinline__ void single_block_scan_1024(const T* __restrict__ in,
   single_block_scan<1024, T, T>(in, out, count, sum);
 }
 
-// "Last block done" election without spinning: every block calls this once after its
-// global writes; exactly one block (the last to arrive) gets true and may then read what
-// all the others wrote.  The counter must be 0 on entry and is left at 0.
-__device__ __forceinline__ bool last_block_arrives(int* counter) {
-  __shared__ bool is_last;
-  __threadfence();  // release this block's writes at device scope
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int ticket = atomicAdd(counter, 1);
-    is_last = ticket == int(gridDim.x) - 1;
-    if (is_last) *counter = 0;
-  }
-  __syncthreads();
-  if (is_last) __threadfence();  // acquire the other blocks' writes
-  return is_last;
-}
-
 // Philox4x32-10 block for the "dgs-philox-1" contract.
 struct PhiloxWords { uint32_t w[4]; };
 __device__ __forceinline__ PhiloxWords philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,

@@ -405,6 +405,10 @@ __global__ __launch_bounds__(kBlock) void hop_relabel_kernel(Hop h, int64_t bloc
   DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) relabel_tile<IdT, TableT>(h, table, vb);
 }
 
+__global__ void zero_sizes_kernel(int64_t* __restrict__ sizes, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) sizes[i] = 0;
+}
+
 __global__ __launch_bounds__(kBlock) void clear_kernel(uint4* __restrict__ p, int64_t n16) {
   for (int64_t i = int64_t(blockIdx.x) * kBlock + threadIdx.x; i < n16; i += int64_t(gridDim.x) * kBlock)
     p[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
@@ -646,7 +650,9 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
               "sample_blocks: sizes_host and sizes_ticket go together");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n_seeds == 0) {  // nothing to launch: every size is zero
-    DGS_HIP_TRY(hipMemsetAsync(sizes_dev, 0, sizeof(int64_t) * size_t(3 * n_hops + 1), st));
+    // a fill kernel, not a memset node: the call may be recorded into a graph
+    hipLaunchKernelGGL(zero_sizes_kernel, dim3(1), dim3(64), 0, st, sizes_dev, 3 * n_hops + 1);
+    DGS_LAUNCH_CHECK();
     if (sizes_host) {
       for (int i = 0; i < 3 * n_hops + 1; ++i) sizes_host[i] = 0;
       return dgs_ticket_record(st, sizes_ticket);
