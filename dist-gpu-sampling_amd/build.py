@@ -20,7 +20,7 @@ HIP_LIB = os.path.join(HERE, "libdgs_hip.so")
 TORCH_LIB = os.path.join(HERE, "libdgs.so")
 
 HIP_SOURCES = ["store.hip", "gather.hip", "sample.hip", "weighted.hip", "placement.hip", "unique.hip", "pipeline.hip"]
-HIP_HEADERS = ["common.h", "table.h", "picks.h", "weights.h", "sample_workspace.h"]
+HIP_HEADERS = ["common.h", "table.h", "picks.h", "weights.h", "race.h", "sample_workspace.h"]
 ARCH = "gfx950"
 
 
