@@ -73,6 +73,10 @@ SIGNATURES = {
     "dgs_sample_blocks": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, ctypes.POINTER(c_i64), c_i32, c_i32,
                                          c_u64, c_u32, c_vp, c_u32, c_vp, ctypes.POINTER(BlockOut), c_vp, c_vp,
                                          ctypes.POINTER(c_vp), c_vp, c_sz, c_vp]),
+    "dgs_sample_blocks_weighted_workspace_bytes": (c_sz, [c_i64, ctypes.POINTER(c_i64), c_i32, c_i32]),
+    "dgs_sample_blocks_weighted": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, View, ctypes.POINTER(c_i64), c_i32,
+                                                  c_i32, c_u64, c_u32, c_vp, c_u32, c_vp, ctypes.POINTER(BlockOut),
+                                                  c_vp, c_vp, ctypes.POINTER(c_vp), c_vp, c_sz, c_vp]),
     "dgs_renumber_csc": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp]),
     "dgs_read_back": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp]),
     "dgs_read_back_begin": (ctypes.c_int, [c_vp, c_vp, c_sz, c_vp, ctypes.POINTER(c_vp)]),

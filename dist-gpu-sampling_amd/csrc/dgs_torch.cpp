@@ -511,8 +511,11 @@ class PendingBlocks : public torch::CustomClassHolder {
                                                  const c10::intrusive_ptr<ChunkTensor>& indptr,
                                                  const c10::intrusive_ptr<ChunkTensor>& indices,
                                                  const std::vector<int64_t>& fanouts, bool replace,
-                                                 const c10::intrusive_ptr<ChunkTensor>& features) {
+                                                 const c10::intrusive_ptr<ChunkTensor>& features,
+                                                 const c10::intrusive_ptr<ChunkTensor>& probs =
+                                                     c10::intrusive_ptr<ChunkTensor>()) {
     const int32_t w = id_width(seeds_in, "seeds");
+    if (probs) TORCH_CHECK(probs->dtype() == torch::kFloat32, "probs store must be float32, got ", probs->dtype());
     TORCH_CHECK(seeds_in.scalar_type() == indices->dtype(), "seeds (", seeds_in.scalar_type(), ") and indices (",
                 indices->dtype(), ") must have the same dtype");
     TORCH_CHECK(indptr->dtype() == torch::kInt32 || indptr->dtype() == torch::kInt64,
@@ -545,14 +548,24 @@ class PendingBlocks : public torch::CustomClassHolder {
       outs[h] = dgs_block_out{p->src_[h].data_ptr(), p->dst_[h].data_ptr()};
     }
     torch::Tensor sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
-    const size_t ws_bytes = dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
+    const size_t ws_bytes = probs ? dgs_sample_blocks_weighted_workspace_bytes(n, fanouts.data(), hops, w)
+                                  : dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
     torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
-    const auto rng = next_rng(static_cast<uint32_t>(hops));
     const auto table = indptr->node_table(st);
-    check(dgs_sample_blocks(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops,
-                            replace, rng.first, rng.second, table.first, table.second, p->all_.data_ptr(),
-                            outs.data(), sizes_dev.data_ptr<int64_t>(), p->pinned_.data_ptr<int64_t>(), &p->ticket_,
-                            ws.data_ptr(), ws_bytes, st));
+    TORCH_CHECK(!probs || table.first != nullptr,
+                "weighted sample_blocks needs a node table (fewer than 2^31 nodes, at most 4 streams in use): "
+                "use the per-hop operators here");
+    const auto rng = next_rng(static_cast<uint32_t>(hops));
+    if (probs)
+      check(dgs_sample_blocks_weighted(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), probs->view(),
+                                       fanouts.data(), hops, replace, rng.first, rng.second, table.first,
+                                       table.second, p->all_.data_ptr(), outs.data(), sizes_dev.data_ptr<int64_t>(),
+                                       p->pinned_.data_ptr<int64_t>(), &p->ticket_, ws.data_ptr(), ws_bytes, st));
+    else
+      check(dgs_sample_blocks(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops,
+                              replace, rng.first, rng.second, table.first, table.second, p->all_.data_ptr(),
+                              outs.data(), sizes_dev.data_ptr<int64_t>(), p->pinned_.data_ptr<int64_t>(),
+                              &p->ticket_, ws.data_ptr(), ws_bytes, st));
     // the lengths are final at the ticket; the gather is enqueued before anybody waits for them
     if (features) {
       p->x_ = torch::empty({seeds_max[hops], features->elem_stride()},
@@ -613,6 +626,18 @@ c10::intrusive_ptr<PendingBlocks> SampleBlocksAndIndexBegin(torch::Tensor seeds,
   return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace, features);
 }
 
+// Weighted picks (chunktensor_sampler.py:97-100) through the fused driver; `features` may be None.
+c10::intrusive_ptr<PendingBlocks> SampleBlocksWeightedBegin(torch::Tensor seeds,
+                                                            c10::intrusive_ptr<ChunkTensor> indptr,
+                                                            c10::intrusive_ptr<ChunkTensor> indices,
+                                                            c10::intrusive_ptr<ChunkTensor> probs,
+                                                            std::vector<int64_t> fanouts, bool replace,
+                                                            c10::optional<c10::intrusive_ptr<ChunkTensor>> features) {
+  TORCH_CHECK(probs, "sample_blocks_weighted: probs store is null");
+  return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace,
+                              features.has_value() ? *features : c10::intrusive_ptr<ChunkTensor>(), probs);
+}
+
 int64_t GetCurrentAllocated() { return dgs_current_allocated(); }
 
 // upstream nccl::GetUniqueId / nccl::SetNCCL (src/nccl_context.cc:17-34): there is no
@@ -668,6 +693,7 @@ TORCH_LIBRARY(dgs_ops, m) {
       .def("_CAPI_sample_blocks_and_index", &dgs::SampleBlocksAndIndex)
       .def("_CAPI_sample_blocks_begin", &dgs::SampleBlocksBegin)
       .def("_CAPI_sample_blocks_and_index_begin", &dgs::SampleBlocksAndIndexBegin)
+      .def("_CAPI_sample_blocks_weighted_begin", &dgs::SampleBlocksWeightedBegin)
       // not in upstream: node renumbering (hottest rows first) for the positional stores
       .def("_CAPI_renumber_csc", &dgs::RenumberCSC)
       // not in upstream: the sampling generator's (seed, stream)

@@ -34,9 +34,11 @@
 // scanned per 256-row tile, and the packed edge list (src_local, dst_local) is written
 // (rank of a pick = rank recorded at its id's smallest position).
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.h"
 #include "picks.h"
+#include "race.h"
 #include "table.h"
 
 namespace dgs {
@@ -85,6 +87,8 @@ struct Hop {
   uint32_t* slot;           // [all positions] table slot of a position, bit 31 = first occurrence
   uint32_t* rank_at;        // [all positions] rank of the id first seen at that position
   uint8_t* lost;            // [all positions] non-zero: a smaller position of the same id exists
+  int64_t* long_rows;       // weighted only: [s_max] rows handed to the block-per-row launch
+  int64_t* long_count;      // weighted only: entries of long_rows
   int* pos_cnt;             // [position tiles of this hop] first occurrences per tile
   int64_t* pos_off;         // [position tiles] only when position tiles > kInlineTiles
   void* frontier;           // growing array of distinct ids
@@ -195,6 +199,35 @@ __device__ __forceinline__ void mark_lost(const Hop& h, uint32_t displaced) {
   if (displaced != kNoPosition) h.lost[displaced] = 1;
 }
 
+// What becomes of padded position p: with a pick (edge `edge` of the graph) the picked id goes
+// into the table and p's slot word is recorded; without one the position is marked empty.
+template <typename IdT, typename TableT>
+__device__ __forceinline__ void emit_pick(const Hop& h, const TableT& table, const TierView<IdT>& indices, int64_t p,
+                                          bool have, int64_t edge, bool look_first) {
+  uint32_t word = kInvalidSlot;
+  if (have) {
+    const IdT col = indices.at(edge);
+    bool first;
+    uint32_t displaced;
+    word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
+    if (h.index != 0) {
+      if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
+      mark_lost(h, displaced);
+    }
+  }
+  h.slot[p] = word;
+}
+
+// Ids that repeat a lot (hub sources) are cheaper to insert with a look at the entry first;
+// the previous hop tells: if more than a fifth of its picks were not new ids, look first.
+// (hop 0 has no history: look first only when it is big enough for contention to matter)
+__device__ __forceinline__ bool look_before_insert(const Hop& h, int64_t s) {
+  if (h.prev_nnz == nullptr) return s * h.k >= (int64_t(1) << 17);
+  const int64_t picked = *h.prev_nnz;
+  const int64_t fresh = s - *(h.n_seeds - 1);  // ids the previous hop added to the frontier
+  return fresh * 5 < picked * 4;
+}
+
 // One virtual block of the fill launch: 256 / G seed rows.
 template <typename IdT, typename PtrT, typename TableT, int G>
 __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT& table,
@@ -215,15 +248,7 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
   const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;
-  // Ids that repeat a lot (hub sources) are cheaper to insert with a look at the entry first;
-  // the previous hop tells: if more than a fifth of its picks were not new ids, look first.
-  // (hop 0 has no history: look first only when it is big enough for contention to matter)
-  bool look_first = s * k >= (int64_t(1) << 17);
-  if (h.prev_nnz) {
-    const int64_t picked = *h.prev_nnz;
-    const int64_t fresh = s - *(h.n_seeds - 1);  // ids the previous hop added to the frontier
-    look_first = fresh * 5 < picked * 4;
-  }
+  const bool look_first = look_before_insert(h, s);
   if (l == 0) {
     h.row_cnt[i] = bad ? kBadRow : (replace ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
     if (h.index == 0) {  // the caller's seeds open the mapping list; flag() decides their first bits
@@ -234,21 +259,7 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   }
   uint32_t pos;
   const bool have = pick_position<G>(deg, k, replace, l, group_lane0, rng_seed, h.rng_stream, row, &pos);
-  if (l < k) {
-    const int64_t p = h.pos_base + seed_part(h, s) + i * k + l;
-    uint32_t word = kInvalidSlot;
-    if (have) {
-      const IdT col = indices.at(b + pos);
-      bool first;
-      uint32_t displaced;
-      word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
-      if (h.index != 0) {
-        if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
-        mark_lost(h, displaced);
-      }
-    }
-    h.slot[p] = word;
-  }
+  if (l < k) emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, have, b + pos, look_first);
 }
 
 // Virtual blocks [0, fill_blocks): seed rows of this hop; then relabel_count blocks writing the
@@ -269,6 +280,110 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
     } else {
       const int64_t i = (vb - fill_blocks - relabel_count) * kBlock + threadIdx.x;
       if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+}
+
+// ---- weighted picks (race.h): one wave per seed row, a block per row for long rows ----
+
+constexpr int kWeightedRowsPerBlock = kBlock / kWave;
+
+// One virtual block of the weighted fill launch: four seed rows, a wave each.  Rows above
+// long_row<64>() positions are queued for hop_fill_weighted_long_kernel, which fills their
+// positions; everything else about a row is what fill_rows does.
+template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
+__device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, const TableT& table,
+                                                   const TierView<PtrT>& indptr, const TierView<IdT>& indices,
+                                                   const TierView<float>& probs, uint64_t rng_seed) {
+  const Group<kWave> g;
+  const int64_t s = seeds_of(h);
+  if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
+  const int64_t i = vb * kWeightedRowsPerBlock + threadIdx.x / kWave;
+  if (i >= s) return;  // whole waves leave together
+  const IdT seed = static_cast<const IdT*>(h.seeds)[i];
+  const int64_t row = int64_t(seed);
+  const int64_t b = int64_t(indptr.at(row));
+  const int64_t deg64 = int64_t(indptr.at(row + 1)) - b;
+  const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
+  const uint32_t deg = bad ? 0u : uint32_t(deg64);
+  const int k = h.k;
+  const bool look_first = look_before_insert(h, s);
+  if (g.l == 0) {
+    h.row_cnt[i] = bad ? kBadRow : (REPLACE ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
+    if (h.index == 0) {
+      bool first;
+      uint32_t displaced;
+      h.slot[h.pos_base + i] = table.insert_min(seed, uint32_t(h.pos_base + i), &first, &displaced);
+    }
+  }
+  const int64_t p0 = h.pos_base + seed_part(h, s) + i * k;
+  if (deg == 0) {
+    if (g.l < k) h.slot[p0 + g.l] = kInvalidSlot;
+    return;
+  }
+  if (deg > long_row<kWave>() && (REPLACE || deg > uint32_t(k))) {
+    if (g.l == 0) h.long_rows[atomicAdd(reinterpret_cast<unsigned long long*>(h.long_count), 1ull)] = i;
+    return;
+  }
+  if (REPLACE) {
+    draw_row<kWave>(g, probs, b, int64_t(deg), int64_t(k), rng_seed, h.rng_stream, row, [&](int64_t j, int64_t pick) {
+      emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first);
+    });
+  } else if (deg <= uint32_t(k)) {
+    if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, uint32_t(g.l) < deg, b + g.l, look_first);
+  } else {
+    Race r;
+    race_row<kWave>(r, g, probs, b, deg, k, rng_seed, h.rng_stream, row);
+    if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, r.pos < deg, b + r.pos, look_first);
+  }
+}
+
+// Same layout of virtual blocks as hop_fill_kernel (fill, previous hop's edge list, clearing).
+template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
+__global__ __launch_bounds__(kBlock) void hop_fill_weighted_kernel(Hop h, Hop prev, int64_t fill_blocks,
+                                                                   int64_t relabel_count, uint4* clear_begin,
+                                                                   int64_t clear_n16, TableT table,
+                                                                   TierView<PtrT> indptr, TierView<IdT> indices,
+                                                                   TierView<float> probs, uint64_t rng_seed) {
+  const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
+  const int64_t total = fill_blocks + relabel_count + clear_blocks;
+  for (int64_t vb = blockIdx.x; vb < total; vb += gridDim.x) {
+    if (vb < fill_blocks) {
+      fill_rows_weighted<IdT, PtrT, TableT, REPLACE>(h, vb, table, indptr, indices, probs, rng_seed);
+    } else if (vb < fill_blocks + relabel_count) {
+      relabel_tile<IdT, TableT>(prev, table, vb - fill_blocks);
+    } else {
+      const int64_t i = (vb - fill_blocks - relabel_count) * kBlock + threadIdx.x;
+      if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+}
+
+// The queued long rows of a hop, a 1024-thread block per row.
+template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
+__global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop h, TableT table,
+                                                                            TierView<PtrT> indptr,
+                                                                            TierView<IdT> indices,
+                                                                            TierView<float> probs, uint64_t rng_seed) {
+  __shared__ LongRowScratch lds;
+  const int64_t n_long = *h.long_count;
+  const int64_t s = seeds_of(h);
+  const bool look_first = look_before_insert(h, s);
+  const int k = h.k;
+  for (int64_t t = blockIdx.x; t < n_long; t += gridDim.x) {
+    const int64_t i = h.long_rows[t];
+    const int64_t row = int64_t(static_cast<const IdT*>(h.seeds)[i]);
+    const int64_t b = int64_t(indptr.at(row));
+    const uint32_t deg = uint32_t(int64_t(indptr.at(row + 1)) - b);  // queued rows have a valid degree
+    const int64_t p0 = h.pos_base + seed_part(h, s) + i * k;
+    if (REPLACE) {
+      draw_long_row(lds, probs, b, int64_t(deg), int64_t(k), rng_seed, h.rng_stream, row,
+                    [&](int64_t j, int64_t pick) { emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first); });
+    } else {
+      Race r;
+      race_long_row(r, lds, probs, b, deg, k, rng_seed, h.rng_stream, row);
+      const int l = threadIdx.x;  // wave 0 holds the winners
+      if (l < k) emit_pick<IdT>(h, table, indices, p0 + l, r.pos < deg, b + r.pos, look_first);
     }
   }
 }
@@ -425,6 +540,7 @@ struct Plan {
   int64_t nnz_max[DGS_MAX_HOPS];
   uint32_t capacity = 0;     // hash table slots (one table for all hops)
   size_t table_bytes = 0;    // 0 for the direct table
+  bool weighted = false;     // picks by edge weight: per-hop queues for long rows
 };
 
 dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, int32_t id_bytes,
@@ -468,6 +584,7 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
   uint32_t* slot = c.take<uint32_t>(positions);
   uint32_t* rank_at = c.take<uint32_t>(positions);
   uint8_t* lost = c.take<uint8_t>(positions + 16);
+  int64_t* long_counts = p.weighted ? c.take<int64_t>(DGS_MAX_HOPS) : nullptr;
   int64_t pos_base = 0;
   for (int h = 0; h < p.n_hops; ++h) {
     const size_t s = size_t(p.s_max[h]);
@@ -483,6 +600,8 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
     v.slot = slot;
     v.rank_at = rank_at;
     v.lost = lost;
+    v.long_rows = p.weighted ? c.take<int64_t>(s) : nullptr;
+    v.long_count = p.weighted ? long_counts + h : nullptr;
     v.pos_cnt = c.take<int>(pos_tiles + 1);
     v.pos_off = pos_tiles > size_t(kInlineTiles) ? c.take<int64_t>(pos_tiles) : nullptr;
     v.s_max = p.s_max[h];
@@ -512,10 +631,35 @@ void launch_fill(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* 
                        TierView<PtrT>(indptr), TierView<IdT>(indices), replace, rng_seed);
 }
 
+// The weighted fill of one hop: the main launch (a wave per row) and the block-per-row launch for
+// the rows it queued.  Only the direct table is supported (the entry point insists on one).
+template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
+dgs_status launch_fill_weighted(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* clear_begin,
+                                int64_t clear_n16, const TableT& table, const dgs_view& indptr,
+                                const dgs_view& indices, const dgs_view& probs, uint64_t rng_seed, hipStream_t st) {
+  const int64_t fill_blocks = (cur.s_max + kWeightedRowsPerBlock - 1) / kWeightedRowsPerBlock;
+  const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
+  const int64_t total = fill_blocks + relabel_count + clear_blocks;
+  hipLaunchKernelGGL((hop_fill_weighted_kernel<IdT, PtrT, TableT, REPLACE>), dim3(capped_grid(total)), dim3(kBlock),
+                     0, st, cur, prev, fill_blocks, relabel_count, clear_begin, clear_n16, table,
+                     TierView<PtrT>(indptr), TierView<IdT>(indices), TierView<float>(probs), rng_seed);
+  DGS_LAUNCH_CHECK();
+  const uint32_t long_blocks = uint32_t(cur.s_max < 512 ? (cur.s_max < 1 ? 1 : cur.s_max) : 512);
+  hipLaunchKernelGGL((hop_fill_weighted_long_kernel<IdT, PtrT, TableT, REPLACE>), dim3(long_blocks),
+                     dim3(kLongBlock), 0, st, cur, table, TierView<PtrT>(indptr), TierView<IdT>(indices),
+                     TierView<float>(probs), rng_seed);
+  DGS_LAUNCH_CHECK();
+  return DGS_OK;
+}
+
 template <typename IdT, typename PtrT, typename TableT>
 dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_view& indptr,
-                      const dgs_view& indices, bool replace, uint64_t rng_seed, void** sizes_ticket,
-                      hipStream_t st) {
+                      const dgs_view& indices, const dgs_view* probs, bool replace, uint64_t rng_seed,
+                      void** sizes_ticket, hipStream_t st) {
+  if (p.weighted) {  // the long-row queues of all hops start empty
+    hipLaunchKernelGGL(zero_sizes_kernel, dim3(1), dim3(64), 0, st, hops[0].long_count, p.n_hops);
+    DGS_LAUNCH_CHECK();
+  }
   for (int h = 0; h < p.n_hops; ++h) {
     const Hop& cur = hops[h];
     const Hop prev = h > 0 ? hops[h - 1] : Hop{};
@@ -530,7 +674,16 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
       clear_begin = reinterpret_cast<uint4*>(cur.lost + first);
       clear_n16 = last > first ? (last - first) / 16 : 0;
     }
-    if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
+    if constexpr (std::is_same_v<TableT, DirectTable<IdT>>) {
+      if (p.weighted) {
+        const dgs_status ws = replace ? launch_fill_weighted<IdT, PtrT, TableT, true>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st)
+                                      : launch_fill_weighted<IdT, PtrT, TableT, false>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st);
+        if (ws != DGS_OK) return ws;
+      }
+    }
+    if (p.weighted) {
+      // filled above
+    } else if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else if (cur.k <= 16) launch_fill<IdT, PtrT, TableT, 16>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else launch_fill<IdT, PtrT, TableT, 64>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
@@ -584,20 +737,20 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
 
 template <typename IdT, typename PtrT>
 dgs_status run_blocks_table(const Plan& p, Hop* hops, void* hash_table, void* node_table, uint32_t epoch,
-                            const dgs_view& indptr, const dgs_view& indices, bool replace, uint64_t rng_seed,
-                            void** sizes_ticket, hipStream_t st) {
+                            const dgs_view& indptr, const dgs_view& indices, const dgs_view* probs, bool replace,
+                            uint64_t rng_seed, void** sizes_ticket, hipStream_t st) {
   if (p.kind == TableKind::kDirect)
     return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch), indptr, indices,
-                                                   replace, rng_seed, sizes_ticket, st);
+                                                   probs, replace, rng_seed, sizes_ticket, st);
   const int64_t n16 = int64_t(p.table_bytes / 16);
   hipLaunchKernelGGL(clear_kernel, dim3(capped_grid((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                      static_cast<uint4*>(hash_table), n16);
   DGS_LAUNCH_CHECK();
   if (p.kind == TableKind::kPacked)
     return run_blocks<IdT, PtrT, Table<IdT, true>>(p, hops, Table<IdT, true>(hash_table, p.capacity), indptr,
-                                                   indices, replace, rng_seed, sizes_ticket, st);
+                                                   indices, probs, replace, rng_seed, sizes_ticket, st);
   return run_blocks<IdT, PtrT, Table<IdT, false>>(p, hops, Table<IdT, false>(hash_table, p.capacity), indptr,
-                                                  indices, replace, rng_seed, sizes_ticket, st);
+                                                  indices, probs, replace, rng_seed, sizes_ticket, st);
 }
 
 }  // namespace
@@ -628,17 +781,35 @@ DGS_API size_t dgs_node_table_bytes(int64_t n_nodes) {
   return n_nodes > 0 && n_nodes < 0x7fffffffLL ? size_t(n_nodes) * 8 : 0;
 }
 
-DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
-                                     dgs_view indices, const int64_t* fanouts, int32_t n_hops, int32_t replace,
-                                     uint64_t rng_seed, uint32_t first_stream, void* node_table,
-                                     uint32_t node_table_epoch, void* frontier, const dgs_block_out* outs,
-                                     int64_t* sizes_dev, int64_t* sizes_host, void** sizes_ticket,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
+DGS_API size_t dgs_sample_blocks_weighted_workspace_bytes(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops,
+                                                          int32_t id_bytes) {
+  dgs::Plan p;
+  if (dgs::make_plan(n_seeds, fanouts, n_hops, id_bytes, 1, true, &p) != DGS_OK) return 0;
+  p.weighted = true;
+  return dgs::layout(p, fanouts, nullptr, nullptr, nullptr);
+}
+
+namespace {
+dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
+                               dgs_view indices, const dgs_view* probs, const int64_t* fanouts, int32_t n_hops,
+                               int32_t replace, uint64_t rng_seed, uint32_t first_stream, void* node_table,
+                               uint32_t node_table_epoch, void* frontier, const dgs_block_out* outs,
+                               int64_t* sizes_dev, int64_t* sizes_host, void** sizes_ticket, void* workspace,
+                               size_t workspace_bytes, void* stream) {
   using namespace dgs;
   Plan p;
   // node count = indptr entries - 1
   dgs_status s = make_plan(n_seeds, fanouts, n_hops, id_bytes, indptr.total - 1, node_table != nullptr, &p);
   if (s != DGS_OK) return s;
+  if (probs != nullptr) {
+    DGS_REQUIRE(node_table != nullptr, DGS_ERR_UNSUPPORTED, "sample_blocks_weighted: a node table is required");
+    DGS_REQUIRE(probs->elem_bytes == 4 && probs->total == indices.total, DGS_ERR_INVALID,
+                "sample_blocks_weighted: %lld weights of %d bytes for %lld edges (float32, one per edge)",
+                (long long)probs->total, probs->elem_bytes, (long long)indices.total);
+    p.weighted = true;
+  }
+  const size_t need = probs != nullptr ? dgs_sample_blocks_weighted_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes)
+                                       : dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes);
   DGS_REQUIRE(width_ok(indptr.elem_bytes), DGS_ERR_INVALID, "sample_blocks: indptr width %d", indptr.elem_bytes);
   DGS_REQUIRE(indices.elem_bytes == id_bytes, DGS_ERR_INVALID,
               "sample_blocks: indices width %d differs from the seed width %d", indices.elem_bytes, id_bytes);
@@ -660,9 +831,8 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
     return DGS_OK;
   }
   DGS_REQUIRE(seeds != nullptr && frontier != nullptr, DGS_ERR_INVALID, "sample_blocks: null seeds or frontier");
-  DGS_REQUIRE(workspace != nullptr && workspace_bytes >= dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes),
-              DGS_ERR_WORKSPACE, "sample_blocks: workspace of %zu B, need %zu", workspace_bytes,
-              dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes));
+  DGS_REQUIRE(workspace != nullptr && workspace_bytes >= need, DGS_ERR_WORKSPACE,
+              "sample_blocks: workspace of %zu B, need %zu", workspace_bytes, need);
   DGS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, DGS_ERR_WORKSPACE,
               "sample_blocks: workspace must be 256-byte aligned");
   Hop hops[DGS_MAX_HOPS];
@@ -690,9 +860,33 @@ DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_
   const bool rep = replace != 0;
   if (id_bytes == 8)
     return indptr.elem_bytes == 8
-               ? run_blocks_table<int64_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st)
-               : run_blocks_table<int64_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st);
+               ? run_blocks_table<int64_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st)
+               : run_blocks_table<int64_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st);
   return indptr.elem_bytes == 8
-             ? run_blocks_table<int32_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st)
-             : run_blocks_table<int32_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, rep, rng_seed, sizes_ticket, st);
+             ? run_blocks_table<int32_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st)
+             : run_blocks_table<int32_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st);
+}
+}  // namespace
+
+DGS_API dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
+                                     dgs_view indices, const int64_t* fanouts, int32_t n_hops, int32_t replace,
+                                     uint64_t rng_seed, uint32_t first_stream, void* node_table,
+                                     uint32_t node_table_epoch, void* frontier, const dgs_block_out* outs,
+                                     int64_t* sizes_dev, int64_t* sizes_host, void** sizes_ticket,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+  return sample_blocks_entry(seeds, id_bytes, n_seeds, indptr, indices, nullptr, fanouts, n_hops, replace, rng_seed,
+                             first_stream, node_table, node_table_epoch, frontier, outs, sizes_dev, sizes_host,
+                             sizes_ticket, workspace, workspace_bytes, stream);
+}
+
+DGS_API dgs_status dgs_sample_blocks_weighted(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
+                                              dgs_view indices, dgs_view probs, const int64_t* fanouts,
+                                              int32_t n_hops, int32_t replace, uint64_t rng_seed,
+                                              uint32_t first_stream, void* node_table, uint32_t node_table_epoch,
+                                              void* frontier, const dgs_block_out* outs, int64_t* sizes_dev,
+                                              int64_t* sizes_host, void** sizes_ticket, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+  return sample_blocks_entry(seeds, id_bytes, n_seeds, indptr, indices, &probs, fanouts, n_hops, replace, rng_seed,
+                             first_stream, node_table, node_table_epoch, frontier, outs, sizes_dev, sizes_host,
+                             sizes_ticket, workspace, workspace_bytes, stream);
 }

@@ -67,10 +67,10 @@ class ChunkTensorSampler:
     BlockSampler have no counterpart here).
 
     sample_blocks runs the upstream loop -- per hop one sampling call and one relabel call,
-    over reversed(fanouts).  Uniform sampling goes through the single fused operator when
-    every fanout is at most 64 (`fused=False` forces the per-hop operators; both give
-    identical results); with `chunk_probs` (a float32 ChunkTensor of edge weights) every hop
-    calls the weighted operator, as upstream does (:97-100).
+    over reversed(fanouts) -- through the single fused operator when every fanout is at most
+    64 (`fused=False` forces the per-hop operators; both give identical results).  With
+    `chunk_probs` (a float32 ChunkTensor of edge weights) every hop picks by weight, as
+    upstream does (:97-100).
     """
 
     FUSED_MAX_FANOUT = 64
@@ -81,8 +81,7 @@ class ChunkTensorSampler:
         self.chunk_probs = chunk_probs
         self.fanouts = list(fanouts)
         self.replace = replace
-        self.fused = (fused and chunk_probs is None
-                      and all(0 <= f <= self.FUSED_MAX_FANOUT for f in self.fanouts))
+        self.fused = fused and all(0 <= f <= self.FUSED_MAX_FANOUT for f in self.fanouts)
 
     @staticmethod
     def _blocks(seeds, frontiers, srcs, dsts):
@@ -95,6 +94,8 @@ class ChunkTensorSampler:
     def sample_blocks(self, g, seed_nodes, exclude_eids=None):
         """Returns (input_nodes, seed_nodes, blocks); `g` is unused, as upstream.  Host-side
         seed_nodes (what upstream's DataLoader passes) are uploaded by the operator itself."""
+        if self.fused and self.chunk_probs is not None:
+            return self.submit(g, seed_nodes).result()
         if self.fused:
             frontiers, srcs, dsts, seeds = torch.ops.dgs_ops._CAPI_sample_blocks(
                 seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace)
@@ -121,9 +122,13 @@ class ChunkTensorSampler:
         bandwidth, the next batch's sampling by memory transactions, and they share the machine
         well.  Results come from PendingBatch.result(), in any order."""
         if not self.fused:
-            raise RuntimeError("submit() needs the fused path: uniform sampling with every fanout <= 64")
+            raise RuntimeError("submit() needs the fused path: every fanout <= 64")
         hop_fanouts = list(reversed(self.fanouts))
-        if chunk_features is None:
+        if self.chunk_probs is not None:
+            handle = torch.ops.dgs_ops._CAPI_sample_blocks_weighted_begin(
+                seed_nodes, self.chunk_indptr, self.chunk_indices, self.chunk_probs, hop_fanouts, self.replace,
+                chunk_features)
+        elif chunk_features is None:
             handle = torch.ops.dgs_ops._CAPI_sample_blocks_begin(
                 seed_nodes, self.chunk_indptr, self.chunk_indices, hop_fanouts, self.replace)
         else:
@@ -139,6 +144,8 @@ class ChunkTensorSampler:
         if not self.fused:
             frontier, _, blocks = self.sample_blocks(g, seed_nodes)
             return frontier, seed_nodes, blocks, chunk_features._CAPI_index(frontier)
+        if self.chunk_probs is not None:
+            return self.submit(g, seed_nodes, chunk_features).result()
         frontiers, srcs, dsts, x, seeds = torch.ops.dgs_ops._CAPI_sample_blocks_and_index(
             seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
             chunk_features)

@@ -349,6 +349,28 @@ dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seed
                              void** sizes_ticket, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/*
+ * The same multi-hop driver with weighted picks: every hop chooses neighbours by the
+ * edge weights `probs` (float32, one per edge, laid out like `indices`), by the rules
+ * stated at dgs_sample_fill_weighted.  Results are identical to calling
+ * dgs_sample_neighbors_weighted (rng_stream = first_stream + h) and dgs_unique_relabel
+ * per hop: the loop of ChunkTensorSampler.sample_blocks with chunk_probs
+ * (oppo_bench/single_node/utils/chunktensor_sampler.py:93-118).  All other arguments are
+ * those of dgs_sample_blocks, except that `node_table` is required (DGS_ERR_UNSUPPORTED
+ * without one) and the workspace is sized by the _weighted_ query.
+ */
+size_t dgs_sample_blocks_weighted_workspace_bytes(int64_t n_seeds, const int64_t* fanouts,
+                                                  int32_t n_hops, int32_t id_bytes);
+dgs_status dgs_sample_blocks_weighted(const void* seeds, int32_t id_bytes, int64_t n_seeds,
+                                      dgs_view indptr, dgs_view indices, dgs_view probs,
+                                      const int64_t* fanouts, int32_t n_hops,
+                                      int32_t replace, uint64_t rng_seed,
+                                      uint32_t first_stream, void* node_table,
+                                      uint32_t node_table_epoch, void* frontier,
+                                      const dgs_block_out* outs, int64_t* sizes_dev,
+                                      int64_t* sizes_host, void** sizes_ticket,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Placement                                                                 */
 /* ------------------------------------------------------------------------ */

@@ -173,21 +173,76 @@ def test_weighted_inclusion_frequencies(pkg):
 
 @pytest.mark.parametrize("replace", [False, True])
 def test_weighted_sampler_loop(pkg, oracle, graph, replace):
-    # ChunkTensorSampler with chunk_probs: the upstream loop with the weighted operator per hop
+    # ChunkTensorSampler with chunk_probs: the upstream loop with weighted picks in every hop, through
+    # the fused driver (default), the per-hop operators, and with batches in flight on two streams
     indptr, indices, probs = graph
     rng = np.random.default_rng(2)
-    seeds = rng.permutation(20000)[:512].astype(np.int64)
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big, cache_rate=0.5)
+    pr_ct = pkg.create_chunktensor(torch.from_numpy(probs), 1, big, cache_rate=0.3)
+    feats = rng.standard_normal((20000, 12)).astype(np.float32)
+    x_ct = pkg.create_chunktensor(torch.from_numpy(feats), 1, big)
+    fanouts = [6, 4, 3]
+    batches = [rng.permutation(20000)[:512].astype(np.int64) for _ in range(4)]
+    batches.append(np.array([5, 5, 7, 5], dtype=np.int64))      # repeated seeds
+    batches.append(np.empty(0, dtype=np.int64))
+
+    def check(got, want_f, want_blocks):
+        assert np.array_equal(_np(got[0]), want_f)
+        assert len(got[2]) == 3
+        for g, w in zip(got[2], want_blocks):
+            assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
+            assert (g.num_src, g.num_dst) == (w[2], w[3])
+
+    for fused in (True, False):
+        sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, pr_ct, replace, fused=fused)
+        assert sampler.fused == fused
+        pkg.set_rng_state(31337, 10)
+        for i, b in enumerate(batches):
+            want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, fanouts, replace, 31337, 10 + 3 * i,
+                                                          probs=probs)
+            got = sampler.sample_blocks_and_index(None, torch.from_numpy(b), x_ct)
+            check(got, want_f, want_blocks)
+            assert np.array_equal(_np(got[3]), feats[want_f])
+    # in flight
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, pr_ct, replace)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    pkg.set_rng_state(31337, 10)
+    pending = []
+    for i, b in enumerate(batches):
+        with torch.cuda.stream(streams[i % 2]):
+            pending.append(sampler.submit(None, _dev(b)))
+    for i in reversed(range(len(batches))):
+        want_f, _, want_blocks = oracle.sample_blocks(batches[i], indptr, indices, fanouts, replace, 31337, 10 + 3 * i,
+                                                      probs=probs)
+        check(pending[i].result(), want_f, want_blocks)
+    torch.cuda.synchronize()
+
+
+def test_weighted_fused_long_rows_and_wide_fanout(pkg, oracle):
+    # rows longer than a wave's share (block-per-row launch inside the fused driver), fanout 64,
+    # rows without positive weights, int32 ids with int64 offsets
+    rng = np.random.default_rng(6)
+    deg = np.concatenate([rng.integers(0, 90, size=3000), [2049, 4100, 9000, 30000, 2048, 0, 1]])
+    rng.shuffle(deg)
+    n = deg.size
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, n, size=int(indptr[-1])).astype(np.int32)
+    probs = (rng.random(indices.size) ** 3).astype(np.float32)
+    probs[indptr[10]:indptr[11]] = 0.0
     big = 1 << 40
     ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
     ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
     pr_ct = pkg.create_chunktensor(torch.from_numpy(probs), 1, big)
-    sampler = pkg.ChunkTensorSampler([6, 4, 3], ip_ct, ix_ct, pr_ct, replace)
-    pkg.set_rng_state(31337, 10)
-    frontier, seed_out, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
-    want_frontier, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, [6, 4, 3], replace, 31337, 10,
-                                                         probs=probs)
-    assert np.array_equal(_np(frontier), want_frontier)
-    assert len(blocks) == 3
-    for got, want in zip(blocks, want_blocks):
-        assert np.array_equal(_np(got.src_local), want[0]) and np.array_equal(_np(got.dst_local), want[1])
-        assert (got.num_src, got.num_dst) == (want[2], want[3])
+    long_rows = np.flatnonzero(deg > 2000).astype(np.int32)
+    seeds = np.concatenate([long_rows, rng.integers(0, n, size=400).astype(np.int32)])
+    for fanouts, replace in [([64, 5], False), ([3, 64], True), ([20], False), ([20], True)]:
+        pkg.set_rng_state(99, 0)
+        sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, pr_ct, replace)
+        assert sampler.fused
+        f, _, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
+        want_f, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, replace, 99, 0, probs=probs)
+        assert np.array_equal(_np(f), want_f), (fanouts, replace)
+        for g, w in zip(blocks, want_blocks):
+            assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
