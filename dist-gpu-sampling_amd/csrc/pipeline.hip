@@ -298,12 +298,13 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
   const Group<kWave> g;
   const int64_t s = seeds_of(h);
   if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
-  const int64_t i = vb * kWeightedRowsPerBlock + threadIdx.x / kWave;
+  // the row and everything read for it are the same in all 64 lanes: keep them in scalar registers
+  const int64_t i = vb * kWeightedRowsPerBlock + int64_t(wave_uniform(uint32_t(threadIdx.x / kWave)));
   if (i >= s) return;  // whole waves leave together
-  const IdT seed = static_cast<const IdT*>(h.seeds)[i];
+  const IdT seed = IdT(wave_uniform(int64_t(static_cast<const IdT*>(h.seeds)[i])));
   const int64_t row = int64_t(seed);
-  const int64_t b = int64_t(indptr.at(row));
-  const int64_t deg64 = int64_t(indptr.at(row + 1)) - b;
+  const int64_t b = wave_uniform(int64_t(indptr.at(row)));
+  const int64_t deg64 = wave_uniform(int64_t(indptr.at(row + 1))) - b;
   const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
   const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;

@@ -77,6 +77,16 @@ __device__ __forceinline__ uint64_t lane_read(uint64_t v, int src) {
   return uint64_t(lane_read(uint32_t(v), src)) | (uint64_t(lane_read(uint32_t(v >> 32), src)) << 32);
 }
 
+// A value known to be the same in every lane of the wave, moved to scalar registers: it stops
+// occupying a vector register per lane, and loads addressed by it become scalar loads.
+__device__ __forceinline__ uint32_t wave_uniform(uint32_t v) {
+  return uint32_t(__builtin_amdgcn_readfirstlane(int(v)));
+}
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+  const uint64_t u = uint64_t(v);
+  return int64_t(uint64_t(wave_uniform(uint32_t(u))) | (uint64_t(wave_uniform(uint32_t(u >> 32))) << 32));
+}
+
 // A group's num_picks best so far, ascending over lanes 0 .. k-1; other lanes hold (kNoKey, kNoPos).
 struct Race {
   uint64_t key;
