@@ -287,6 +287,7 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
 // ---- weighted picks (race.h): one wave per seed row, a block per row for long rows ----
 
 constexpr int kWeightedRowsPerBlock = kBlock / kWave;
+constexpr int64_t kMaxLongGrid = 512;
 
 // One virtual block of the weighted fill launch: four seed rows, a wave each.  Rows above
 // long_row<64>() positions are queued for hop_fill_weighted_long_kernel, which fills their
@@ -645,7 +646,8 @@ dgs_status launch_fill_weighted(const Hop& cur, const Hop& prev, int64_t relabel
                      0, st, cur, prev, fill_blocks, relabel_count, clear_begin, clear_n16, table,
                      TierView<PtrT>(indptr), TierView<IdT>(indices), TierView<float>(probs), rng_seed);
   DGS_LAUNCH_CHECK();
-  const uint32_t long_blocks = uint32_t(cur.s_max < 512 ? (cur.s_max < 1 ? 1 : cur.s_max) : 512);
+  // two 1024-thread blocks fit a CU: at most one round over the 256 CUs
+  const uint32_t long_blocks = uint32_t(cur.s_max < kMaxLongGrid ? (cur.s_max < 1 ? 1 : cur.s_max) : kMaxLongGrid);
   hipLaunchKernelGGL((hop_fill_weighted_long_kernel<IdT, PtrT, TableT, REPLACE>), dim3(long_blocks),
                      dim3(kLongBlock), 0, st, cur, table, TierView<PtrT>(indptr), TierView<IdT>(indices),
                      TierView<float>(probs), rng_seed);
@@ -657,7 +659,7 @@ template <typename IdT, typename PtrT, typename TableT>
 dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_view& indptr,
                       const dgs_view& indices, const dgs_view* probs, bool replace, uint64_t rng_seed,
                       void** sizes_ticket, hipStream_t st) {
-  if (p.weighted) {  // the long-row queues of all hops start empty
+  if (p.weighted) {  // the long-row queues of all hops start empty (their counters are one array, hop 0's first)
     hipLaunchKernelGGL(zero_sizes_kernel, dim3(1), dim3(64), 0, st, hops[0].long_count, p.n_hops);
     DGS_LAUNCH_CHECK();
   }
@@ -675,15 +677,13 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
       clear_begin = reinterpret_cast<uint4*>(cur.lost + first);
       clear_n16 = last > first ? (last - first) / 16 : 0;
     }
-    if constexpr (std::is_same_v<TableT, DirectTable<IdT>>) {
-      if (p.weighted) {
+    if (p.weighted) {
+      // only instantiated for the direct table: the entry point refuses weighted calls without one
+      if constexpr (std::is_same_v<TableT, DirectTable<IdT>>) {
         const dgs_status ws = replace ? launch_fill_weighted<IdT, PtrT, TableT, true>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st)
                                       : launch_fill_weighted<IdT, PtrT, TableT, false>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st);
         if (ws != DGS_OK) return ws;
       }
-    }
-    if (p.weighted) {
-      // filled above
     } else if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else if (cur.k <= 16) launch_fill<IdT, PtrT, TableT, 16>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
