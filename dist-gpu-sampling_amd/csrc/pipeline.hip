@@ -342,7 +342,7 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
 
 // Same layout of virtual blocks as hop_fill_kernel (fill, previous hop's edge list, clearing).
 template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
-__global__ __launch_bounds__(kBlock) void hop_fill_weighted_kernel(Hop h, Hop prev, int64_t fill_blocks,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(5, 8))) void hop_fill_weighted_kernel(Hop h, Hop prev, int64_t fill_blocks,
                                                                    int64_t relabel_count, uint4* clear_begin,
                                                                    int64_t clear_n16, TableT table,
                                                                    TierView<PtrT> indptr, TierView<IdT> indices,
