@@ -334,9 +334,8 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
   } else if (deg <= uint32_t(k)) {
     if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, uint32_t(g.l) < deg, b + g.l, look_first);
   } else {
-    Race r;
-    race_row<kWave>(r, g, probs, b, deg, k, rng_seed, h.rng_stream, row);
-    if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, r.pos < deg, b + r.pos, look_first);
+    const uint32_t pos = race_row<kWave>(g, probs, b, deg, k, rng_seed, h.rng_stream, row);
+    if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, pos < deg, b + pos, look_first);
   }
 }
 

@@ -113,13 +113,13 @@ __device__ __forceinline__ void race_refresh_last(Race& r, int k) {
 
 // Bitonic sort of one (key, position) pair per lane over every G-lane group, ascending.  With
 // kByKeyOnly the positions ride along uncompared, which is right whenever the keys are distinct.
-template <int G, bool kByKeyOnly>
-__device__ __forceinline__ void group_sort(uint64_t& key, uint32_t& pos, int l) {
+template <int G, bool kByKeyOnly, typename KeyT>
+__device__ __forceinline__ void group_sort(KeyT& key, uint32_t& pos, int l) {
 #pragma unroll
   for (int size = 2; size <= G; size <<= 1) {
 #pragma unroll
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      const uint64_t ok = lane_xor(key, stride);
+      const KeyT ok = lane_xor(key, stride);
       const uint32_t op = lane_xor(pos, stride);
       const bool take_min = ((l & stride) == 0) == ((l & size) == 0);
       // distinct pairs: "the other one is smaller" decides both the lower and the upper lane
@@ -222,10 +222,39 @@ __device__ __forceinline__ uint64_t lowest_bar_after_sync(uint64_t* bars, int la
   return lowest_bar(bars, lane);
 }
 
-// Runs positions [begin, end) of the group's row, in steps of `stride`, through its race.  begin
-// and stride are multiples of 4 G: one Philox block per lane covers 4 G positions (four words
-// each), and the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the group.
-// `bars` (block-per-row kernel only) is the block's table of published last keys.
+// Race keys of the four G-position steps of the stretch that begins at position sb (a multiple of
+// 4 G) of the group's row, kNoKey from `end` on: one Philox block per lane covers the stretch
+// (four words each), the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the
+// group.  The four steps are independent: their loads are issued together and their key
+// arithmetic (long dependent float64 chains) interleaves.
+template <int G>
+__device__ __forceinline__ void stretch_keys(const Group<G>& g, const TierView<float>& probs, int64_t start,
+                                             uint64_t sb, uint64_t end, uint64_t rng_seed, uint32_t rng_stream,
+                                             int64_t row, uint64_t ck[4]) {
+  float wt[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
+    wt[c] = p < end ? probs.at(start + int64_t(p)) : 0.0f;
+  }
+  PhiloxWords w{{0, 0, 0, 0}};
+  if (sb + 4u * uint32_t(g.l) < end)
+    w = philox4x32_10(0x80000000u | (uint32_t(sb >> 2) + uint32_t(g.l)), rng_stream, uint32_t(uint64_t(row)),
+                      uint32_t(uint64_t(row) >> 32), uint32_t(rng_seed), uint32_t(rng_seed >> 32));
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int src = (G / 4) * c + (g.l >> 2);
+    const uint32_t a0 = __shfl(w.w[0], src, G), a1 = __shfl(w.w[1], src, G);
+    const uint32_t a2 = __shfl(w.w[2], src, G), a3 = __shfl(w.w[3], src, G);
+    const uint32_t x = (g.l & 2) ? ((g.l & 1) ? a3 : a2) : ((g.l & 1) ? a1 : a0);
+    const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
+    ck[c] = p < end ? race_key(x, wt[c], uint32_t(p)) : kNoKey;
+  }
+}
+
+// Runs positions [begin, end) of the group's row, in steps of `stride` (begin and stride multiples
+// of 4 G), through its race.  `bars` (block-per-row kernel only) is the block's table of published
+// last keys.
 template <int G>
 __device__ __forceinline__ void race_scan(Race& r, const Group<G>& g, const TierView<float>& probs, int64_t start,
                                           uint64_t begin, uint64_t end, uint64_t stride, int k, uint64_t rng_seed,
@@ -233,28 +262,8 @@ __device__ __forceinline__ void race_scan(Race& r, const Group<G>& g, const Tier
   bool first = true;
   uint64_t published = kNoKey;
   for (uint64_t sb = begin; __ballot(sb < end); sb += stride) {
-    // the four steps of this stretch are independent until they meet the race: their loads are
-    // issued together and their key arithmetic (long dependent float64 chains) interleaves
-    float wt[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
-      wt[c] = p < end ? probs.at(start + int64_t(p)) : 0.0f;
-    }
-    PhiloxWords w{{0, 0, 0, 0}};
-    if (sb + 4u * uint32_t(g.l) < end)
-      w = philox4x32_10(0x80000000u | (uint32_t(sb >> 2) + uint32_t(g.l)), rng_stream, uint32_t(uint64_t(row)),
-                        uint32_t(uint64_t(row) >> 32), uint32_t(rng_seed), uint32_t(rng_seed >> 32));
     uint64_t ck[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int src = (G / 4) * c + (g.l >> 2);
-      const uint32_t a0 = __shfl(w.w[0], src, G), a1 = __shfl(w.w[1], src, G);
-      const uint32_t a2 = __shfl(w.w[2], src, G), a3 = __shfl(w.w[3], src, G);
-      const uint32_t x = (g.l & 2) ? ((g.l & 1) ? a3 : a2) : ((g.l & 1) ? a1 : a0);
-      const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
-      ck[c] = p < end ? race_key(x, wt[c], uint32_t(p)) : kNoKey;
-    }
+    stretch_keys<G>(g, probs, start, sb, end, rng_seed, rng_stream, row, ck);
     const uint64_t bar = bars != nullptr ? lowest_bar(bars, g.l) : kNoKey;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -273,6 +282,121 @@ __device__ __forceinline__ void race_scan(Race& r, const Group<G>& g, const Tier
       if (g.l == 0) __atomic_store_n(&bars[threadIdx.x / kWave], published, __ATOMIC_RELAXED);
     }
   }
+}
+
+// ---- the same race on the upper halves of the keys ----
+//
+// The upper 32 bits of a key (sign, exponent, 20 bits of the fraction) decide nearly every
+// comparison.  A group first races on them alone, at a fraction of the instructions of 64-bit
+// compare-and-move sequences, and keeps track of whether that was enough: it was unless two of the
+// kept halves are equal, or a candidate that was dropped (refused at the bar, cut after the first
+// sort, or pushed out) had the half that ends up as the bar.  Then, and only then, the row is
+// raced again on full (key, position) pairs.  Halves of unusable weights (0x7ff00000) tie with
+// each other, which only matters when they reach the kept entries.
+
+constexpr uint32_t kNoHalf = 0xffffffffu;  // upper half of kNoKey
+
+// Lane l < k holds the l-th smallest half and its position; lanes from k on hold leftovers that
+// nothing reads.
+struct HalfRace {
+  uint32_t key;
+  uint32_t pos;
+  uint32_t last;  // entry of lane k-1 (the bar)
+  uint32_t tie;   // the latest bar value that a dropped candidate shared (kNoHalf: none)
+};
+
+template <int G>
+__device__ __forceinline__ uint32_t group_read(uint32_t v, int src) {
+  if constexpr (G == kWave) return lane_read(v, src);
+  else return __shfl(v, src, G);
+}
+
+template <int G>
+__device__ __forceinline__ void half_race_seed(HalfRace& r, const Group<G>& g, uint32_t h, uint32_t p, int k) {
+  r.key = h;
+  r.pos = p;
+  group_sort<G, true>(r.key, r.pos, g.l);
+  r.last = group_read<G>(r.key, k - 1);
+  const uint32_t cut = group_read<G>(r.key, k < G ? k : G - 1);  // first entry that is dropped
+  r.tie = (k < G && cut == r.last) ? cut : kNoHalf;
+}
+
+// G more candidates: halves h, positions base + l.
+template <int G>
+__device__ __forceinline__ void half_race_offer(HalfRace& r, const Group<G>& g, uint32_t h, uint32_t base, int k) {
+  uint64_t hits = g.ballot(h < r.last);
+  if (g.ballot(h == r.last)) r.tie = r.last;
+  if constexpr (G == kWave) {
+    while (hits) {
+      const int b = __builtin_ctzll(hits);
+      hits &= hits - 1;
+      const uint32_t v = lane_read(h, b);
+      if (v >= r.last) {  // the bar moved since the ballot
+        if (v == r.last) r.tie = v;
+        continue;
+      }
+      const uint32_t pk = lane_below(r.key);
+      const uint32_t pp = lane_below(r.pos);
+      if (v < r.key) {  // an entry above the newcomer moves up or makes room
+        const bool shift = g.l > 0 && v < pk;
+        r.key = shift ? pk : v;
+        r.pos = shift ? pp : base + uint32_t(b);
+      }
+      const uint32_t pushed_out = r.last;
+      r.last = lane_read(r.key, k - 1);
+      if (r.last == pushed_out) r.tie = pushed_out;
+    }
+  } else {
+    while (__ballot(hits != 0)) {
+      const bool has = hits != 0;
+      const int b = has ? __builtin_ctzll(hits) : 0;
+      hits &= hits - 1;
+      const uint32_t v = __shfl(h, b, G);
+      const uint32_t pk = lane_below(r.key);
+      const uint32_t pp = lane_below(r.pos);
+      const bool in = has && v < r.last;
+      if (has && v == r.last) r.tie = v;
+      if (in && v < r.key) {
+        const bool shift = g.l > 0 && v < pk;
+        r.key = shift ? pk : v;
+        r.pos = shift ? pp : base + uint32_t(b);
+      }
+      const uint32_t pushed_out = r.last;
+      r.last = __shfl(r.key, k - 1, G);
+      if (in && r.last == pushed_out) r.tie = pushed_out;
+    }
+  }
+}
+
+// Positions [0, end) of the group's row through the race on halves.
+template <int G>
+__device__ __forceinline__ void half_race_scan(HalfRace& r, const Group<G>& g, const TierView<float>& probs,
+                                               int64_t start, uint64_t end, int k, uint64_t rng_seed,
+                                               uint32_t rng_stream, int64_t row) {
+  bool first = true;
+  for (uint64_t sb = 0; __ballot(sb < end); sb += 4u * G) {
+    uint64_t ck[4];
+    stretch_keys<G>(g, probs, start, sb, end, rng_seed, rng_stream, row, ck);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint64_t cb = sb + uint64_t(G) * c;
+      if (!__ballot(cb < end)) break;
+      const uint32_t h = uint32_t(ck[c] >> 32);
+      if (first) {
+        half_race_seed<G>(r, g, h, uint32_t(cb) + uint32_t(g.l), k);
+        first = false;
+      } else {
+        half_race_offer<G>(r, g, h, uint32_t(cb), k);
+      }
+    }
+  }
+}
+
+// Whether the halves left the group's winners or their order open.
+template <int G>
+__device__ __forceinline__ bool half_race_open(const HalfRace& r, const Group<G>& g, int k) {
+  const uint32_t below = lane_below(r.key);
+  return r.tie == r.last || g.ballot(g.l > 0 && g.l < k && r.key == below) != 0;
 }
 
 // ---- with replacement ----
@@ -364,13 +488,27 @@ struct LongRowScratch {
   float max[kLongWaves];
 };
 
-// Without replacement, a row of up to long_row<G>() positions raced by one G-lane group: on
-// return lane l < k of the group holds the l-th winner in r.pos (end = 0: nothing races).
+// Without replacement, a row of up to long_row<G>() positions raced by one G-lane group (end = 0:
+// nothing races): returns, in lane l < k of the group, the position of the l-th winner (kNoPos in
+// a group without a row).  Groups whose halves left something open race again on full keys; the
+// wave's other groups idle through that with empty candidates.
 template <int G>
-__device__ __forceinline__ void race_row(Race& r, const Group<G>& g, const TierView<float>& probs, int64_t start,
-                                         uint32_t end, int k, uint64_t rng_seed, uint32_t rng_stream, int64_t row) {
-  race_reset(r);
-  race_scan<G>(r, g, probs, start, 0, end, 4 * G, k, rng_seed, rng_stream, row);
+__device__ __forceinline__ uint32_t race_row(const Group<G>& g, const TierView<float>& probs, int64_t start,
+                                             uint32_t end, int k, uint64_t rng_seed, uint32_t rng_stream,
+                                             int64_t row) {
+  HalfRace hr;
+  hr.key = hr.last = hr.tie = kNoHalf;
+  hr.pos = kNoPos;
+  half_race_scan<G>(hr, g, probs, start, end, k, rng_seed, rng_stream, row);
+  const bool again = end > 0 && half_race_open<G>(hr, g, k);
+  uint32_t pos = end > 0 ? hr.pos : kNoPos;
+  if (__ballot(again)) {
+    Race r;
+    race_reset(r);
+    race_scan<G>(r, g, probs, start, 0, again ? end : 0u, 4 * G, k, rng_seed, rng_stream, row);
+    if (again) pos = r.pos;
+  }
+  return pos;
 }
 
 // Without replacement, a long row raced by a whole 1024-thread block: each wave races an

@@ -60,11 +60,10 @@ __global__ __launch_bounds__(kTile) void fill_weighted_kernel(const IdT* __restr
       }
     }
   }
-  Race r;
-  race_row<G>(r, g, probs, start, end, k, rng_seed, rng_stream, row);
-  if (end > 0 && g.l < k && r.pos < end) {  // a row that races has more than k positions: every entry is filled
+  const uint32_t pos = race_row<G>(g, probs, start, end, k, rng_seed, rng_stream, row);
+  if (end > 0 && g.l < k && pos < end) {  // a row that races has more than k positions: every entry is filled
     out_rows[off + g.l] = IdT(row);
-    out_cols[off + g.l] = indices.at(start + r.pos);
+    out_cols[off + g.l] = indices.at(start + pos);
   }
 }
 
