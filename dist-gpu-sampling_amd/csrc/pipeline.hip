@@ -286,12 +286,18 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
 
 // ---- weighted picks (race.h): one wave per seed row, a block per row for long rows ----
 
-constexpr int kWeightedRowsPerBlock = kBlock / kWave;
 constexpr int64_t kMaxLongGrid = 512;
 
-// One virtual block of the weighted fill launch: four seed rows, a wave each.  Rows above
-// long_row<64>() positions are queued for hop_fill_weighted_long_kernel, which fills their
-// positions; everything else about a row is what fill_rows does.
+// Lanes that one row's picks occupy when a wave writes them out: the wave races its rows one
+// after the other (64 lanes on a row), parks every row's picks in that row's lanes and then
+// inserts and records the picks of all its rows in one go, so that the instructions of that step
+// are not spent on a mostly idle wave.
+__host__ __device__ __forceinline__ int weighted_row_lanes(int64_t k) { return k <= 16 ? 16 : (k <= 32 ? 32 : kWave); }
+inline int64_t weighted_rows_per_block(int64_t k) { return (kBlock / kWave) * (kWave / weighted_row_lanes(k)); }
+
+// One virtual block of the weighted fill launch: four waves with 64 / weighted_row_lanes(k) seed
+// rows each.  Rows above long_row<64>() positions are queued for hop_fill_weighted_long_kernel,
+// which fills their positions; everything else about a row is what fill_rows does.
 template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
 __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, const TableT& table,
                                                    const TierView<PtrT>& indptr, const TierView<IdT>& indices,
@@ -299,44 +305,59 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
   const Group<kWave> g;
   const int64_t s = seeds_of(h);
   if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
-  // the row and everything read for it are the same in all 64 lanes: keep them in scalar registers
-  const int64_t i = vb * kWeightedRowsPerBlock + int64_t(wave_uniform(uint32_t(threadIdx.x / kWave)));
-  if (i >= s) return;  // whole waves leave together
-  const IdT seed = IdT(wave_uniform(int64_t(static_cast<const IdT*>(h.seeds)[i])));
-  const int64_t row = int64_t(seed);
-  const int64_t b = wave_uniform(int64_t(indptr.at(row)));
-  const int64_t deg64 = wave_uniform(int64_t(indptr.at(row + 1))) - b;
-  const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
-  const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;
+  const int lanes = weighted_row_lanes(k);
+  const int rows = kWave / lanes;
+  const int64_t first = (vb * (kBlock / kWave) + int64_t(wave_uniform(uint32_t(threadIdx.x / kWave)))) * rows;
+  if (first >= s) return;  // whole waves leave together
+  // every lane looks up the row whose picks it will write out
+  const int mine = g.l / lanes;  // that row among the wave's
+  const int l = g.l - mine * lanes;
+  const int64_t i = first + mine;
+  int64_t b = 0;
+  uint32_t deg = 0;
+  bool bad = false;
+  IdT seed = 0;
+  if (i < s) {
+    seed = static_cast<const IdT*>(h.seeds)[i];
+    b = int64_t(indptr.at(int64_t(seed)));
+    const int64_t deg64 = int64_t(indptr.at(int64_t(seed) + 1)) - b;
+    bad = deg64 < 0 || deg64 > 0xffffffffLL;
+    deg = bad ? 0u : uint32_t(deg64);
+  }
   const bool look_first = look_before_insert(h, s);
-  if (g.l == 0) {
+  if (i < s && l == 0) {
     h.row_cnt[i] = bad ? kBadRow : (REPLACE ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
     if (h.index == 0) {
-      bool first;
+      bool first_seen;
       uint32_t displaced;
-      h.slot[h.pos_base + i] = table.insert_min(seed, uint32_t(h.pos_base + i), &first, &displaced);
+      h.slot[h.pos_base + i] = table.insert_min(seed, uint32_t(h.pos_base + i), &first_seen, &displaced);
     }
   }
-  const int64_t p0 = h.pos_base + seed_part(h, s) + i * k;
-  if (deg == 0) {
-    if (g.l < k) h.slot[p0 + g.l] = kInvalidSlot;
-    return;
+  // rows that are copied need no work; long rows are queued and written by the other launch
+  const bool is_long = deg > long_row<kWave>() && (REPLACE || deg > uint32_t(k));
+  if (is_long && l == 0) h.long_rows[atomicAdd(reinterpret_cast<unsigned long long*>(h.long_count), 1ull)] = i;
+  uint32_t pick = uint32_t(l);  // what a copied row keeps: its positions in order
+  for (int r = 0; r < rows; ++r) {
+    // row r of the wave, in scalar registers
+    const int src = r * lanes;
+    const uint32_t rdeg = lane_read(deg, src);
+    const bool rlong = rdeg > long_row<kWave>() && (REPLACE || rdeg > uint32_t(k));
+    if (rdeg == 0 || rlong || (!REPLACE && rdeg <= uint32_t(k))) continue;
+    const int64_t rrow = int64_t(lane_read(uint64_t(int64_t(seed)), src));
+    const int64_t rb = int64_t(lane_read(uint64_t(b), src));
+    uint32_t won = kNoPos;  // lane j: pick j of this row
+    if (REPLACE) {  // at most 64 draws: draw j is found by lane j
+      draw_row<kWave>(g, probs, rb, int64_t(rdeg), int64_t(k), rng_seed, h.rng_stream, rrow,
+                      [&](int64_t, int64_t at) { won = uint32_t(at); });
+    } else {
+      won = race_row<kWave>(g, probs, rb, rdeg, k, rng_seed, h.rng_stream, rrow);
+    }
+    const uint32_t parked = __shfl(won, l, kWave);
+    if (mine == r) pick = parked;
   }
-  if (deg > long_row<kWave>() && (REPLACE || deg > uint32_t(k))) {
-    if (g.l == 0) h.long_rows[atomicAdd(reinterpret_cast<unsigned long long*>(h.long_count), 1ull)] = i;
-    return;
-  }
-  if (REPLACE) {
-    draw_row<kWave>(g, probs, b, int64_t(deg), int64_t(k), rng_seed, h.rng_stream, row, [&](int64_t j, int64_t pick) {
-      emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first);
-    });
-  } else if (deg <= uint32_t(k)) {
-    if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, uint32_t(g.l) < deg, b + g.l, look_first);
-  } else {
-    const uint32_t pos = race_row<kWave>(g, probs, b, deg, k, rng_seed, h.rng_stream, row);
-    if (g.l < k) emit_pick<IdT>(h, table, indices, p0 + g.l, pos < deg, b + pos, look_first);
-  }
+  if (i < s && l < k && !is_long)
+    emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, pick < deg, b + pick, look_first);
 }
 
 // Same layout of virtual blocks as hop_fill_kernel (fill, previous hop's edge list, clearing).
@@ -638,7 +659,8 @@ template <typename IdT, typename PtrT, typename TableT, bool REPLACE>
 dgs_status launch_fill_weighted(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* clear_begin,
                                 int64_t clear_n16, const TableT& table, const dgs_view& indptr,
                                 const dgs_view& indices, const dgs_view& probs, uint64_t rng_seed, hipStream_t st) {
-  const int64_t fill_blocks = (cur.s_max + kWeightedRowsPerBlock - 1) / kWeightedRowsPerBlock;
+  const int64_t rows_per_block = weighted_rows_per_block(cur.k);
+  const int64_t fill_blocks = (cur.s_max + rows_per_block - 1) / rows_per_block;
   const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
   const int64_t total = fill_blocks + relabel_count + clear_blocks;
   hipLaunchKernelGGL((hop_fill_weighted_kernel<IdT, PtrT, TableT, REPLACE>), dim3(capped_grid(total)), dim3(kBlock),
