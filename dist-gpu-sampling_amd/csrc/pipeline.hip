@@ -402,10 +402,9 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
       draw_long_row(lds, probs, b, int64_t(deg), int64_t(k), rng_seed, h.rng_stream, row,
                     [&](int64_t j, int64_t pick) { emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first); });
     } else {
-      Race r;
-      race_long_row(r, lds, probs, b, deg, k, rng_seed, h.rng_stream, row);
+      const uint32_t pos = race_long_row(lds, probs, b, deg, k, rng_seed, h.rng_stream, row);
       const int l = threadIdx.x;  // wave 0 holds the winners
-      if (l < k) emit_pick<IdT>(h, table, indices, p0 + l, r.pos < deg, b + r.pos, look_first);
+      if (l < k) emit_pick<IdT>(h, table, indices, p0 + l, pos < deg, b + pos, look_first);
     }
   }
 }

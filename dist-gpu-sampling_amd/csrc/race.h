@@ -222,21 +222,25 @@ __device__ __forceinline__ uint64_t lowest_bar_after_sync(uint64_t* bars, int la
   return lowest_bar(bars, lane);
 }
 
-// Race keys of the four G-position steps of the stretch that begins at position sb (a multiple of
-// 4 G) of the group's row, kNoKey from `end` on: one Philox block per lane covers the stretch
-// (four words each), the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the
-// group.  The four steps are independent: their loads are issued together and their key
-// arithmetic (long dependent float64 chains) interleaves.
+// Weights of the four G-position steps of the stretch that begins at position sb (a multiple of
+// 4 G) of the group's row, 0 from `end` on.
 template <int G>
-__device__ __forceinline__ void stretch_keys(const Group<G>& g, const TierView<float>& probs, int64_t start,
-                                             uint64_t sb, uint64_t end, uint64_t rng_seed, uint32_t rng_stream,
-                                             int64_t row, uint64_t ck[4]) {
-  float wt[4];
+__device__ __forceinline__ void stretch_weights(const Group<G>& g, const TierView<float>& probs, int64_t start,
+                                                uint64_t sb, uint64_t end, float wt[4]) {
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
     wt[c] = p < end ? probs.at(start + int64_t(p)) : 0.0f;
   }
+}
+
+// Race keys of that stretch, kNoKey from `end` on: one Philox block per lane covers the stretch
+// (four words each), the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the
+// group.  The four steps are independent: their key arithmetic (long dependent float64 chains)
+// interleaves.
+template <int G>
+__device__ __forceinline__ void stretch_keys(const Group<G>& g, const float wt[4], uint64_t sb, uint64_t end,
+                                             uint64_t rng_seed, uint32_t rng_stream, int64_t row, uint64_t ck[4]) {
   PhiloxWords w{{0, 0, 0, 0}};
   if (sb + 4u * uint32_t(g.l) < end)
     w = philox4x32_10(0x80000000u | (uint32_t(sb >> 2) + uint32_t(g.l)), rng_stream, uint32_t(uint64_t(row)),
@@ -250,6 +254,15 @@ __device__ __forceinline__ void stretch_keys(const Group<G>& g, const TierView<f
     const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
     ck[c] = p < end ? race_key(x, wt[c], uint32_t(p)) : kNoKey;
   }
+}
+
+template <int G>
+__device__ __forceinline__ void stretch_keys(const Group<G>& g, const TierView<float>& probs, int64_t start,
+                                             uint64_t sb, uint64_t end, uint64_t rng_seed, uint32_t rng_stream,
+                                             int64_t row, uint64_t ck[4]) {
+  float wt[4];
+  stretch_weights<G>(g, probs, start, sb, end, wt);
+  stretch_keys<G>(g, wt, sb, end, rng_seed, rng_stream, row, ck);
 }
 
 // Runs positions [begin, end) of the group's row, in steps of `stride` (begin and stride multiples
@@ -305,6 +318,11 @@ struct HalfRace {
   uint32_t tie;   // the latest bar value that a dropped candidate shared (kNoHalf: none)
 };
 
+__device__ __forceinline__ void half_race_reset(HalfRace& r) {
+  r.key = r.last = r.tie = kNoHalf;
+  r.pos = kNoPos;
+}
+
 template <int G>
 __device__ __forceinline__ uint32_t group_read(uint32_t v, int src) {
   if constexpr (G == kWave) return lane_read(v, src);
@@ -321,9 +339,9 @@ __device__ __forceinline__ void half_race_seed(HalfRace& r, const Group<G>& g, u
   r.tie = (k < G && cut == r.last) ? cut : kNoHalf;
 }
 
-// G more candidates: halves h, positions base + l.
+// G more candidates: halves h, positions p.
 template <int G>
-__device__ __forceinline__ void half_race_offer(HalfRace& r, const Group<G>& g, uint32_t h, uint32_t base, int k) {
+__device__ __forceinline__ void half_race_offer(HalfRace& r, const Group<G>& g, uint32_t h, uint32_t p, int k) {
   uint64_t hits = g.ballot(h < r.last);
   if (g.ballot(h == r.last)) r.tie = r.last;
   if constexpr (G == kWave) {
@@ -340,7 +358,7 @@ __device__ __forceinline__ void half_race_offer(HalfRace& r, const Group<G>& g, 
       if (v < r.key) {  // an entry above the newcomer moves up or makes room
         const bool shift = g.l > 0 && v < pk;
         r.key = shift ? pk : v;
-        r.pos = shift ? pp : base + uint32_t(b);
+        r.pos = shift ? pp : lane_read(p, b);
       }
       const uint32_t pushed_out = r.last;
       r.last = lane_read(r.key, k - 1);
@@ -352,6 +370,7 @@ __device__ __forceinline__ void half_race_offer(HalfRace& r, const Group<G>& g, 
       const int b = has ? __builtin_ctzll(hits) : 0;
       hits &= hits - 1;
       const uint32_t v = __shfl(h, b, G);
+      const uint32_t vp = __shfl(p, b, G);
       const uint32_t pk = lane_below(r.key);
       const uint32_t pp = lane_below(r.pos);
       const bool in = has && v < r.last;
@@ -359,7 +378,7 @@ __device__ __forceinline__ void half_race_offer(HalfRace& r, const Group<G>& g, 
       if (in && v < r.key) {
         const bool shift = g.l > 0 && v < pk;
         r.key = shift ? pk : v;
-        r.pos = shift ? pp : base + uint32_t(b);
+        r.pos = shift ? pp : vp;
       }
       const uint32_t pushed_out = r.last;
       r.last = __shfl(r.key, k - 1, G);
@@ -382,11 +401,12 @@ __device__ __forceinline__ void half_race_scan(HalfRace& r, const Group<G>& g, c
       const uint64_t cb = sb + uint64_t(G) * c;
       if (!__ballot(cb < end)) break;
       const uint32_t h = uint32_t(ck[c] >> 32);
+      const uint32_t p = uint32_t(cb) + uint32_t(g.l);
       if (first) {
-        half_race_seed<G>(r, g, h, uint32_t(cb) + uint32_t(g.l), k);
+        half_race_seed<G>(r, g, h, p, k);
         first = false;
       } else {
-        half_race_offer<G>(r, g, h, uint32_t(cb), k);
+        half_race_offer<G>(r, g, h, p, k);
       }
     }
   }
@@ -482,10 +502,15 @@ __device__ __forceinline__ uint64_t locate_draws(const Group<G>& g, const TierVi
 // LDS of a block that works on long rows.
 struct LongRowScratch {
   uint64_t key[kLongBlock];
+  uint32_t half[kLongBlock];
   uint32_t pos[kLongBlock];
   uint64_t bars[kLongWaves];
   uint64_t sum[kLongWaves];
   float max[kLongWaves];
+  uint32_t half_bars[kLongWaves];
+  uint32_t ties[kLongWaves];
+  uint32_t listed;  // entries of half[] / pos[]
+  uint32_t open;    // the halves did not settle the row
 };
 
 // Without replacement, a row of up to long_row<G>() positions raced by one G-lane group (end = 0:
@@ -497,8 +522,7 @@ __device__ __forceinline__ uint32_t race_row(const Group<G>& g, const TierView<f
                                              uint32_t end, int k, uint64_t rng_seed, uint32_t rng_stream,
                                              int64_t row) {
   HalfRace hr;
-  hr.key = hr.last = hr.tie = kNoHalf;
-  hr.pos = kNoPos;
+  half_race_reset(hr);
   half_race_scan<G>(hr, g, probs, start, end, k, rng_seed, rng_stream, row);
   const bool again = end > 0 && half_race_open<G>(hr, g, k);
   uint32_t pos = end > 0 ? hr.pos : kNoPos;
@@ -511,14 +535,14 @@ __device__ __forceinline__ uint32_t race_row(const Group<G>& g, const TierView<f
   return pos;
 }
 
-// Without replacement, a long row raced by a whole 1024-thread block: each wave races an
-// interleaved share of the row, then the waves' winners are merged pairwise (wave w takes over the
-// entries of wave w + step: 16 lists become one in four rounds; entries beyond the lowest
+// Without replacement, a long row raced by a whole 1024-thread block on full keys: each wave
+// races an interleaved share of the row, then the waves' winners are merged pairwise (wave w takes
+// over the entries of wave w + step: 16 lists become one in four rounds; entries beyond the lowest
 // published bar cannot be among the row's best).  On return lane l < k of wave 0 holds the l-th
 // winner in r.pos.  Every thread of the block must call it.
-__device__ __forceinline__ void race_long_row(Race& r, LongRowScratch& lds, const TierView<float>& probs,
-                                              int64_t start, uint32_t deg, int k, uint64_t rng_seed,
-                                              uint32_t rng_stream, int64_t row) {
+__device__ __forceinline__ void race_long_row_full(Race& r, LongRowScratch& lds, const TierView<float>& probs,
+                                                   int64_t start, uint32_t deg, int k, uint64_t rng_seed,
+                                                   uint32_t rng_stream, int64_t row) {
   const Group<kWave> g;
   const int wave = threadIdx.x / kWave;
   if (threadIdx.x < kLongWaves) lds.bars[threadIdx.x] = kNoKey;
@@ -536,6 +560,100 @@ __device__ __forceinline__ void race_long_row(Race& r, LongRowScratch& lds, cons
     }
     __syncthreads();  // the arrays are rewritten by the next round and by the block's next row
   }
+}
+
+__device__ __forceinline__ uint32_t lowest_half_bar(uint32_t* bars, int lane) {
+  uint32_t v = __atomic_load_n(&bars[lane & (kLongWaves - 1)], __ATOMIC_RELAXED);
+#pragma unroll
+  for (int stride = 1; stride < kLongWaves; stride <<= 1) {
+    const uint32_t o = lane_xor(v, stride);
+    if (o < v) v = o;
+  }
+  return v;
+}
+
+// Without replacement, a long row raced by a whole 1024-thread block (every thread must call it):
+// returns, in lane l < k of wave 0, the position of the l-th winner.  The race runs on key halves
+// first.  Each wave races an interleaved share of the row and publishes its bar, which lets all
+// of them drop candidates beyond the lowest bar unseen; the entries that survive the final lowest
+// bar (between k and 16 k, usually close to k) are listed in LDS and raced by wave 0.  Whether the
+// halves settled the row is judged as in a group's race, with every wave's record of ties at its
+// bar taken into account: a dropped candidate can only share the final bar if it shared its own
+// wave's bar when it was dropped.  An unsettled row is raced again on full keys.
+__device__ __forceinline__ uint32_t race_long_row(LongRowScratch& lds, const TierView<float>& probs, int64_t start,
+                                                  uint32_t deg, int k, uint64_t rng_seed, uint32_t rng_stream,
+                                                  int64_t row) {
+  const Group<kWave> g;
+  const int wave = threadIdx.x / kWave;
+  if (threadIdx.x < kLongWaves) lds.half_bars[threadIdx.x] = kNoHalf;
+  if (threadIdx.x == 0) lds.listed = 0;
+  __syncthreads();
+  HalfRace r;
+  half_race_reset(r);
+  bool first = true;
+  uint32_t published = kNoHalf;
+  for (uint64_t sb = 256u * wave; __ballot(sb < deg); sb += 256u * kLongWaves) {
+    uint64_t ck[4];
+    stretch_keys<kWave>(g, probs, start, sb, deg, rng_seed, rng_stream, row, ck);
+    const uint32_t bar = lowest_half_bar(lds.half_bars, g.l);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint64_t cb = sb + uint64_t(kWave) * c;
+      if (!__ballot(cb < deg)) break;
+      const uint32_t h = uint32_t(ck[c] >> 32);
+      const uint32_t p = uint32_t(cb) + uint32_t(g.l);
+      if (first) {
+        half_race_seed<kWave>(r, g, h, p, k);
+        first = false;
+      } else {
+        half_race_offer<kWave>(r, g, h > bar ? kNoHalf : h, p, k);
+      }
+    }
+    if (r.last < published) {
+      published = r.last;
+      if (g.l == 0) __atomic_store_n(&lds.half_bars[wave], published, __ATOMIC_RELAXED);
+    }
+  }
+  if (g.l == 0) lds.ties[wave] = r.tie;
+  __syncthreads();  // every wave has published its final bar
+  const uint32_t bar = lowest_half_bar(lds.half_bars, g.l);
+  {
+    const bool keep = g.l < k && r.key <= bar;  // a wave that raced nothing holds kNoHalf only
+    const uint64_t kept = __ballot(keep);
+    uint32_t base = 0;
+    if (g.l == 0 && kept) base = atomicAdd(&lds.listed, uint32_t(__builtin_popcountll(kept)));
+    base = wave_uniform(base);
+    if (keep) {
+      const uint32_t at = base + uint32_t(__builtin_popcountll(kept & ((uint64_t(1) << g.l) - 1)));
+      lds.half[at] = r.key;
+      lds.pos[at] = r.pos;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const uint32_t listed = lds.listed;
+    half_race_reset(r);
+    for (uint32_t cb = 0; cb < listed; cb += kWave) {
+      const uint32_t at = cb + uint32_t(g.l);
+      const uint32_t h = at < listed ? lds.half[at] : kNoHalf;
+      const uint32_t p = at < listed ? lds.pos[at] : kNoPos;
+      if (cb == 0) half_race_seed<kWave>(r, g, h, p, k);
+      else half_race_offer<kWave>(r, g, h, p, k);
+    }
+    const bool dropped_at_bar = __ballot(g.l < kLongWaves && lds.ties[g.l & (kLongWaves - 1)] == r.last) != 0;
+    const bool open = half_race_open<kWave>(r, g, k) || dropped_at_bar;
+    if (g.l == 0) lds.open = open ? 1u : 0u;
+  }
+  __syncthreads();
+  const bool again = lds.open != 0;
+  __syncthreads();  // lds.open and the lists are rewritten by the block's next row
+  uint32_t pos = wave == 0 ? r.pos : kNoPos;
+  if (again) {
+    Race full;
+    race_long_row_full(full, lds, probs, start, deg, k, rng_seed, rng_stream, row);
+    pos = wave == 0 ? full.pos : kNoPos;
+  }
+  return pos;
 }
 
 // With replacement, a row of up to long_row<G>() positions (deg = 0: nothing to draw) handled by

@@ -83,12 +83,11 @@ __global__ __launch_bounds__(kLongBlock) void fill_weighted_long_kernel(const Id
     const int64_t off = a.tile_off[i / kTile] + a.row_off[i];
     const int64_t row = int64_t(seeds[i]);
     const uint32_t deg = a.row_deg[i];
-    Race r;
-    race_long_row(r, lds, probs, start, deg, k, rng_seed, rng_stream, row);
+    const uint32_t pos = race_long_row(lds, probs, start, deg, k, rng_seed, rng_stream, row);
     const int l = threadIdx.x;
-    if (l < k && r.pos < deg) {  // wave 0 holds the winners; deg > k: every entry is filled
+    if (l < k && pos < deg) {  // wave 0 holds the winners; deg > k: every entry is filled
       out_rows[off + l] = IdT(row);
-      out_cols[off + l] = indices.at(start + r.pos);
+      out_cols[off + l] = indices.at(start + pos);
     }
   }
 }
