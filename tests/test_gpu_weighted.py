@@ -246,3 +246,41 @@ def test_weighted_fused_long_rows_and_wide_fanout(pkg, oracle):
         assert np.array_equal(_np(f), want_f), (fanouts, replace)
         for g, w in zip(blocks, want_blocks):
             assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
+
+
+def test_weighted_rows_that_the_key_halves_leave_open(pkg, oracle):
+    # the race first compares the upper 32 bits of the keys and repeats a row on full keys when
+    # those tie where it matters: infinite weights (all keys 0), fewer usable weights than picks
+    # (the unusable ones tie), on rows served by a lane group, by a wave and by a whole block;
+    # plus ordinary rows sharing their waves with such rows
+    rng = np.random.default_rng(12)
+    deg = np.array([40, 300, 1500, 2500, 6000, 18000] * 3 + [30, 50, 64, 65, 200, 33, 17, 90])
+    n = deg.size
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, n, size=int(indptr[-1])).astype(np.int64)
+    probs = (rng.random(indices.size) + 0.01).astype(np.float32)
+    for row in range(0, 6):          # every third weight infinite
+        probs[indptr[row]:indptr[row + 1]:3] = np.inf
+    for row in range(6, 12):         # three usable weights near the end of the row
+        probs[indptr[row]:indptr[row + 1]] = 0.0
+        probs[indptr[row + 1] - 9:indptr[row + 1]:3] = 1.5
+    for row in range(12, 18):        # usable weights only in the first 64 positions, fewer than some fanouts
+        probs[indptr[row] + 20:indptr[row + 1]] = np.nan
+    seeds = rng.permutation(n).astype(np.int64)
+    capi = pkg.capi
+    ip, ix, pr = _dev(indptr), _dev(indices), _dev(probs)
+    for k in (2, 7, 16, 31, 64):
+        want_r, want_c = oracle.sample_neighbors_weighted(seeds, indptr, indices, probs, k, False, 5, 2)
+        r, c, _ = capi.sample_neighbors_weighted(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix),
+                                                 capi.tensor_view(pr), k, False, 5, 2)
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c), k
+    big = 1 << 40
+    cts = [pkg.create_chunktensor(torch.from_numpy(a), 1, big) for a in (indptr, indices, probs)]
+    for fanouts in ([7, 3], [33], [16, 2]):
+        pkg.set_rng_state(1234, 3)
+        sampler = pkg.ChunkTensorSampler(fanouts, cts[0], cts[1], cts[2], False)
+        f, _, blocks = sampler.sample_blocks(None, torch.from_numpy(seeds))
+        want_f, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, False, 1234, 3, probs=probs)
+        assert np.array_equal(_np(f), want_f), fanouts
+        for g, w in zip(blocks, want_blocks):
+            assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
