@@ -62,27 +62,6 @@ std::vector<int64_t> read_back(const torch::Tensor& dev, int64_t count) {
   return std::vector<int64_t>(p, p + count);
 }
 
-// The same read split around other launches: the copy is enqueued now, the host waits later.
-struct PendingRead {
-  void* ticket = nullptr;
-  int64_t count = 0;
-  const int64_t* host = nullptr;
-  std::vector<int64_t> wait() {
-    check(dgs_read_back_wait(ticket));
-    return std::vector<int64_t>(host, host + count);
-  }
-};
-PendingRead read_back_begin(const torch::Tensor& dev, int64_t count) {
-  thread_local torch::Tensor pinned =
-      torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-  TORCH_CHECK(count <= 32);
-  PendingRead r;
-  r.count = count;
-  r.host = pinned.data_ptr<int64_t>();
-  check(dgs_read_back_begin(pinned.data_ptr(), dev.data_ptr(), sizeof(int64_t) * count, current_stream(), &r.ticket));
-  return r;
-}
-
 // ---- generator state for the sampling ops ------------------------------------
 std::mutex g_rng_mutex;
 uint64_t g_rng_seed = 7777;  // upstream's constant, used until the caller sets one
