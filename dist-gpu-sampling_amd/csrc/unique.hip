@@ -5,8 +5,9 @@
 // a "first occurrence" when the table holds exactly that position.  Flags are
 // scanned tile by tile, first occurrences are compacted in input order (which is
 // what makes the result independent of the table layout) and the table value
-// becomes the id's rank.  Every key remembers its slot, so only ids that were
-// not part of the mapping list are probed a second time.
+// becomes the id's rank.  Every mapping id remembers its slot, so a tensor that
+// is both mapped and relabelled (the picked neighbours of the upstream sampler
+// loop) is not probed a second time.
 #include "common.h"
 #include "table.h"
 
@@ -35,23 +36,6 @@ __device__ __forceinline__ IdT seg_load(const dgs_segments& s, int64_t i) {
     }
   }
   return p[j];
-}
-
-template <typename IdT>
-__device__ __forceinline__ void seg_store(const dgs_segments& s, int64_t i, IdT v) {
-  IdT* p = static_cast<IdT*>(const_cast<void*>(s.ptr[0]));
-  int64_t j = i;
-#pragma unroll
-  for (int k = 1; k < DGS_MAX_SEGMENTS; ++k) {
-    if (k < s.count && i >= s.len[k - 1]) {
-      i -= s.len[k - 1];
-      p = static_cast<IdT*>(const_cast<void*>(s.ptr[k]));
-      j = i;
-    } else {
-      i = -1;
-    }
-  }
-  p[j] = v;
 }
 
 __global__ __launch_bounds__(kThreads) void fill_ones_kernel(uint4* __restrict__ p, int64_t n16) {
@@ -123,14 +107,36 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(dgs_segments mapping,
   }
 }
 
+// Where element i of a segment list lives: its segment and its offset inside it.
+__device__ __forceinline__ void seg_locate(const dgs_segments& s, int64_t i, int* seg, int64_t* off) {
+  int k = 0;
+  while (k + 1 < s.count && i >= s.len[k]) {
+    i -= s.len[k];
+    ++k;
+  }
+  *seg = k;
+  *off = i;
+}
+
+// Mapping positions of the requiring segments that are mapping segments themselves (-1: not one).
+struct SegmentAlias {
+  int64_t mapping_begin[DGS_MAX_SEGMENTS];
+};
+
 // out[j] = rank of requiring[j], -1 when the id is not in the table.
 template <typename IdT, typename TableT>
 __global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring, int64_t m, TableT table,
+                                                          const uint32_t* __restrict__ slot, SegmentAlias alias,
                                                           dgs_segments out) {
   const int64_t j = int64_t(blockIdx.x) * kThreads + threadIdx.x;
   if (j >= m) return;
-  const uint32_t s = table.find(seg_load<IdT>(requiring, j));
-  seg_store<IdT>(out, j, s > table.mask ? IdT(-1) : IdT(table.value(s)));
+  int seg;
+  int64_t off;
+  seg_locate(requiring, j, &seg, &off);
+  uint32_t s;
+  if (alias.mapping_begin[seg] >= 0) s = slot[alias.mapping_begin[seg] + off] & ~kFirstBit;
+  else s = table.find(static_cast<const IdT*>(requiring.ptr[seg])[off]);
+  static_cast<IdT*>(const_cast<void*>(out.ptr[seg]))[off] = s > table.mask ? IdT(-1) : IdT(table.value(s));
 }
 
 struct UniqueWorkspace {
@@ -193,8 +199,18 @@ dgs_status run_unique_relabel(const dgs_segments& mapping, int64_t n, const dgs_
     DGS_LAUNCH_CHECK();
   }
   if (m > 0) {
+    SegmentAlias alias;
+    for (int r = 0; r < DGS_MAX_SEGMENTS; ++r) {
+      alias.mapping_begin[r] = -1;
+      int64_t begin = 0;
+      for (int k = 0; k < mapping.count && r < requiring.count; ++k) {
+        if (requiring.len[r] > 0 && mapping.ptr[k] == requiring.ptr[r] && mapping.len[k] == requiring.len[r])
+          alias.mapping_begin[r] = begin;
+        begin += mapping.len[k];
+      }
+    }
     hipLaunchKernelGGL((lookup_kernel<IdT, TableT>), dim3(uint32_t((m + kThreads - 1) / kThreads)), dim3(kThreads),
-                       0, st, requiring, m, table, out);
+                       0, st, requiring, m, table, w.slot, alias, out);
     DGS_LAUNCH_CHECK();
   }
   return DGS_OK;

@@ -143,6 +143,13 @@ def test_unique_relabel_parity(pkg, oracle, dtype, n, hi):
     u2, outs = pkg.ops._CAPI_tensor_relabel([_dev(seeds), _dev(cols)], [_dev(rows), _dev(cols), _dev(extra)])
     assert np.array_equal(_np(u2), want_u) and np.array_equal(_np(outs[1]), want_c)
     assert _np(outs[2]).tolist() == [-1] and outs[0].dtype == _dev(rows).dtype
+    # the same device tensor on both sides, as the upstream loop passes its picked neighbours
+    # (their slots are reused instead of probed again), next to a shorter view of it
+    d_seeds, d_cols = _dev(seeds), _dev(cols)
+    u3, outs3 = pkg.ops._CAPI_tensor_relabel([d_seeds, d_cols], [d_cols, _dev(rows), d_cols[: n // 2], d_seeds])
+    assert np.array_equal(_np(u3), want_u) and np.array_equal(_np(outs3[0]), want_c)
+    assert np.array_equal(_np(outs3[1]), want_r) and np.array_equal(_np(outs3[2]), want_c[: n // 2])
+    assert np.array_equal(_np(outs3[3]), np.arange(seeds.size))
 
 
 def test_unique_many_segments(pkg, oracle):
