@@ -125,3 +125,15 @@ def test_placement_host_arithmetic(oracle):
     assert pl.expected_hit_rate(d, 2) == 0.8 and pl.expected_hit_rate(torch.zeros(3), 1) == 0.0
     with pytest.raises(ValueError):
         pl.degree_order(indptr, by="sideways")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # the benchmark measures one GPU; asking for more ends with a message, before any GPU work
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for argv, env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "4"})):
+        p = subprocess.run([sys.executable, os.path.join(root, "bench.py")] + argv, capture_output=True, text=True,
+                           env={**os.environ, **env}, timeout=120)
+        assert p.returncode != 0 and "ONE GPU" in p.stderr and p.stdout.strip() == ""
