@@ -259,9 +259,10 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
   torch::Tensor ws = device_bytes(ws_bytes, seeds.device());
   torch::Tensor nnz_dev = torch::empty({2}, seeds.options().dtype(torch::kInt64));
 
-  // Worst case n * num_picks ids per output: when that is modest the whole hop is
-  // enqueued before the one blocking length read; otherwise count first.
-  const bool one_shot = num_picks <= (int64_t(1) << 20) && n * num_picks <= (int64_t(1) << 28);
+  // Worst case n * num_picks ids per output: when that is modest (two buffers of at most 256 MB,
+  // of which the results are prefixes) the whole hop is enqueued before the one blocking length
+  // read; otherwise count first and allocate exactly.
+  const bool one_shot = num_picks <= (int64_t(1) << 20) && n * num_picks <= (int64_t(1) << 25);
   torch::Tensor rows, cols;
   std::vector<int64_t> len;
   if (one_shot) {
