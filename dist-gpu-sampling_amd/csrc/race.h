@@ -222,25 +222,21 @@ __device__ __forceinline__ uint64_t lowest_bar_after_sync(uint64_t* bars, int la
   return lowest_bar(bars, lane);
 }
 
-// Weights of the four G-position steps of the stretch that begins at position sb (a multiple of
-// 4 G) of the group's row, 0 from `end` on.
+// Race keys of the four G-position steps of the stretch that begins at position sb (a multiple of
+// 4 G) of the group's row, kNoKey from `end` on: one Philox block per lane covers the stretch
+// (four words each), the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the
+// group.  The four steps are independent: their loads are issued together and their key
+// arithmetic (long dependent float64 chains) interleaves.
 template <int G>
-__device__ __forceinline__ void stretch_weights(const Group<G>& g, const TierView<float>& probs, int64_t start,
-                                                uint64_t sb, uint64_t end, float wt[4]) {
+__device__ __forceinline__ void stretch_keys(const Group<G>& g, const TierView<float>& probs, int64_t start,
+                                             uint64_t sb, uint64_t end, uint64_t rng_seed, uint32_t rng_stream,
+                                             int64_t row, uint64_t ck[4]) {
+  float wt[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
     wt[c] = p < end ? probs.at(start + int64_t(p)) : 0.0f;
   }
-}
-
-// Race keys of that stretch, kNoKey from `end` on: one Philox block per lane covers the stretch
-// (four words each), the word of position sb + G c + l sits in lane (G / 4) c + l / 4 of the
-// group.  The four steps are independent: their key arithmetic (long dependent float64 chains)
-// interleaves.
-template <int G>
-__device__ __forceinline__ void stretch_keys(const Group<G>& g, const float wt[4], uint64_t sb, uint64_t end,
-                                             uint64_t rng_seed, uint32_t rng_stream, int64_t row, uint64_t ck[4]) {
   PhiloxWords w{{0, 0, 0, 0}};
   if (sb + 4u * uint32_t(g.l) < end)
     w = philox4x32_10(0x80000000u | (uint32_t(sb >> 2) + uint32_t(g.l)), rng_stream, uint32_t(uint64_t(row)),
@@ -254,15 +250,6 @@ __device__ __forceinline__ void stretch_keys(const Group<G>& g, const float wt[4
     const uint64_t p = sb + uint64_t(G) * c + uint32_t(g.l);
     ck[c] = p < end ? race_key(x, wt[c], uint32_t(p)) : kNoKey;
   }
-}
-
-template <int G>
-__device__ __forceinline__ void stretch_keys(const Group<G>& g, const TierView<float>& probs, int64_t start,
-                                             uint64_t sb, uint64_t end, uint64_t rng_seed, uint32_t rng_stream,
-                                             int64_t row, uint64_t ck[4]) {
-  float wt[4];
-  stretch_weights<G>(g, probs, start, sb, end, wt);
-  stretch_keys<G>(g, wt, sb, end, rng_seed, rng_stream, row, ck);
 }
 
 // Runs positions [begin, end) of the group's row, in steps of `stride` (begin and stride multiples
