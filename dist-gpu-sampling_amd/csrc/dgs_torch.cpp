@@ -179,11 +179,14 @@ class ChunkTensor : public torch::CustomClassHolder {
   // (one entry per node).  Created on first use; returns (pointer, epoch for this call).
   // Calls in flight on different streams must not share a table, so there is one per stream
   // (up to kMaxNodeTables; further streams get none and the call uses a hash table instead).
+  // Two calls on the same stream share their table one after the other, which is only right if
+  // all launches of the first precede all launches of the second: the caller holds
+  // enqueue_lock() from before this call until its last launch is enqueued.
+  std::unique_lock<std::mutex> enqueue_lock() { return std::unique_lock<std::mutex>(node_table_mutex_); }
   std::pair<void*, uint32_t> node_table(void* stream) {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
     if (bytes == 0 || bytes > (size_t(8) << 30)) return {nullptr, 0u};
-    std::lock_guard<std::mutex> lock(node_table_mutex_);
     auto it = node_tables_.find(stream);
     if (it == node_tables_.end()) {
       if (node_tables_.size() >= kMaxNodeTables) return {nullptr, 0u};
@@ -531,6 +534,8 @@ class PendingBlocks : public torch::CustomClassHolder {
     const size_t ws_bytes = probs ? dgs_sample_blocks_weighted_workspace_bytes(n, fanouts.data(), hops, w)
                                   : dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
     torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
+    // host threads that sample from the same graph enqueue their calls one at a time
+    const std::unique_lock<std::mutex> one_call_at_a_time = indptr->enqueue_lock();
     const auto table = indptr->node_table(st);
     TORCH_CHECK(!probs || table.first != nullptr,
                 "weighted sample_blocks needs a node table (fewer than 2^31 nodes, at most 4 streams in use): "

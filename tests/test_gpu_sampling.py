@@ -351,3 +351,47 @@ def test_batches_in_flight_on_two_streams(pkg, oracle, graph):
         want_f, _, _ = oracle.sample_blocks(batches[0], indptr, indices, fanouts, False, 4321, 50)
         assert np.array_equal(_np(f), want_f)
         pkg.set_rng_state(4321, 50)
+
+
+def test_host_threads_sampling_from_one_graph_on_one_stream(pkg, oracle):
+    # two host threads submit batches on the same stream: their calls share that stream's node
+    # table, so the launches of one call must not be interleaved with another's.  Full
+    # neighbourhoods (fanout >= every degree) make the result independent of which rng stream a
+    # call happened to draw.
+    import threading
+    rng = np.random.default_rng(5)
+    n = 4000
+    deg = rng.integers(0, 7, size=n)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, n, size=int(indptr[-1])).astype(np.int64)
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    fanouts = [6, 6, 6]
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct)
+    batches = [rng.integers(0, n, size=300).astype(np.int64) for _ in range(40)]
+    dev_batches = [_dev(b) for b in batches]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    results, errors = {}, []
+
+    def work(ids):
+        try:
+            with torch.cuda.stream(stream):
+                for i in ids:
+                    results[i] = sampler.submit(None, dev_batches[i]).result()
+        except Exception as e:  # surfaced below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(range(t, 40, 2),)) for t in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for i, b in enumerate(batches):
+        want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, fanouts, False, 1, 0)
+        assert np.array_equal(_np(results[i][0]), want_f), i
+        for gb, wb in zip(results[i][2], want_blocks):
+            assert np.array_equal(_np(gb.src_local), wb[0]) and np.array_equal(_np(gb.dst_local), wb[1])
