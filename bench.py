@@ -194,31 +194,17 @@ def store_from_device(dgs, t, capacity_bytes):
     return ct
 
 
-def run_batches(sampler, seed_batches, features, inflight, consume=lambda r: None):
-    """The timed loop: every batch is submitted on one of `inflight` streams in turn and collected
-    once `inflight` batches are queued, so that many batches share the GPU at any time.
-    `consume` turns each result into what the caller keeps (the big buffers are dropped at once so
-    the allocator can hand them to the next batch).  The caller brackets the call with
-    synchronisations."""
+def run_batches(sampler, seed_batches, features, inflight, consume=lambda r: None, hand_over=False):
+    """The timed loop: the package's BatchPipeline submits every batch on one of `inflight` streams
+    in turn and hands each one out once `inflight` batches are queued, so that many batches share
+    the GPU at any time.  `consume` turns each result into what the caller keeps (the big buffers
+    are dropped at once so the allocator can hand them to the next batch).  The caller brackets
+    the call with synchronisations.  Nothing here touches a batch on another stream than its own,
+    so by default the pipeline does not hand batches over to the calling stream."""
     if inflight <= 1 or not sampler.fused:
         return [consume(sampler.sample_blocks_and_index(None, b, features)) for b in seed_batches]
-    if len(getattr(run_batches, "streams", [])) != inflight:
-        run_batches.streams = [torch.cuda.Stream() for _ in range(inflight)]
-    streams = run_batches.streams
-    start = torch.cuda.current_stream()
-    for st in streams:
-        st.wait_stream(start)
-    out, queue = [], []
-    for i, b in enumerate(seed_batches):
-        with torch.cuda.stream(streams[i % inflight]):
-            queue.append(sampler.submit(None, b, features))
-        if len(queue) >= inflight:
-            out.append(consume(queue.pop(0).result()))
-    while queue:
-        out.append(consume(queue.pop(0).result()))
-    for st in streams:
-        start.wait_stream(st)
-    return out
+    pipeline = sys.modules[type(sampler).__module__].BatchPipeline(sampler, features, inflight, hand_over=hand_over)
+    return [consume(r) for r in pipeline(seed_batches)]
 
 
 def time_call(fn, reps):
@@ -464,6 +450,16 @@ def main():
     run_batches(sampler, batches[args.warmup:], ct_feats, 1)
     torch.cuda.synchronize()
     ms_latency = 1e3 * (time.perf_counter() - t0) / args.steps
+    # batches in flight again, each handed over to the calling stream (made to wait for the batch,
+    # buffers recorded there): what a consumer on another stream than the batch's own sees
+    ms_handed_over = None
+    if inflight > 1:
+        run_batches(sampler, batches[:args.warmup], ct_feats, inflight, hand_over=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_batches(sampler, batches[args.warmup:], ct_feats, inflight, hand_over=True)
+        torch.cuda.synchronize()
+        ms_handed_over = 1e3 * (time.perf_counter() - t0) / args.steps
 
     # Stage split and the dominant kernel's duration, on the same batches: events on torch's
     # current stream (the one the C ABI launches on) around the sampler call and around the
@@ -516,6 +512,7 @@ def main():
                                f"{', weighted by a float32 weight per edge' if cfg.get('weighted') else ''}, then gather",
                    "fanouts": cfg["fanouts"], "batch": cfg["batch"], "batches_in_flight": inflight},
         "ms_per_batch_alone": ms_latency,
+        "ms_per_step_handed_over": ms_handed_over,
         "sample_edges_per_s": edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
         "ms_sample_relabel": ms_sample,

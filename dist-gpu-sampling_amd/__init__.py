@@ -28,6 +28,7 @@ from . import capi  # noqa: E402
 torch.ops.load_library(TORCH_LIB)
 
 from .sampler import (  # noqa: E402
+    BatchPipeline,
     ChunkTensorSampler,
     Block,
     PendingBatch,
@@ -43,5 +44,5 @@ from . import loading_factor  # noqa: E402
 ChunkTensor = torch.classes.dgs_classes.ChunkTensor
 ops = torch.ops.dgs_ops
 
-__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "Block", "PendingBatch", "create_chunktensor",
+__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "create_chunktensor",
            "create_dgs_communicator", "get_available_memory", "set_rng_state", "HIP_LIB", "TORCH_LIB"]

@@ -2,7 +2,7 @@
 (oppo_bench/single_node/utils/chunktensor_sampler.py) at world size 1, without
 DGL: a block is a plain record instead of a DGLBlock.
 """
-from collections import namedtuple
+from collections import deque, namedtuple
 
 import torch
 
@@ -150,3 +150,76 @@ class ChunkTensorSampler:
             seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
             chunk_features)
         return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts), x
+
+
+_pipeline_streams = []
+
+
+def pipeline_streams(n):
+    """The first n of the streams that BatchPipeline objects run on by default.  They are shared by
+    all pipelines of the process: a graph keeps one node table per stream that ever sampled from
+    it (at most four), so pipelines that come and go should not each bring new streams."""
+    while len(_pipeline_streams) < n:
+        _pipeline_streams.append(torch.cuda.Stream())
+    return _pipeline_streams[:n]
+
+
+class BatchPipeline:
+    """Runs seed batches through a ChunkTensorSampler with `inflight` batches on the GPU at any
+    time, each on a stream of its own (what upstream leaves to the DataLoader's prefetching):
+
+        for input_nodes, seeds, blocks, x in BatchPipeline(sampler, feats_ct)(seed_batches):
+            ...                                   # on the caller's current stream
+
+    Results come back in submission order, as ChunkTensorSampler.sample_blocks[_and_index] returns
+    them.  Before a batch is handed out the caller's stream is made to wait for the batch's last
+    kernels, and the batch's tensors are recorded on that stream, so they can be used there (and
+    dropped) without further care.  With hand_over=False neither happens: the batch's last kernels
+    may still be running on the stream it was submitted on, and whoever uses it elsewhere orders
+    that stream behind it; a consumer that works on the batch's own stream needs nothing, and the
+    allocator can reuse the batch's buffers as soon as they are dropped (measured on a 288 MB
+    feature block per batch: 5 % more batches per second).
+    By default all pipelines share pipeline_streams(inflight).
+    Streams of one pipeline should sit on different hardware queues to overlap; the first
+    streams of torch's pool do.
+    """
+
+    def __init__(self, sampler, chunk_features=None, inflight=2, streams=None, hand_over=True):
+        self.hand_over = hand_over
+        if inflight < 1:
+            raise ValueError("inflight must be at least 1")
+        self.sampler = sampler
+        self.chunk_features = chunk_features
+        self.streams = list(streams) if streams is not None else pipeline_streams(inflight)
+        if not self.streams:
+            raise ValueError("no streams to run on")
+
+    def _hand_out(self, pending, consumer):
+        out = pending.result()
+        if not self.hand_over:
+            return out
+        consumer.wait_stream(pending.stream)
+        tensors = [out[0]]
+        for b in out[2]:
+            tensors += [b.src_local, b.dst_local]
+        if out[2]:
+            tensors.append(out[2][-1].dst_ids)  # the seeds on the device (an upload, if they came from the host)
+        if len(out) > 3:
+            tensors.append(out[3])
+        for t in tensors:  # frontiers and seeds are views of these or of the caller's own tensor
+            if t.is_cuda:
+                t.record_stream(consumer)
+        return out
+
+    def __call__(self, seed_batches):
+        consumer = torch.cuda.current_stream()
+        for st in self.streams:
+            st.wait_stream(consumer)  # whatever produced the seeds and the stores comes first
+        queue = deque()
+        for i, seeds in enumerate(seed_batches):
+            with torch.cuda.stream(self.streams[i % len(self.streams)]):
+                queue.append(self.sampler.submit(None, seeds, self.chunk_features))
+            if len(queue) >= len(self.streams):
+                yield self._hand_out(queue.popleft(), consumer)
+        while queue:
+            yield self._hand_out(queue.popleft(), consumer)

@@ -395,3 +395,44 @@ def test_host_threads_sampling_from_one_graph_on_one_stream(pkg, oracle):
         assert np.array_equal(_np(results[i][0]), want_f), i
         for gb, wb in zip(results[i][2], want_blocks):
             assert np.array_equal(_np(gb.src_local), wb[0]) and np.array_equal(_np(gb.dst_local), wb[1])
+
+
+def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph):
+    # BatchPipeline: batches in flight on its own streams, results in submission order, usable on
+    # the caller's stream at once (reduced there right away, buffers dropped while later batches
+    # are still running), host and device seeds, uniform and weighted samplers
+    indptr, indices = graph
+    big = 1 << 40
+    rng = np.random.default_rng(8)
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    probs = (rng.random(indices.size) + 0.1).astype(np.float32)
+    pr_ct = pkg.create_chunktensor(torch.from_numpy(probs), 1, big)
+    feats = rng.standard_normal((20000, 24)).astype(np.float32)
+    x_ct = pkg.create_chunktensor(torch.from_numpy(feats), 1, big, cache_rate=0.6)
+    fanouts = [6, 4]
+    batches = [rng.integers(0, 20000, size=900).astype(np.int64) for _ in range(11)]
+    for weights, inflight in ((None, 2), (None, 3), (pr_ct, 2), (None, 1)):
+        sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, weights)
+        pipe = pkg.BatchPipeline(sampler, x_ct, inflight)
+        pkg.set_rng_state(99, 7)
+        feeds = [torch.from_numpy(b) if i % 2 else _dev(b) for i, b in enumerate(batches)]
+        sums, kept = [], []
+        for i, (f, seeds, blocks, x) in enumerate(pipe(feeds)):
+            sums.append(x.double().sum(dim=0))           # on the caller's stream, no extra wait
+            kept.append((f.clone(), [(b.src_local.clone(), b.dst_local.clone()) for b in blocks]))
+            assert seeds is feeds[i]
+            del f, blocks, x
+        torch.cuda.synchronize()
+        assert len(kept) == len(batches)
+        for i, b in enumerate(batches):
+            want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, fanouts, False, 99, 7 + 2 * i,
+                                                          probs=None if weights is None else probs)
+            assert np.array_equal(_np(kept[i][0]), want_f), (inflight, i)
+            for (src, dst), wb in zip(kept[i][1], want_blocks):
+                assert np.array_equal(_np(src), wb[0]) and np.array_equal(_np(dst), wb[1])
+            assert np.allclose(_np(sums[i]), feats[want_f].astype(np.float64).sum(axis=0), rtol=0, atol=1e-9)
+    with pytest.raises(ValueError):
+        pkg.BatchPipeline(sampler, x_ct, 0)
+    with pytest.raises(RuntimeError):
+        list(pkg.BatchPipeline(pkg.ChunkTensorSampler([100], ip_ct, ix_ct), x_ct)([_dev(batches[0])]))
