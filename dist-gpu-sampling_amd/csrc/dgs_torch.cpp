@@ -18,6 +18,7 @@
 //   - random picks come from a counter-based generator whose (seed, stream) is
 //     settable; upstream re-seeds the constant 7777 on every call
 //     (src/cuda/rowwise_sampling_with_chunk_tensor.cu:162).
+#include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/custom_class.h>
 #include <torch/script.h>
@@ -183,14 +184,27 @@ class ChunkTensor : public torch::CustomClassHolder {
   // all launches of the first precede all launches of the second: the caller holds
   // enqueue_lock() from before this call until its last launch is enqueued.
   std::unique_lock<std::mutex> enqueue_lock() { return std::unique_lock<std::mutex>(node_table_mutex_); }
-  std::pair<void*, uint32_t> node_table(void* stream) {
+  // `must_have`: when every table belongs to another stream, take over the one that was used
+  // longest ago, after waiting for the device to go idle (nothing else says when that stream's
+  // last call on it has finished); without it such a caller gets no table.
+  std::pair<void*, uint32_t> node_table(void* stream, bool must_have = false) {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
     if (bytes == 0 || bytes > (size_t(8) << 30)) return {nullptr, 0u};
     auto it = node_tables_.find(stream);
     if (it == node_tables_.end()) {
-      if (node_tables_.size() >= kMaxNodeTables) return {nullptr, 0u};
-      it = node_tables_.emplace(stream, NodeTable{}).first;
+      if (node_tables_.size() >= kMaxNodeTables) {
+        if (!must_have) return {nullptr, 0u};
+        auto oldest = node_tables_.begin();
+        for (auto jt = node_tables_.begin(); jt != node_tables_.end(); ++jt)
+          if (jt->second.last_use < oldest->second.last_use) oldest = jt;
+        c10::hip::device_synchronize();
+        NodeTable taken = std::move(oldest->second);
+        node_tables_.erase(oldest);
+        it = node_tables_.emplace(stream, std::move(taken)).first;
+      } else {
+        it = node_tables_.emplace(stream, NodeTable{}).first;
+      }
     }
     NodeTable& t = it->second;
     if (!t.entries.defined() || t.epoch >= 0xffffff00u) {
@@ -198,6 +212,7 @@ class ChunkTensor : public torch::CustomClassHolder {
                               torch::TensorOptions().dtype(torch::kInt64).device(device_));
       t.epoch = 0;
     }
+    t.last_use = ++uses_;
     return {t.entries.data_ptr(), ++t.epoch};
   }
 
@@ -218,7 +233,9 @@ class ChunkTensor : public torch::CustomClassHolder {
   struct NodeTable {
     torch::Tensor entries;
     uint32_t epoch = 0;
+    uint64_t last_use = 0;
   };
+  uint64_t uses_ = 0;
   static constexpr size_t kMaxNodeTables = 4;
   std::map<void*, NodeTable> node_tables_;
   std::mutex node_table_mutex_;
@@ -536,10 +553,9 @@ class PendingBlocks : public torch::CustomClassHolder {
     torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
     // host threads that sample from the same graph enqueue their calls one at a time
     const std::unique_lock<std::mutex> one_call_at_a_time = indptr->enqueue_lock();
-    const auto table = indptr->node_table(st);
+    const auto table = indptr->node_table(st, /*must_have=*/static_cast<bool>(probs));
     TORCH_CHECK(!probs || table.first != nullptr,
-                "weighted sample_blocks needs a node table (fewer than 2^31 nodes, at most 4 streams in use): "
-                "use the per-hop operators here");
+                "weighted sample_blocks needs a node table (fewer than 2^31 nodes): use the per-hop operators here");
     const auto rng = next_rng(static_cast<uint32_t>(hops));
     if (probs)
       check(dgs_sample_blocks_weighted(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), probs->view(),

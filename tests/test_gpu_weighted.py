@@ -284,3 +284,27 @@ def test_weighted_rows_that_the_key_halves_leave_open(pkg, oracle):
         assert np.array_equal(_np(f), want_f), fanouts
         for g, w in zip(blocks, want_blocks):
             assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
+
+
+def test_weighted_fused_on_more_streams_than_node_tables(pkg, oracle, graph):
+    # a graph keeps at most four node tables, one per stream; the weighted fused driver needs one,
+    # so a fifth and sixth stream take over the table that was used longest ago
+    indptr, indices, probs = graph
+    big = 1 << 40
+    cts = [pkg.create_chunktensor(torch.from_numpy(a), 1, big) for a in (indptr, indices, probs)]
+    sampler = pkg.ChunkTensorSampler([5, 3], *cts)
+    rng = np.random.default_rng(9)
+    streams = [torch.cuda.Stream() for _ in range(6)]
+    batches = [rng.integers(0, 20000, size=400).astype(np.int64) for _ in range(14)]
+    pkg.set_rng_state(555, 0)
+    pending = []
+    for i, b in enumerate(batches):
+        with torch.cuda.stream(streams[(i * 5) % 6]):
+            pending.append(sampler.submit(None, _dev(b)))
+    for i, b in enumerate(batches):
+        want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, [5, 3], False, 555, 2 * i, probs=probs)
+        f, _, blocks = pending[i].result()
+        assert np.array_equal(_np(f), want_f), i
+        for g, w in zip(blocks, want_blocks):
+            assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
+    torch.cuda.synchronize()
