@@ -60,6 +60,8 @@ SIGNATURES = {
                                        c_vp, c_sz, c_vp]),
     "dgs_sample_neighbors": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32,
                                             c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_neighbors_static": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32,
+                                                   c_vp, c_vp, c_vp, c_vp]),
     "dgs_sample_fill_weighted": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32, c_vp,
                                                 c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_neighbors_weighted": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, View, c_i64, c_i32, c_u64,
@@ -206,6 +208,21 @@ def sample_neighbors(seeds, indptr_view, indices_view, num_picks, replace, rng_s
     check(lib.dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr_view, indices_view, num_picks, int(replace),
                                    rng_seed, rng_stream, rows.data_ptr(), cols.data_ptr(), nnz.data_ptr(),
                                    ws.data_ptr(), nb, stream_ptr()))
+    cnt, flags = read_i64(nnz, 2)
+    return rows[:cnt], cols[:cnt], flags
+
+
+STATIC_MAX_SEEDS = 65536  # DGS_STATIC_MAX_SEEDS
+
+
+def sample_neighbors_static(seeds, indptr_view, indices_view, num_picks, replace, rng_seed, rng_stream,
+                            rows, cols, nnz):
+    """dgs_sample_neighbors_static into caller-provided buffers (rows / cols: n * num_picks ids,
+    nnz: int64[2]); nothing is allocated here or in the library.  Returns (coo_row, coo_col, flags)."""
+    n = seeds.numel()
+    check(lib.dgs_sample_neighbors_static(seeds.data_ptr(), seeds.element_size(), n, indptr_view, indices_view,
+                                          num_picks, int(replace), rng_seed, rng_stream, rows.data_ptr(),
+                                          cols.data_ptr(), nnz.data_ptr(), stream_ptr()))
     cnt, flags = read_i64(nnz, 2)
     return rows[:cnt], cols[:cnt], flags
 

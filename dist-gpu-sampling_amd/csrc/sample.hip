@@ -10,12 +10,41 @@
 //           larger num_picks: one wave per row, Floyd's kept set in LDS.
 // Random picks follow the "dgs-philox-1" contract: every (seed, stream, row, draw) names one
 // Philox block, so results do not depend on the launch shape.
+#include <mutex>
+
 #include "common.h"
 #include "picks.h"
 #include "sample_workspace.h"
 
 namespace dgs {
 namespace {
+
+// Scratch of the entry point that allocates nothing: one copy per GPU, held until the process
+// ends.  In host code the array's name is only a stand-in; the device address of each GPU's copy
+// comes from hipGetSymbolAddress (static_scratch_of) and is what kernels and checks receive.
+constexpr int64_t kStaticMaxSeeds = DGS_STATIC_MAX_SEEDS;
+constexpr size_t kStaticScratchBytes = size_t(2) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+void* g_static_scratch[kMaxDevices] = {};
+
+// The current device's copy of `scratch`, looked up once per device.
+dgs_status static_scratch_of(void** out) {
+  int dev = -1;
+  DGS_HIP_TRY(hipGetDevice(&dev));
+  DGS_REQUIRE(dev >= 0 && dev < kMaxDevices, DGS_ERR_UNSUPPORTED, "sample_neighbors_static: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_scratch[dev] == nullptr) {
+    void* p = nullptr;
+    DGS_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    DGS_REQUIRE(p != nullptr && (reinterpret_cast<uintptr_t>(p) & 255) == 0, DGS_ERR_HIP,
+                "sample_neighbors_static: scratch symbol resolved to %p", p);
+    g_static_scratch[dev] = p;
+  }
+  *out = g_static_scratch[dev];
+  return DGS_OK;
+}
 
 constexpr int kMaxGroupPicks = 64;   // fill_group_kernel handles num_picks <= 64
 constexpr int kMaxLdsPicks = 2048;   // fill_wave_kernel keeps Floyd's set in LDS
@@ -262,4 +291,24 @@ DGS_API dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes, int
   if (s != DGS_OK) return s;
   return dgs_sample_fill(seeds, id_bytes, n_seeds, indices, num_picks, replace, rng_seed, rng_stream, out_rows,
                          out_cols, workspace, workspace_bytes, stream);
+}
+
+DGS_API dgs_status dgs_sample_neighbors_static(const void* seeds, int32_t id_bytes, int64_t n_seeds,
+                                               dgs_view indptr, dgs_view indices, int64_t num_picks,
+                                               int32_t replace, uint64_t rng_seed, uint32_t rng_stream,
+                                               void* out_rows, void* out_cols, int64_t* nnz_dev, void* stream) {
+  using namespace dgs;
+  DGS_REQUIRE(n_seeds >= 0 && n_seeds <= kStaticMaxSeeds, DGS_ERR_UNSUPPORTED,
+              "sample_neighbors_static: %lld seeds, at most %lld fit the static scratch (use dgs_sample_neighbors "
+              "with a workspace)", (long long)n_seeds, (long long)kStaticMaxSeeds);
+  DGS_REQUIRE(sample_workspace_layout(n_seeds, nullptr, nullptr) <= kStaticScratchBytes, DGS_ERR_UNSUPPORTED,
+              "sample_neighbors_static: scratch of %zu B is too small for %lld seeds", kStaticScratchBytes,
+              (long long)n_seeds);
+  void* ws = nullptr;
+  const dgs_status s = static_scratch_of(&ws);
+  if (s != DGS_OK) return s;
+  // every word of the layout that the fill reads is written by the count pass of the same call,
+  // so nothing of the previous call's contents has to be cleared
+  return dgs_sample_neighbors(seeds, id_bytes, n_seeds, indptr, indices, num_picks, replace, rng_seed, rng_stream,
+                              out_rows, out_cols, nnz_dev, ws, kStaticScratchBytes, stream);
 }

@@ -216,6 +216,27 @@ dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes,
                                 void* stream);
 
 /*
+ * dgs_sample_neighbors without a workspace argument and without any allocation.  No
+ * counterpart in the reference; it is for callers that cannot allocate device memory at the
+ * point of the call: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  The per-seed temporaries live in a fixed array inside the library (2 MiB per GPU,
+ * held until the process ends), which bounds the call to DGS_STATIC_MAX_SEEDS seeds
+ * (DGS_ERR_UNSUPPORTED above that).  Arguments, outputs (out_rows / out_cols hold
+ * n_seeds * num_picks ids), flags and results are those of dgs_sample_neighbors.  Calls on one
+ * GPU share that GPU's array: two calls that overlap in time on the same GPU (different
+ * streams or host threads) race; calls on one stream do not.  The first call on a device
+ * looks the array's address up and should be made outside graph capture.
+ */
+#define DGS_STATIC_MAX_SEEDS 65536
+dgs_status dgs_sample_neighbors_static(const void* seeds, int32_t id_bytes,
+                                       int64_t n_seeds, dgs_view indptr,
+                                       dgs_view indices, int64_t num_picks,
+                                       int32_t replace, uint64_t rng_seed,
+                                       uint32_t rng_stream, void* out_rows,
+                                       void* out_cols, int64_t* nnz_dev,
+                                       void* stream);
+
+/*
  * One weighted hop: like dgs_sample_neighbors with a float32 weight per edge
  * (`probs`, a view of E floats laid out like `indices`).  Replaces
  * RowWiseSamplingProbCUDA and RowWiseSamplingProbWithChunkTensorCUDA
