@@ -353,7 +353,6 @@ def run_large(args, dgs):
     }
     if cfg["hbm_rows"] < 1.0:
         local, _, host_ids = ct_x._CAPI_split_index(frontier)
-        host_ids = host_ids[host_ids > hot_rows]  # the row that straddles the boundary belongs to neither tier
         t_local = time_call(lambda: ct_x._CAPI_local_index(local), 5)
         t_host = time_call(lambda: ct_x._CAPI_host_index(host_ids), 3)
         dev_gbps = local.numel() * (2 * row_bytes + 4) / t_local / 1e9

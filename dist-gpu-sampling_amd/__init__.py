@@ -35,6 +35,7 @@ from .sampler import (  # noqa: E402
     create_chunktensor,
     create_dgs_communicator,
     get_available_memory,
+    set_gather_buffer_cap,
     set_rng_state,
 )
 
@@ -45,4 +46,4 @@ ChunkTensor = torch.classes.dgs_classes.ChunkTensor
 ops = torch.ops.dgs_ops
 
 __all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "create_chunktensor",
-           "create_dgs_communicator", "get_available_memory", "set_rng_state", "HIP_LIB", "TORCH_LIB"]
+           "create_dgs_communicator", "get_available_memory", "set_rng_state", "set_gather_buffer_cap", "HIP_LIB", "TORCH_LIB"]

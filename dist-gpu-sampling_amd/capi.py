@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libdgs_hip.so")
 
 DGS_OK, DGS_ERR_INVALID, DGS_ERR_HIP, DGS_ERR_WORKSPACE, DGS_ERR_UNSUPPORTED, DGS_ERR_RANGE = range(6)
 TIER_ANY, TIER_DEVICE, TIER_HOST = 0, 1, 2
+DEBUG_FORCE_SPLIT_TABLE, DEBUG_WEIGHTED_GROUP = 0, 1
 MAX_SEGMENTS = 8
 
 c_i64, c_i32, c_u64, c_u32, c_vp, c_sz = (ctypes.c_int64, ctypes.c_int32, ctypes.c_uint64, ctypes.c_uint32,
@@ -42,6 +43,7 @@ SIGNATURES = {
     "dgs_last_error": (ctypes.c_char_p, []),
     "dgs_status_name": (ctypes.c_char_p, [ctypes.c_int]),
     "dgs_abi_version": (ctypes.c_int, []),
+    "dgs_debug_set": (ctypes.c_int, [c_i32, c_i64]),
     "dgs_store_split": (ctypes.c_int, [c_i64, c_i32, c_i64, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)]),
     "dgs_store_create": (ctypes.c_int, [c_i64, c_i32, c_i64, ctypes.POINTER(c_vp)]),
     "dgs_store_destroy": (ctypes.c_int, [c_vp]),
@@ -50,8 +52,8 @@ SIGNATURES = {
     "dgs_store_slices": (ctypes.c_int, [c_vp, ctypes.POINTER(c_vp), ctypes.POINTER(c_i64),
                                         ctypes.POINTER(c_vp), ctypes.POINTER(c_i64)]),
     "dgs_current_allocated": (c_i64, []),
-    "dgs_gather_rows": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i32, c_vp]),
-    "dgs_gather_rows_dyn": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_i32, c_vp]),
+    "dgs_gather_rows": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i32, c_vp, c_vp]),
+    "dgs_gather_rows_dyn": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_i32, c_vp, c_vp]),
     "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
     "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_workspace_bytes": (c_sz, [c_i64]),
@@ -87,6 +89,7 @@ SIGNATURES = {
     "dgs_ticket_stream_wait": (ctypes.c_int, [c_vp, c_vp]),
     "dgs_ticket_wait": (ctypes.c_int, [c_vp]),
     "dgs_ticket_release": (ctypes.c_int, [c_vp]),
+    "dgs_stream_query": (ctypes.c_int, [c_vp, ctypes.POINTER(c_i32)]),
 }
 
 if not os.path.exists(LIB_PATH):
@@ -166,11 +169,13 @@ def read_i64(dev_tensor, count):
     return host.tolist()
 
 
-def gather_rows(view, row_elems, index, dtype, tier=TIER_ANY):
+def gather_rows(view, row_elems, index, dtype, tier=TIER_ANY, bad_index=None):
+    """`bad_index`: optional int64[1] device tensor that the kernel sets to 1 on an index outside
+    the rows the tier holds (the caller clears it)."""
     n = index.numel()
     out = torch.empty((n, row_elems), dtype=dtype, device=index.device)
     check(lib.dgs_gather_rows(view, row_elems, index.data_ptr(), index.element_size(), n, out.data_ptr(), tier,
-                              stream_ptr()))
+                              bad_index.data_ptr() if bad_index is not None else None, stream_ptr()))
     return out
 
 
@@ -311,7 +316,7 @@ def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_se
     if feature_view is not None:
         x = torch.empty((smax[hops], feature_row_elems), dtype=feature_dtype, device=seeds.device)
         check(lib.dgs_gather_rows_dyn(feature_view, feature_row_elems, frontier.data_ptr(), w, smax[hops],
-                                      sizes.data_ptr() + 8 * hops, x.data_ptr(), TIER_ANY, stream_ptr()))
+                                      sizes.data_ptr() + 8 * hops, x.data_ptr(), TIER_ANY, None, stream_ptr()))
     sz = read_i64(sizes, 3 * hops + 1)
     result = [(frontier[:sz[h + 1]], s[:sz[hops + 1 + h]], d[:sz[hops + 1 + h]]) for h, (s, d) in enumerate(bufs)]
     if x is not None:

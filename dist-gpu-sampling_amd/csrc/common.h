@@ -40,6 +40,9 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 inline bool width_ok(int32_t b) { return b == 4 || b == 8; }
 
+// Value of a dgs_debug_set option (0 unless a test set it).
+int64_t debug_option(int32_t option);
+
 // Carves aligned pieces out of a caller-provided workspace.
 struct Carver {
   char* base;
@@ -65,10 +68,17 @@ struct TierView {
   const T* dev;
   const T* host;
   int64_t thr;
+  int64_t n;  // elements in the whole store: what an index is checked against before it is used
   __host__ explicit TierView(const dgs_view& v)
-      : dev(static_cast<const T*>(v.dev)), host(static_cast<const T*>(v.host)), thr(v.threshold) {}
+      : dev(static_cast<const T*>(v.dev)), host(static_cast<const T*>(v.host)), thr(v.threshold), n(v.total) {}
   __device__ __forceinline__ T at(int64_t i) const { return i < thr ? dev[i] : host[i - thr]; }
 };
+
+// Whether `row` names a row of the CSC offsets array `indptr` (entries row and row + 1 exist).
+template <typename T>
+__device__ __forceinline__ bool row_in_range(const TierView<T>& indptr, int64_t row) {
+  return row >= 0 && row < indptr.n - 1;
+}
 
 // Exclusive scan of one value per thread over a block of NT threads (NT multiple of 64).
 // Returns the exclusive prefix; *total receives the block sum (same value in all threads).

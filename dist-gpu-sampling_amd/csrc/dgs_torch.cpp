@@ -17,8 +17,12 @@
 //     f32 only, src/dgs_headers.h:60-74);
 //   - random picks come from a counter-based generator whose (seed, stream) is
 //     settable; upstream re-seeds the constant 7777 on every call
-//     (src/cuda/rowwise_sampling_with_chunk_tensor.cu:162).
+//     (src/cuda/rowwise_sampling_with_chunk_tensor.cu:162);
+//   - seed ids and gather indices outside the graph / the store are refused instead of
+//     dereferenced (upstream does not check, src/cuda/index_with_chunk_tensor.cu:16-23):
+//     sampling raises; a gather zero-fills the row and the store raises at its next call.
 #include <c10/hip/HIPFunctions.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/custom_class.h>
 #include <torch/script.h>
@@ -76,6 +80,20 @@ std::pair<uint64_t, uint32_t> next_rng(uint32_t calls = 1) {
   return {g_rng_seed, first};
 }
 
+// Above this many bytes a worst-case feature buffer is not allocated: the fused operator waits
+// for the frontier's size and allocates exactly (see PendingBlocks::Begin).
+std::atomic<int64_t> g_gather_buffer_cap{int64_t(2) << 30};
+
+// What the error bits of a sampling call mean (include/dgs_hip.h, sizes_dev / nnz_dev flags).
+void check_sampling_flags(int64_t flags, const char* who, int hop) {
+  if (flags == 0) return;
+  const std::string where = hop >= 0 ? std::string(who) + ": hop " + std::to_string(hop) : std::string(who);
+  TORCH_CHECK((flags & 2) == 0, where, ": a seed id is not a row of the graph (outside 0 .. nodes - 1)");
+  TORCH_CHECK((flags & 4) == 0, where, ": a neighbour id stored in the graph is not a node (outside 0 .. nodes - 1)");
+  TORCH_CHECK((flags & 1) == 0, where, ": a seed row has a degree of 2^32 or more, or offsets outside the edge array");
+  TORCH_CHECK(false, where, ": error bits ", flags);
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------
@@ -103,8 +121,30 @@ class ChunkTensor : public torch::CustomClassHolder {
     check(dgs_store_view(store_, &view_));
     // torch on ROCm names its GPU device type CUDA; only the index comes from the HIP stream
     device_ = c10::Device(c10::DeviceType::CUDA, c10::hip::getCurrentHIPStream().device_index());
+    // the word a gather sets when it meets an index outside the store (pinned: the host reads it
+    // without a copy, the kernels write it through its device mapping)
+    bad_index_ = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
   }
   ~ChunkTensor() override { dgs_store_destroy(store_); }
+
+  // Raises if a gather that has run since the last check met an index outside the rows it may
+  // read (those output rows were zero-filled).  Gathers are asynchronous, so the error surfaces
+  // at the store's next operator call, or here after a synchronisation.
+  void CheckErrors() {
+    int64_t* w = bad_index_.data_ptr<int64_t>();
+    if (__atomic_load_n(w, __ATOMIC_RELAXED) != 0) {
+      __atomic_store_n(w, int64_t(0), __ATOMIC_RELAXED);
+      TORCH_CHECK(false, "ChunkTensor: an earlier gather was given row ids outside the store (or outside the "
+                         "tier of _CAPI_local_index / _CAPI_host_index); those output rows were filled with zeros");
+    }
+  }
+  void SynchronizeAndCheck() {
+    void* ticket = nullptr;
+    check(dgs_ticket_record(current_stream(), &ticket));
+    check(dgs_ticket_wait(ticket));
+    CheckErrors();
+  }
+  int64_t* bad_index_word() const { return bad_index_.data_ptr<int64_t>(); }
 
   // upstream GetHostTensor (src/chunk_tensor.cc:151-160): flat, non-owning
   torch::Tensor GetHostTensor() {
@@ -139,13 +179,15 @@ class ChunkTensor : public torch::CustomClassHolder {
     check(dgs_store_load(store_, data.data_ptr(), total_));
   }
 
-  torch::Tensor Gather(const torch::Tensor& index_in, int32_t tier) const {
+  torch::Tensor Gather(const torch::Tensor& index_in, int32_t tier) {
+    CheckErrors();
     DGS_CHECK_GPU(index_in);
     const int32_t w = id_width(index_in, "index");
     torch::Tensor index = index_in.contiguous();
     const int64_t n = index.numel();
     torch::Tensor out = torch::empty({n, elem_stride_}, torch::TensorOptions().dtype(dtype_).device(index.device()));
-    check(dgs_gather_rows(view_, elem_stride_, index.data_ptr(), w, n, out.data_ptr(), tier, current_stream()));
+    check(dgs_gather_rows(view_, elem_stride_, index.data_ptr(), w, n, out.data_ptr(), tier, bad_index_word(),
+                          current_stream()));
     return out;
   }
   // upstream Index / LocalIndex / RemoteIndex / HostIndex (src/chunk_tensor.cc:207-221)
@@ -161,6 +203,7 @@ class ChunkTensor : public torch::CustomClassHolder {
 
   // upstream SplitIndex (src/chunk_tensor.cc:202-205)
   std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> SplitIndex(torch::Tensor index_in) {
+    CheckErrors();
     DGS_CHECK_GPU(index_in);
     const int32_t w = id_width(index_in, "index");
     torch::Tensor index = index_in.contiguous().view({-1});
@@ -184,9 +227,10 @@ class ChunkTensor : public torch::CustomClassHolder {
   // all launches of the first precede all launches of the second: the caller holds
   // enqueue_lock() from before this call until its last launch is enqueued.
   std::unique_lock<std::mutex> enqueue_lock() { return std::unique_lock<std::mutex>(node_table_mutex_); }
-  // `must_have`: when every table belongs to another stream, take over the one that was used
-  // longest ago, after waiting for the device to go idle (nothing else says when that stream's
-  // last call on it has finished); without it such a caller gets no table.
+  // When every table belongs to another stream, the caller takes over the one used longest ago
+  // among those whose stream has nothing left to run (a stream that is no longer used, such as
+  // one made per epoch).  If all of them are busy: with `must_have` the table used longest ago is
+  // taken after waiting for the device to go idle, without it the caller gets no table.
   std::pair<void*, uint32_t> node_table(void* stream, bool must_have = false) {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
@@ -194,13 +238,25 @@ class ChunkTensor : public torch::CustomClassHolder {
     auto it = node_tables_.find(stream);
     if (it == node_tables_.end()) {
       if (node_tables_.size() >= kMaxNodeTables) {
-        if (!must_have) return {nullptr, 0u};
-        auto oldest = node_tables_.begin();
-        for (auto jt = node_tables_.begin(); jt != node_tables_.end(); ++jt)
+        auto pick = node_tables_.end(), oldest = node_tables_.begin();
+        for (auto jt = node_tables_.begin(); jt != node_tables_.end(); ++jt) {
           if (jt->second.last_use < oldest->second.last_use) oldest = jt;
-        c10::hip::device_synchronize();
-        NodeTable taken = std::move(oldest->second);
-        node_tables_.erase(oldest);
+          int32_t idle = 0;
+          check(dgs_stream_query(jt->first, &idle));
+          if (idle && (pick == node_tables_.end() || jt->second.last_use < pick->second.last_use)) pick = jt;
+        }
+        if (pick == node_tables_.end()) {
+          if (!must_have) return {nullptr, 0u};
+          c10::hip::device_synchronize();
+          pick = oldest;
+        }
+        NodeTable taken = std::move(pick->second);
+        node_tables_.erase(pick);
+        // the memory came from another stream's pool: it must not be handed out again while
+        // this stream still uses it
+        // (torch on ROCm files its allocations under the device type CUDA, hence the stream type)
+        if (taken.entries.defined())
+          taken.entries.record_stream(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap());
         it = node_tables_.emplace(stream, std::move(taken)).first;
       } else {
         it = node_tables_.emplace(stream, NodeTable{}).first;
@@ -230,6 +286,7 @@ class ChunkTensor : public torch::CustomClassHolder {
   dgs_store* store_ = nullptr;
   dgs_view view_{};
   c10::Device device_{c10::DeviceType::CUDA, 0};
+  torch::Tensor bad_index_;
   struct NodeTable {
     torch::Tensor entries;
     uint32_t epoch = 0;
@@ -310,10 +367,7 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
       check(dgs_sample_fill(seeds.data_ptr(), w, n, indices, num_picks, replace, rng.first, rng.second,
                             rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st));
   }
-  TORCH_CHECK((len[1] & 1) == 0, "sample_neighbors: a seed row has a degree of 2^32 or more");
-  TORCH_CHECK((len[1] & 2) == 0,
-              "sample_neighbors: num_picks above 2048 without replacement needs every sampled row to have at most "
-              "num_picks neighbours");
+  check_sampling_flags(len[1], "sample_neighbors", -1);
   return std::make_tuple(rows.narrow(0, 0, len[0]), cols.narrow(0, 0, len[0]));
 }
 
@@ -486,10 +540,14 @@ class PendingBlocks : public torch::CustomClassHolder {
   }
 
   BlocksResult Finish() {
-    TORCH_CHECK(ticket_ != nullptr, "PendingBlocks: already finished");
-    void* t = ticket_;
-    ticket_ = nullptr;
-    const dgs_status ws_status = dgs_ticket_wait(t);
+    TORCH_CHECK(!finished_, "PendingBlocks: already finished");
+    finished_ = true;
+    dgs_status ws_status = DGS_OK;
+    if (ticket_ != nullptr) {  // still null when Begin had to wait for the sizes itself
+      void* t = ticket_;
+      ticket_ = nullptr;
+      ws_status = dgs_ticket_wait(t);
+    }
     check(gather_status_);
     check(ws_status);
     const int64_t* sizes_host = pinned_.data_ptr<int64_t>();
@@ -497,8 +555,7 @@ class PendingBlocks : public torch::CustomClassHolder {
     const std::vector<int64_t> sz(sizes_host, sizes_host + n_sizes);
     std::vector<torch::Tensor> frontier(hops_);
     for (int h = 0; h < hops_; ++h) {
-      TORCH_CHECK(sz[2 * hops_ + 1 + h] == 0, "sample_blocks: a seed row of hop ", h,
-                  " has a degree of 2^32 or more");
+      check_sampling_flags(sz[2 * hops_ + 1 + h], "sample_blocks", h);
       frontier[h] = all_.narrow(0, 0, sz[h + 1]);
       src_[h] = src_[h].narrow(0, 0, sz[hops_ + 1 + h]);
       dst_[h] = dst_[h].narrow(0, 0, sz[hops_ + 1 + h]);
@@ -513,8 +570,10 @@ class PendingBlocks : public torch::CustomClassHolder {
                                                  const std::vector<int64_t>& fanouts, bool replace,
                                                  const c10::intrusive_ptr<ChunkTensor>& features,
                                                  const c10::intrusive_ptr<ChunkTensor>& probs =
-                                                     c10::intrusive_ptr<ChunkTensor>()) {
+                                                     c10::intrusive_ptr<ChunkTensor>(),
+                                                 const std::pair<uint64_t, uint32_t>* own_rng = nullptr) {
     const int32_t w = id_width(seeds_in, "seeds");
+    if (features) features->CheckErrors();
     if (probs) TORCH_CHECK(probs->dtype() == torch::kFloat32, "probs store must be float32, got ", probs->dtype());
     TORCH_CHECK(seeds_in.scalar_type() == indices->dtype(), "seeds (", seeds_in.scalar_type(), ") and indices (",
                 indices->dtype(), ") must have the same dtype");
@@ -556,7 +615,9 @@ class PendingBlocks : public torch::CustomClassHolder {
     const auto table = indptr->node_table(st, /*must_have=*/static_cast<bool>(probs));
     TORCH_CHECK(!probs || table.first != nullptr,
                 "weighted sample_blocks needs a node table (fewer than 2^31 nodes): use the per-hop operators here");
-    const auto rng = next_rng(static_cast<uint32_t>(hops));
+    // the caller's own (seed, first stream) when given, else the next `hops` streams of the
+    // process-wide generator
+    const auto rng = own_rng != nullptr ? *own_rng : next_rng(static_cast<uint32_t>(hops));
     if (probs)
       check(dgs_sample_blocks_weighted(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), probs->view(),
                                        fanouts.data(), hops, replace, rng.first, rng.second, table.first,
@@ -567,19 +628,35 @@ class PendingBlocks : public torch::CustomClassHolder {
                               replace, rng.first, rng.second, table.first, table.second, p->all_.data_ptr(),
                               outs.data(), sizes_dev.data_ptr<int64_t>(), p->pinned_.data_ptr<int64_t>(),
                               &p->ticket_, ws.data_ptr(), ws_bytes, st));
-    // the lengths are final at the ticket; the gather is enqueued before anybody waits for them
     if (features) {
-      p->x_ = torch::empty({seeds_max[hops], features->elem_stride()},
-                           torch::TensorOptions().dtype(features->dtype()).device(dev));
-      p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
-                                              seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops,
-                                              p->x_.data_ptr(), DGS_TIER_ANY, st);
+      const auto xopt = torch::TensorOptions().dtype(features->dtype()).device(dev);
+      const int64_t row_bytes = features->elem_stride() * static_cast<int64_t>(c10::elementSize(features->dtype()));
+      if (seeds_max[hops] * row_bytes <= g_gather_buffer_cap.load()) {
+        // the lengths are final at the ticket; the gather is enqueued before anybody waits for
+        // them, into a buffer for the worst case of which the result is a prefix
+        p->x_ = torch::empty({seeds_max[hops], features->elem_stride()}, xopt);
+        p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
+                                                seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops,
+                                                p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
+      } else {
+        // the worst case would be too large a buffer (it grows with the product of the fanouts,
+        // the frontier does not): wait for the frontier's size and gather into exactly that many
+        // rows, as upstream's exact-size output (src/cuda/index_with_chunk_tensor.cu:29-53)
+        void* t = p->ticket_;
+        p->ticket_ = nullptr;
+        check(dgs_ticket_wait(t));
+        const int64_t rows = p->pinned_.data_ptr<int64_t>()[hops];
+        p->x_ = torch::empty({rows, features->elem_stride()}, xopt);
+        p->gather_status_ = dgs_gather_rows(features->view(), features->elem_stride(), p->all_.data_ptr(), w, rows,
+                                            p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
+      }
     }
     return p;
   }
 
  private:
   int hops_ = 0;
+  bool finished_ = false;
   void* ticket_ = nullptr;
   dgs_status gather_status_ = DGS_OK;
   torch::Tensor pinned_, seeds_, all_, x_;
@@ -639,6 +716,28 @@ c10::intrusive_ptr<PendingBlocks> SampleBlocksWeightedBegin(torch::Tensor seeds,
                               features.has_value() ? *features : c10::intrusive_ptr<ChunkTensor>(), probs);
 }
 
+// Any of the *_begin operators with the generator state passed in: the hops draw from streams
+// rng_stream, rng_stream + 1, ... of seed rng_seed and the process-wide generator is left alone,
+// so a caller that keeps its own counter gets the same picks whatever other threads do.
+c10::intrusive_ptr<PendingBlocks> SampleBlocksSubmit(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr,
+                                                     c10::intrusive_ptr<ChunkTensor> indices,
+                                                     c10::optional<c10::intrusive_ptr<ChunkTensor>> probs,
+                                                     std::vector<int64_t> fanouts, bool replace,
+                                                     c10::optional<c10::intrusive_ptr<ChunkTensor>> features,
+                                                     int64_t rng_seed, int64_t rng_stream) {
+  const std::pair<uint64_t, uint32_t> rng{static_cast<uint64_t>(rng_seed), static_cast<uint32_t>(rng_stream)};
+  return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace,
+                              features.has_value() ? *features : c10::intrusive_ptr<ChunkTensor>(),
+                              probs.has_value() ? *probs : c10::intrusive_ptr<ChunkTensor>(), &rng);
+}
+
+// Largest worst-case feature buffer (bytes) the fused operators allocate ahead of the sizes.
+void SetGatherBufferCap(int64_t bytes) {
+  TORCH_CHECK(bytes >= 0, "gather buffer cap must be >= 0");
+  g_gather_buffer_cap.store(bytes);
+}
+int64_t GetGatherBufferCap() { return g_gather_buffer_cap.load(); }
+
 int64_t GetCurrentAllocated() { return dgs_current_allocated(); }
 
 // upstream nccl::GetUniqueId / nccl::SetNCCL (src/nccl_context.cc:17-34): there is no
@@ -675,7 +774,9 @@ TORCH_LIBRARY(dgs_classes, m) {
       .def("_CAPI_local_index", &ChunkTensor::LocalIndex)
       .def("_CAPI_remote_index", &ChunkTensor::RemoteIndex)
       .def("_CAPI_host_index", &ChunkTensor::HostIndex)
-      .def("_CAPI_load_from_tensor", &ChunkTensor::LoadFromTensor);
+      .def("_CAPI_load_from_tensor", &ChunkTensor::LoadFromTensor)
+      // not in upstream: waits for the current stream, then raises if a gather met a bad row id
+      .def("_CAPI_synchronize_and_check", &ChunkTensor::SynchronizeAndCheck);
   // not in upstream: a sample_blocks call in flight
   m.class_<PendingBlocks>("PendingBlocks").def("_CAPI_finish", &PendingBlocks::Finish);
 }
@@ -695,6 +796,9 @@ TORCH_LIBRARY(dgs_ops, m) {
       .def("_CAPI_sample_blocks_begin", &dgs::SampleBlocksBegin)
       .def("_CAPI_sample_blocks_and_index_begin", &dgs::SampleBlocksAndIndexBegin)
       .def("_CAPI_sample_blocks_weighted_begin", &dgs::SampleBlocksWeightedBegin)
+      .def("_CAPI_sample_blocks_submit", &dgs::SampleBlocksSubmit)
+      .def("_CAPI_set_gather_buffer_cap", &dgs::SetGatherBufferCap)
+      .def("_CAPI_get_gather_buffer_cap", &dgs::GetGatherBufferCap)
       // not in upstream: node renumbering (hottest rows first) for the positional stores
       .def("_CAPI_renumber_csc", &dgs::RenumberCSC)
       // not in upstream: the sampling generator's (seed, stream)

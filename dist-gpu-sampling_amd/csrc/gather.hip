@@ -7,6 +7,10 @@
 // so one wave covers 2.56 rows).  VEC divides both the row size and the byte
 // offset of the device/host boundary, hence no chunk ever straddles the tiers
 // and a straddling ROW is still resolved exactly, chunk by chunk.
+//
+// Index values are checked before they address anything: a row outside the rows the
+// requested tier holds is not read, its output row is filled with zero bytes and the
+// caller's flag word (if any) is set.
 #include "common.h"
 
 namespace dgs {
@@ -42,12 +46,15 @@ __device__ __forceinline__ const char* resolve(const char* dev, const char* host
 // chunk c -> row c / cpr, column c % cpr; the division runs on a block-local
 // 32-bit offset with a precomputed reciprocal (exact while
 // (cpr + kChunksPerBlock) * cpr < 2^32, guaranteed by kMaxFlatChunksPerRow).
+// Rows [row_lo, row_hi) are the ones the launch may read.
 template <int VEC, int TIER, typename IndexT, bool STRIDE>
 __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, uint32_t cpr, uint32_t magic, const IndexT* __restrict__ index,
-    int64_t total_chunks, const int64_t* __restrict__ n_rows_dev, char* __restrict__ out) {
+    int64_t total_chunks, const int64_t* __restrict__ n_rows_dev, int64_t row_lo, int64_t row_hi,
+    int64_t* __restrict__ bad_index, char* __restrict__ out) {
   using C = typename Chunk<VEC>::type;
+  bool bad = false;
   if (n_rows_dev) total_chunks = *n_rows_dev * cpr;  // row count decided on the device
   // STRIDE: the grid is smaller than the tile count (capped launch), blocks stride over the tiles
   for (int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock; c0 < total_chunks;
@@ -66,8 +73,13 @@ __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
         const uint32_t q = cpr == 1 ? lc : __umulhi(lc, magic);
         const uint32_t col = lc - q * cpr;
         const int64_t src_row = int64_t(index[row0 + q]);
-        const int64_t g = src_row * row_bytes + int64_t(col) * VEC;
-        val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+        if (src_row >= row_lo && src_row < row_hi) {
+          const int64_t g = src_row * row_bytes + int64_t(col) * VEC;
+          val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+        } else {
+          val[u] = C(0);
+          bad = true;
+        }
       }
     }
 #pragma unroll
@@ -76,6 +88,7 @@ __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
       if (ok[u]) __builtin_nontemporal_store(val[u], reinterpret_cast<C*>(out + (c0 + t) * VEC));
     }
   }
+  if (bad && bad_index) *bad_index = 1;
 }
 
 // Rows wider than kMaxFlatChunksPerRow chunks: a block owns one segment of
@@ -84,18 +97,24 @@ template <int VEC, int TIER, typename IndexT>
 __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, int64_t cpr, int64_t blocks_per_row, const IndexT* __restrict__ index,
-    const int64_t* __restrict__ n_rows_dev, char* __restrict__ out) {
+    const int64_t* __restrict__ n_rows_dev, int64_t row_lo, int64_t row_hi, int64_t* __restrict__ bad_index,
+    char* __restrict__ out) {
   using C = typename Chunk<VEC>::type;
   const int64_t row = int64_t(blockIdx.x) / blocks_per_row;
   if (n_rows_dev && row >= *n_rows_dev) return;
   const int64_t seg = int64_t(blockIdx.x) - row * blocks_per_row;
   const int64_t src_row = int64_t(index[row]);
+  const bool in_range = src_row >= row_lo && src_row < row_hi;
+  if (!in_range && bad_index && threadIdx.x == 0) *bad_index = 1;
 #pragma unroll
   for (int u = 0; u < kGatherUnroll; ++u) {
     const int64_t col = seg * kChunksPerBlock + u * kGatherThreads + threadIdx.x;
     if (col < cpr) {
-      const int64_t g = src_row * row_bytes + col * VEC;
-      C v = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+      C v = C(0);
+      if (in_range) {
+        const int64_t g = src_row * row_bytes + col * VEC;
+        v = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+      }
       *reinterpret_cast<C*>(out + row * row_bytes + col * VEC) = v;
     }
   }
@@ -103,9 +122,14 @@ __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
 
 template <int VEC, int TIER, typename IndexT>
 dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index, int64_t n,
-                         const int64_t* n_dev, void* out, hipStream_t st) {
+                         const int64_t* n_dev, int64_t* bad_index, void* out, hipStream_t st) {
   const int64_t cpr = row_bytes / VEC;
   const int64_t thr_bytes = v.threshold * v.elem_bytes;
+  // rows the tier holds whole: the device tier the rows that end at or before the boundary, the
+  // host tier the rows that begin at or after it (a straddling row is served by the "any" kernel)
+  const int64_t n_rows = v.total * v.elem_bytes / row_bytes;
+  const int64_t row_lo = TIER == DGS_TIER_HOST ? (thr_bytes + row_bytes - 1) / row_bytes : 0;
+  const int64_t row_hi = TIER == DGS_TIER_DEVICE ? thr_bytes / row_bytes : n_rows;
   const char* dev = static_cast<const char*>(v.dev);
   const char* host = static_cast<const char*>(v.host);
   if (cpr <= kMaxFlatChunksPerRow) {
@@ -118,20 +142,21 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
     if (blocks < tiles)
       hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, true>), dim3(uint32_t(blocks)),
                          dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
-                         magic, static_cast<const IndexT*>(index), total_chunks, n_dev,
-                         static_cast<char*>(out));
+                         magic, static_cast<const IndexT*>(index), total_chunks, n_dev, row_lo, row_hi,
+                         bad_index, static_cast<char*>(out));
     else
       hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, false>), dim3(uint32_t(blocks)),
                          dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
-                         magic, static_cast<const IndexT*>(index), total_chunks, n_dev,
-                         static_cast<char*>(out));
+                         magic, static_cast<const IndexT*>(index), total_chunks, n_dev, row_lo, row_hi,
+                         bad_index, static_cast<char*>(out));
   } else {
     const int64_t bpr = (cpr + kChunksPerBlock - 1) / kChunksPerBlock;
     DGS_REQUIRE(n * bpr <= 0x7fffffff, DGS_ERR_UNSUPPORTED, "gather: %lld rows of %lld B exceed one launch",
                 (long long)n, (long long)row_bytes);
     hipLaunchKernelGGL((gather_wide_kernel<VEC, TIER, IndexT>), dim3(uint32_t(n * bpr)),
                        dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, cpr, bpr,
-                       static_cast<const IndexT*>(index), n_dev, static_cast<char*>(out));
+                       static_cast<const IndexT*>(index), n_dev, row_lo, row_hi, bad_index,
+                       static_cast<char*>(out));
   }
   DGS_LAUNCH_CHECK();
   return DGS_OK;
@@ -139,20 +164,22 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
 
 template <int VEC, int TIER>
 dgs_status dispatch_index(const dgs_view& v, int64_t row_bytes, const void* index,
-                          int32_t index_bytes, int64_t n, const int64_t* n_dev, void* out, hipStream_t st) {
-  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, out, st)
-                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, out, st);
+                          int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t* bad, void* out,
+                          hipStream_t st) {
+  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, bad, out, st)
+                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, bad, out, st);
 }
 
 template <int TIER>
 dgs_status dispatch_vec(int vec, const dgs_view& v, int64_t row_bytes, const void* index,
-                        int32_t index_bytes, int64_t n, const int64_t* n_dev, void* out, hipStream_t st) {
+                        int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t* bad, void* out,
+                        hipStream_t st) {
   switch (vec) {
-    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
-    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
-    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
-    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
-    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
   }
 }
 
@@ -253,7 +280,7 @@ __global__ __launch_bounds__(kSplitThreads) void split_scatter_kernel(
 
 namespace {
 dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_t index_bytes, int64_t n,
-                        const int64_t* n_dev, void* out, int32_t tier, void* stream) {
+                        const int64_t* n_dev, void* out, int32_t tier, int64_t* bad, void* stream) {
   using namespace dgs;
   DGS_REQUIRE(width_ok(index_bytes), DGS_ERR_INVALID, "gather: index width %d is not 4 or 8", index_bytes);
   DGS_REQUIRE(n >= 0 && row_elems > 0, DGS_ERR_INVALID, "gather: n=%lld row_elems=%lld", (long long)n,
@@ -267,30 +294,34 @@ dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_
   // an "any" gather over a single-tier store needs no per-chunk test
   if (tier == DGS_TIER_ANY && v.threshold == v.total) tier = DGS_TIER_DEVICE;
   if (tier == DGS_TIER_ANY && v.threshold == 0) tier = DGS_TIER_HOST;
+  // A row that straddles the boundary is listed as a host row by dgs_split_index; it begins in
+  // the device slice, so the host-only address arithmetic would reach in front of the host slice
+  // (as upstream's HostAt does, src/chunk_tensor.h:56-58).  Such a store is served chunk by chunk.
+  if (tier == DGS_TIER_HOST && v.threshold > 0 && v.threshold % row_elems != 0) tier = DGS_TIER_ANY;
   DGS_REQUIRE(tier == DGS_TIER_HOST || v.dev != nullptr, DGS_ERR_INVALID, "gather: store has no device slice");
   DGS_REQUIRE(tier == DGS_TIER_DEVICE || v.host != nullptr, DGS_ERR_INVALID, "gather: store has no host slice");
   const int64_t row_bytes = row_elems * v.elem_bytes;
   const int vec = pick_vec(v, row_bytes, out, tier);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (tier) {
-    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, out, st);
-    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, out, st);
-    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, out, st);
+    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
   }
 }
 }  // namespace
 
 DGS_API dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
                                    int32_t index_bytes, int64_t n, void* out, int32_t tier,
-                                   void* stream) {
-  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, out, tier, stream);
+                                   int64_t* bad_index, void* stream) {
+  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, out, tier, bad_index, stream);
 }
 
 DGS_API dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
                                        int32_t index_bytes, int64_t n_max, const int64_t* n_rows_dev,
-                                       void* out, int32_t tier, void* stream) {
+                                       void* out, int32_t tier, int64_t* bad_index, void* stream) {
   DGS_REQUIRE(n_rows_dev != nullptr, DGS_ERR_INVALID, "gather_dyn: null n_rows_dev");
-  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, out, tier, stream);
+  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, out, tier, bad_index, stream);
 }
 
 DGS_API size_t dgs_split_index_workspace_bytes(int64_t n) {

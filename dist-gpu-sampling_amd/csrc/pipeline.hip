@@ -33,7 +33,6 @@
 // Off the critical path, as surplus blocks of later launches: per-row pick counts are
 // scanned per 256-row tile, and the packed edge list (src_local, dst_local) is written
 // (rank of a pick = rank recorded at its id's smallest position).
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -50,7 +49,11 @@ constexpr int kPosItems = 4;
 constexpr int kPosTile = kBlock * kPosItems;   // padded positions per flag/compact block
 constexpr uint32_t kFirstBit = 0x80000000u;
 constexpr uint32_t kInvalidSlot = 0xffffffffu; // padded position that holds no pick
-constexpr uint32_t kBadRow = 0xffffffffu;      // row_cnt marker: degree >= 2^32
+// row_cnt markers of rows that make the call fail (bit (kBadRow - marker) of the hop's flag word)
+constexpr uint32_t kBadRow = 0xffffffffu;      // degree >= 2^32, or offsets outside the edge array
+constexpr uint32_t kBadSeed = 0xfffffffeu;     // the seed id is not a row of the graph
+constexpr uint32_t kBadPick = 0xfffffffdu;     // a picked neighbour id is outside what the table holds
+__device__ __forceinline__ bool is_bad_row(uint32_t row_cnt) { return row_cnt >= kBadPick; }
 constexpr int kMaxPicks = 64;
 constexpr int64_t kMaxPositions = int64_t(1) << 30;
 constexpr int64_t kInlineTiles = 2048;         // above this a separate scan launch is used
@@ -75,7 +78,7 @@ struct Hop {
   const int64_t* prev_nnz;  // device scalar: edges of the previous hop (NULL in hop 0)
   int64_t* n_unique;        // device scalar: frontier size after this hop
   int64_t* nnz;             // device scalar: edges of this hop
-  int64_t* flags;           // device scalar: non-zero on a bad row
+  int64_t* flags;           // device scalar: bit 0 degree, bit 1 seed id, bit 2 picked id of a bad row
   int64_t* host_sizes;      // optional pinned mirror of the whole sizes array (NULL: none)
   int32_t n_hops;           // layout of the mirror: [0..H] seeds, then H edge counts, then H flags
   int32_t pad0_;
@@ -129,6 +132,19 @@ __device__ __forceinline__ T block_sum(T v, T* lds /* NT/64 */) {
   return s;
 }
 
+template <int NT>
+__device__ __forceinline__ int block_or(int v, int* lds /* NT/64 */) {
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) v |= __shfl_xor(v, d, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
+  __syncthreads();
+  int s = 0;
+#pragma unroll
+  for (int w = 0; w < NT / kWave; ++w) s |= lds[w];
+  __syncthreads();
+  return s;
+}
+
 // ---- packed edge list of one hop (off the critical path) -----------------------------
 
 // One block per 256-row tile: scan of the rows' pick counts.
@@ -142,7 +158,7 @@ __device__ __forceinline__ void offsets_tile(const Hop& h, int tile) {
   int c = 0;
   if (i < s) {
     const uint32_t rc = h.row_cnt[i];
-    if (rc == kBadRow) bad = 1; else c = int(rc);
+    if (is_bad_row(rc)) atomicOr(&bad, 1 << (kBadRow - rc)); else c = int(rc);
   }
   int total;
   const int ex = block_exclusive_scan<kBlock, int>(c, &total, lds);
@@ -180,7 +196,7 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   const int64_t i = tile * kRowTile + r;
   if (r >= kRowTile || i >= s) return;
   const uint32_t rc = h.row_cnt[i];
-  if (rc == kBadRow || uint32_t(l) >= rc) return;
+  if (is_bad_row(rc) || uint32_t(l) >= rc) return;
   const int64_t o = prefix + h.row_off[i] + l;
   const int64_t p = h.pos_base + seed_part(h, s) + i * k + l;
   static_cast<IdT*>(h.src_local)[o] = IdT(rank_of(h, table, p, h.slot[p]));
@@ -201,21 +217,28 @@ __device__ __forceinline__ void mark_lost(const Hop& h, uint32_t displaced) {
 
 // What becomes of padded position p: with a pick (edge `edge` of the graph) the picked id goes
 // into the table and p's slot word is recorded; without one the position is marked empty.
+// Returns false when the picked id is one the table cannot hold (the position then stays empty
+// and the caller marks the row bad): the id is checked before it addresses anything.
 template <typename IdT, typename TableT>
-__device__ __forceinline__ void emit_pick(const Hop& h, const TableT& table, const TierView<IdT>& indices, int64_t p,
+__device__ __forceinline__ bool emit_pick(const Hop& h, const TableT& table, const TierView<IdT>& indices, int64_t p,
                                           bool have, int64_t edge, bool look_first) {
   uint32_t word = kInvalidSlot;
+  bool ok = true;
   if (have) {
     const IdT col = indices.at(edge);
-    bool first;
-    uint32_t displaced;
-    word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
-    if (h.index != 0) {
-      if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
-      mark_lost(h, displaced);
+    ok = table.holds(col);
+    if (ok) {
+      bool first;
+      uint32_t displaced;
+      word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
+      if (h.index != 0) {
+        if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
+        mark_lost(h, displaced);
+      }
     }
   }
   h.slot[p] = word;
+  return ok;
 }
 
 // Ids that repeat a lot (hub sources) are cheaper to insert with a look at the entry first;
@@ -242,24 +265,32 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   const int group_lane0 = (threadIdx.x & (kWave - 1)) - l;
   const IdT seed = static_cast<const IdT*>(h.seeds)[i];
   const int64_t row = int64_t(seed);
-  const int64_t b = int64_t(indptr.at(row));
-  const int64_t e = int64_t(indptr.at(row + 1));
-  const int64_t deg64 = e - b;
-  const bool bad = deg64 < 0 || deg64 > 0xffffffffLL;
+  // nothing is addressed by an id or an offset before it has been checked
+  const bool seed_ok = row_in_range(indptr, row) && table.holds(seed);
+  int64_t b = 0, deg64 = 0;
+  if (seed_ok) {
+    b = int64_t(indptr.at(row));
+    deg64 = int64_t(indptr.at(row + 1)) - b;
+  }
+  const bool bad = deg64 < 0 || deg64 > 0xffffffffLL || b < 0 || b + deg64 > indices.n;
   const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;
   const bool look_first = look_before_insert(h, s);
-  if (l == 0) {
-    h.row_cnt[i] = bad ? kBadRow : (replace ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
-    if (h.index == 0) {  // the caller's seeds open the mapping list; flag() decides their first bits
-      bool first;
-      uint32_t displaced;
-      h.slot[h.pos_base + i] = table.insert_min(seed, uint32_t(h.pos_base + i), &first, &displaced);
-    }
+  if (l == 0 && h.index == 0) {  // the caller's seeds open the mapping list; flag() decides their first bits
+    bool first;
+    uint32_t displaced;
+    h.slot[h.pos_base + i] =
+        seed_ok ? table.insert_min(seed, uint32_t(h.pos_base + i), &first, &displaced) : kInvalidSlot;
   }
   uint32_t pos;
   const bool have = pick_position<G>(deg, k, replace, l, group_lane0, rng_seed, h.rng_stream, row, &pos);
-  if (l < k) emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, have, b + pos, look_first);
+  bool pick_ok = true;
+  if (l < k) pick_ok = emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, have, b + pos, look_first);
+  constexpr uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << (G & 63)) - 1);
+  const bool picks_ok = ((__ballot(!pick_ok) >> group_lane0) & group_mask) == 0;
+  if (l == 0)
+    h.row_cnt[i] = !seed_ok ? kBadSeed : bad ? kBadRow : !picks_ok ? kBadPick
+                 : (replace ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
 }
 
 // Virtual blocks [0, fill_blocks): seed rows of this hop; then relabel_count blocks writing the
@@ -318,21 +349,25 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
   uint32_t deg = 0;
   bool bad = false;
   IdT seed = 0;
+  bool seed_ok = true;
   if (i < s) {
     seed = static_cast<const IdT*>(h.seeds)[i];
-    b = int64_t(indptr.at(int64_t(seed)));
-    const int64_t deg64 = int64_t(indptr.at(int64_t(seed) + 1)) - b;
-    bad = deg64 < 0 || deg64 > 0xffffffffLL;
+    // nothing is addressed by an id or an offset before it has been checked
+    seed_ok = row_in_range(indptr, int64_t(seed)) && table.holds(seed);
+    int64_t deg64 = 0;
+    if (seed_ok) {
+      b = int64_t(indptr.at(int64_t(seed)));
+      deg64 = int64_t(indptr.at(int64_t(seed) + 1)) - b;
+    }
+    bad = deg64 < 0 || deg64 > 0xffffffffLL || b < 0 || b + deg64 > indices.n;
     deg = bad ? 0u : uint32_t(deg64);
   }
   const bool look_first = look_before_insert(h, s);
-  if (i < s && l == 0) {
-    h.row_cnt[i] = bad ? kBadRow : (REPLACE ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
-    if (h.index == 0) {
-      bool first_seen;
-      uint32_t displaced;
-      h.slot[h.pos_base + i] = table.insert_min(seed, uint32_t(h.pos_base + i), &first_seen, &displaced);
-    }
+  if (i < s && l == 0 && h.index == 0) {
+    bool first_seen;
+    uint32_t displaced;
+    h.slot[h.pos_base + i] =
+        seed_ok ? table.insert_min(seed, uint32_t(h.pos_base + i), &first_seen, &displaced) : kInvalidSlot;
   }
   // rows that are copied need no work; long rows are queued and written by the other launch
   const bool is_long = deg > long_row<kWave>() && (REPLACE || deg > uint32_t(k));
@@ -356,8 +391,14 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
     const uint32_t parked = __shfl(won, l, kWave);
     if (mine == r) pick = parked;
   }
+  bool pick_ok = true;
   if (i < s && l < k && !is_long)
-    emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, pick < deg, b + pick, look_first);
+    pick_ok = emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, pick < deg, b + pick, look_first);
+  const uint64_t row_mask = lanes == kWave ? ~uint64_t(0) : ((uint64_t(1) << lanes) - 1);
+  const bool picks_ok = ((__ballot(!pick_ok) >> (mine * lanes)) & row_mask) == 0;
+  if (i < s && l == 0)
+    h.row_cnt[i] = !seed_ok ? kBadSeed : bad ? kBadRow : !picks_ok ? kBadPick
+                 : (REPLACE ? (deg == 0 ? 0u : uint32_t(k)) : (deg < uint32_t(k) ? deg : uint32_t(k)));
 }
 
 // Same layout of virtual blocks as hop_fill_kernel (fill, previous hop's edge list, clearing).
@@ -400,11 +441,13 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
     const int64_t p0 = h.pos_base + seed_part(h, s) + i * k;
     if (REPLACE) {
       draw_long_row(lds, probs, b, int64_t(deg), int64_t(k), rng_seed, h.rng_stream, row,
-                    [&](int64_t j, int64_t pick) { emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first); });
+                    [&](int64_t j, int64_t pick) {
+                      if (!emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first)) h.row_cnt[i] = kBadPick;
+                    });
     } else {
       const uint32_t pos = race_long_row(lds, probs, b, deg, k, rng_seed, h.rng_stream, row);
       const int l = threadIdx.x;  // wave 0 holds the winners
-      if (l < k) emit_pick<IdT>(h, table, indices, p0 + l, pos < deg, b + pos, look_first);
+      if (l < k && !emit_pick<IdT>(h, table, indices, p0 + l, pos < deg, b + pos, look_first)) h.row_cnt[i] = kBadPick;
     }
   }
 }
@@ -490,22 +533,23 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, const T
     // this hop's lengths, written even when there is nothing to do: frontier size, edge count
     // (row tiles were scanned by the surplus blocks of the flag launch) and error flag
     const int64_t row_tiles = (s + kRowTile - 1) / kRowTile;
-    int64_t edges = 0, bad = 0;
+    int64_t edges = 0;
+    int bad = 0;
     for (int64_t j = threadIdx.x; j < row_tiles; j += kBlock) {
       edges += h.tile_sum[j];
-      bad += h.tile_flag[j];
+      bad |= h.tile_flag[j];
     }
     edges = block_sum<kBlock, int64_t>(edges, lds64);
-    bad = block_sum<kBlock, int64_t>(bad, lds64);
+    bad = block_or<kBlock>(bad, lds);
     if (threadIdx.x == 0) {
       *h.n_unique = rank0 + all;
       *h.nnz = edges;
-      *h.flags = bad != 0;
+      *h.flags = bad;
       if (h.host_sizes) {
         if (h.index == 0) h.host_sizes[0] = s;
         h.host_sizes[h.index + 1] = rank0 + all;
         h.host_sizes[h.n_hops + 1 + h.index] = edges;
-        h.host_sizes[2 * h.n_hops + 1 + h.index] = bad != 0;
+        h.host_sizes[2 * h.n_hops + 1 + h.index] = bad;
       }
     }
   }
@@ -589,7 +633,7 @@ dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, in
     // ids fit the packed slot when every node id is below 2^32 - 1
     p->kind = id_bytes == 4 || (n_nodes >= 0 && n_nodes < 0xffffffffLL) ? TableKind::kPacked : TableKind::kSplit;
     // test hook: exercise the split (id array + value array) table on small graphs
-    if (id_bytes == 8 && getenv("DGS_FORCE_SPLIT_TABLE") != nullptr) p->kind = TableKind::kSplit;
+    if (id_bytes == 8 && debug_option(DGS_DEBUG_FORCE_SPLIT_TABLE) != 0) p->kind = TableKind::kSplit;
     p->capacity = table_capacity(p->s_max[n_hops]);
     p->table_bytes = size_t(p->capacity) * (p->kind == TableKind::kPacked ? 8 : size_t(id_bytes) + 4);
   }
@@ -761,8 +805,8 @@ dgs_status run_blocks_table(const Plan& p, Hop* hops, void* hash_table, void* no
                             const dgs_view& indptr, const dgs_view& indices, const dgs_view* probs, bool replace,
                             uint64_t rng_seed, void** sizes_ticket, hipStream_t st) {
   if (p.kind == TableKind::kDirect)
-    return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch), indptr, indices,
-                                                   probs, replace, rng_seed, sizes_ticket, st);
+    return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch, uint32_t(indptr.total - 1)),
+                                                   indptr, indices, probs, replace, rng_seed, sizes_ticket, st);
   const int64_t n16 = int64_t(p.table_bytes / 16);
   hipLaunchKernelGGL(clear_kernel, dim3(capped_grid((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                      static_cast<uint4*>(hash_table), n16);

@@ -7,10 +7,12 @@
 //   scan  : one block turns the tile totals into tile offsets and the edge count;
 //   fill  : num_picks <= 64: a group of G lanes per seed row over the whole grid (G = 8..64,
 //           the smallest power of two holding num_picks), so a wave64 serves 64/G rows;
-//           larger num_picks: one wave per row, Floyd's kept set in LDS.
+//           larger num_picks: one wave per row, Floyd's kept set in LDS (num_picks <= 2048) or
+//           in the row's own output slots (any num_picks).
 // Random picks follow the "dgs-philox-1" contract: every (seed, stream, row, draw) names one
 // Philox block, so results do not depend on the launch shape.
 #include <mutex>
+#include <type_traits>
 
 #include "common.h"
 #include "picks.h"
@@ -49,7 +51,7 @@ dgs_status static_scratch_of(void** out) {
 constexpr int kMaxGroupPicks = 64;   // fill_group_kernel handles num_picks <= 64
 constexpr int kMaxLdsPicks = 2048;   // fill_wave_kernel keeps Floyd's set in LDS
 constexpr int kFlagDegree = 1;       // some row has degree >= 2^32
-constexpr int kFlagPicks = 2;        // deg > num_picks > kMaxLdsPicks without replacement
+constexpr int kFlagSeed = 2;         // some seed id is not a row of the graph
 
 template <typename IdT, typename PtrT>
 __global__ __launch_bounds__(kTile) void sample_count_kernel(
@@ -64,12 +66,15 @@ __global__ __launch_bounds__(kTile) void sample_count_kernel(
   int64_t c = 0;
   if (i < n_seeds) {
     const int64_t row = int64_t(seeds[i]);
-    const int64_t b = int64_t(indptr.at(row));
-    const int64_t e = int64_t(indptr.at(row + 1));
-    int64_t deg = e - b;
+    int64_t b = 0, deg = 0;
     int bad = 0;
-    if (deg < 0 || deg > 0xffffffffLL) { bad |= kFlagDegree; deg = 0; }
-    if (!replace && k > kMaxLdsPicks && deg > k) { bad |= kFlagPicks; deg = 0; }
+    if (row_in_range(indptr, row)) {  // checked before the offsets are read
+      b = int64_t(indptr.at(row));
+      deg = int64_t(indptr.at(row + 1)) - b;
+      if (deg < 0 || deg > 0xffffffffLL) { bad |= kFlagDegree; deg = 0; }
+    } else {
+      bad |= kFlagSeed;
+    }
     if (bad) atomicOr(&flag, bad);
     row_start[i] = b;
     row_deg[i] = uint32_t(deg);
@@ -124,7 +129,7 @@ __global__ __launch_bounds__(kTile) void fill_group_kernel(
 }
 
 // Any num_picks: one wave per row, lanes stride over the slots; Floyd's kept set lives in LDS
-// (num_picks <= kMaxLdsPicks whenever it is needed: larger requests were zeroed by the count pass).
+// (num_picks <= kMaxLdsPicks; the launcher sends larger requests to fill_wave_global_kernel).
 template <typename IdT>
 __global__ __launch_bounds__(kTile) void fill_wave_kernel(
     const IdT* __restrict__ seeds, int64_t n_seeds, const int64_t* __restrict__ row_start,
@@ -182,6 +187,77 @@ __global__ __launch_bounds__(kTile) void fill_wave_kernel(
   }
 }
 
+// num_picks above kMaxLdsPicks: one wave per row, Floyd's kept set lives in the row's own slots
+// of out_cols (a position fits an id slot) and is turned into neighbour ids at the end.  Slots are
+// resolved 64 at a time: every lane first compares its candidate with all positions kept by
+// earlier batches (read 64 at a time, handed round with __shfl), then the batch settles its own
+// order lane by lane as pick_position does.
+template <typename IdT>
+__global__ __launch_bounds__(kTile) void fill_wave_global_kernel(
+    const IdT* __restrict__ seeds, int64_t n_seeds, const int64_t* __restrict__ row_start,
+    const uint32_t* __restrict__ row_deg, const int64_t* __restrict__ row_off,
+    const int64_t* __restrict__ tile_off, TierView<IdT> indices, int64_t k, bool replace, uint64_t rng_seed,
+    uint32_t rng_stream, IdT* __restrict__ out_rows, IdT* __restrict__ out_cols) {
+  using U = typename std::make_unsigned<IdT>::type;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t i = int64_t(blockIdx.x) * (kTile / kWave) + wave;
+  if (i >= n_seeds) return;  // whole waves leave together
+  const int64_t start = row_start[i];
+  const int64_t off = tile_off[i / kTile] + row_off[i];
+  const int64_t row = int64_t(seeds[i]);
+  const uint32_t deg = row_deg[i];
+  if (replace) {
+    if (deg > 0) {
+      for (int64_t s = lane; s < k; s += kWave) {
+        const uint32_t p = philox_bounded(rng_seed, rng_stream, row, uint32_t(s), deg);
+        out_rows[off + s] = IdT(row);
+        out_cols[off + s] = indices.at(start + p);
+      }
+    }
+    return;
+  }
+  if (int64_t(deg) <= k) {
+    for (uint32_t s = lane; s < deg; s += kWave) {
+      out_rows[off + s] = IdT(row);
+      out_cols[off + s] = indices.at(start + s);
+    }
+    return;
+  }
+  U* kept = reinterpret_cast<U*>(out_cols + off);  // [k] positions, zero-extended
+  const uint32_t base_top = deg - uint32_t(k);
+  for (int64_t s0 = 0; s0 < k; s0 += kWave) {
+    const int64_t s = s0 + lane;
+    const bool live = s < k;
+    const uint32_t top = base_top + uint32_t(s);
+    uint32_t cand = 0xffffffffu;  // no kept position has this value: deg <= 2^32 - 1
+    if (live) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(s), top + 1u);
+    // against the batches before this one (their stores were fenced below)
+    bool hit = false;
+    for (int64_t q0 = 0; q0 < s0; q0 += kWave) {
+      const uint32_t mine = uint32_t(kept[q0 + lane]);  // s0 is a multiple of 64: always in range
+#pragma unroll 8
+      for (int j = 0; j < kWave; ++j) hit |= __shfl(mine, j, kWave) == cand;
+    }
+    uint32_t keep = hit ? top : cand;
+    // inside the batch: slot t sees what the slots before it finally kept
+    const int batch = int(k - s0 < kWave ? k - s0 : kWave);
+    for (int t = 1; t < batch; ++t) {
+      const uint32_t c = __shfl(cand, t, kWave);
+      const bool clash = __ballot(keep == c && lane < t) != 0;
+      if (lane == t && clash && !hit) keep = top;
+    }
+    if (live) kept[s] = U(keep);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
+  for (int64_t s = lane; s < k; s += kWave) {
+    out_rows[off + s] = IdT(row);
+    out_cols[off + s] = indices.at(start + int64_t(uint32_t(kept[s])));
+  }
+}
+
 template <typename IdT, typename PtrT>
 dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr, int64_t k, bool replace,
                      const SampleWorkspace& w, int64_t* nnz_dev, hipStream_t st) {
@@ -221,8 +297,14 @@ dgs_status run_fill(const void* seeds, int64_t n_seeds, const dgs_view& indices,
     else if (kk <= 16) launch_group<IdT, 16>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
     else if (kk <= 32) launch_group<IdT, 32>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
     else launch_group<IdT, 64>(seeds, n_seeds, w, indices, kk, replace, rng_seed, rng_stream, out_rows, out_cols, st);
+  } else if (k > kMaxLdsPicks) {
+    const int64_t blocks = (n_seeds + kTile / kWave - 1) / (kTile / kWave);
+    hipLaunchKernelGGL((fill_wave_global_kernel<IdT>), dim3(uint32_t(blocks)), dim3(kTile), 0, st,
+                       static_cast<const IdT*>(seeds), n_seeds, w.row_start, w.row_deg, w.row_off, w.tile_off,
+                       TierView<IdT>(indices), k, replace, rng_seed, rng_stream, static_cast<IdT*>(out_rows),
+                       static_cast<IdT*>(out_cols));
   } else {
-    const int64_t kk = k < kMaxLdsPicks ? k : kMaxLdsPicks;
+    const int64_t kk = k;
     const size_t lds = replace ? 0 : size_t(kTile / kWave) * size_t(kk) * sizeof(uint32_t);
     const int64_t blocks = (n_seeds + kTile / kWave - 1) / (kTile / kWave);
     hipLaunchKernelGGL((fill_wave_kernel<IdT>), dim3(uint32_t(blocks)), dim3(kTile), lds, st,

@@ -24,6 +24,12 @@ void set_error(const char* fmt, ...) {
 // HBM bytes held by live stores (upstream src/cuda_context.h:11-38, made atomic).
 static std::atomic<int64_t> g_allocated{0};
 
+constexpr int kDebugOptions = 2;
+static std::atomic<int64_t> g_debug[kDebugOptions];
+int64_t debug_option(int32_t option) {
+  return option >= 0 && option < kDebugOptions ? g_debug[option].load(std::memory_order_relaxed) : 0;
+}
+
 }  // namespace dgs
 
 struct dgs_store {
@@ -51,7 +57,13 @@ DGS_API const char* dgs_status_name(dgs_status s) {
   }
 }
 
-DGS_API int dgs_abi_version(void) { return 1; }
+DGS_API int dgs_abi_version(void) { return 2; }
+
+DGS_API dgs_status dgs_debug_set(int32_t option, int64_t value) {
+  DGS_REQUIRE(option >= 0 && option < dgs::kDebugOptions, DGS_ERR_INVALID, "debug_set: unknown option %d", option);
+  dgs::g_debug[option].store(value, std::memory_order_relaxed);
+  return DGS_OK;
+}
 
 DGS_API dgs_status dgs_store_split(int64_t total_elems, int32_t elem_bytes, int64_t capacity_bytes,
                                    int64_t* device_elems, int64_t* host_elems) {
@@ -224,6 +236,18 @@ DGS_API dgs_status dgs_ticket_release(void* ticket) {
   DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_release: null ticket");
   std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
   dgs::g_event_pool.push_back(static_cast<hipEvent_t>(ticket));
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_stream_query(void* stream, int32_t* idle) {
+  DGS_REQUIRE(idle != nullptr, DGS_ERR_INVALID, "stream_query: null output");
+  const hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
+  if (e == hipErrorNotReady) {
+    *idle = 0;
+    return DGS_OK;
+  }
+  if (e != hipSuccess) (void)hipGetLastError();  // a handle that names no live stream: nothing can be pending on it
+  *idle = 1;
   return DGS_OK;
 }
 

@@ -42,6 +42,9 @@ struct Table<IdT, true> {
   __host__ __device__ Table(void* base, uint32_t capacity)
       : slots(static_cast<unsigned long long*>(base)), mask(capacity - 1) {}
 
+  // ids the table can hold: 0 .. 2^32 - 2 (the all-ones word marks an empty slot)
+  __device__ __forceinline__ bool holds(IdT key) const { return uint64_t(int64_t(key)) < 0xffffffffull; }
+
   __device__ __forceinline__ uint32_t insert(IdT key, uint32_t idx) const {
     const unsigned long long packed = (static_cast<unsigned long long>(uint32_t(key)) << 32) | idx;
     uint32_t pos = hash_id(uint32_t(key)) & mask;
@@ -110,6 +113,9 @@ struct Table<IdT, false> {
         vals(reinterpret_cast<uint32_t*>(static_cast<char*>(base) + size_t(capacity) * sizeof(IdT))),
         mask(capacity - 1) {}
 
+  // ids the table can hold: every id >= 0 (-1 marks an empty slot)
+  __device__ __forceinline__ bool holds(IdT key) const { return key >= 0; }
+
   __device__ __forceinline__ uint32_t insert(IdT key, uint32_t idx) const {
     using W = typename AtomicWord<IdT>::type;
     uint32_t pos = hash_id(uint64_t(int64_t(key))) & mask;
@@ -160,10 +166,14 @@ template <typename IdT>
 struct DirectTable {
   unsigned long long* entries;
   uint32_t tag;  // ~epoch
+  uint32_t n;    // entries: one per node
   static constexpr uint32_t kNoSlot = 0xffffffffu;
 
-  __host__ __device__ DirectTable(void* base, uint32_t epoch)
-      : entries(static_cast<unsigned long long*>(base)), tag(~epoch) {}
+  __host__ __device__ DirectTable(void* base, uint32_t epoch, uint32_t n_nodes)
+      : entries(static_cast<unsigned long long*>(base)), tag(~epoch), n(n_nodes) {}
+
+  // ids the table has an entry for; everything else must be kept away from insert_min
+  __device__ __forceinline__ bool holds(IdT key) const { return uint64_t(int64_t(key)) < uint64_t(n); }
 
   // `look_first`: read the entry before the atomic.  A value already below v (a stale read can
   // only be larger than the truth) settles the matter without an atomic, which is what keeps

@@ -5,7 +5,6 @@
 // group of G lanes (G = 16, 32 or 64, so a wave64 serves up to four rows; chosen on the host from
 // num_picks); rows of more than 32 G neighbours are queued (one atomic per such row) and then
 // handled by a second launch that spends a 1024-thread block on a row.
-#include <cstdlib>
 
 #include "common.h"
 #include "race.h"
@@ -171,9 +170,8 @@ dgs_status run_fill_weighted(const void* seeds_v, int64_t n_seeds, const dgs_vie
   // Without replacement a wider group seeds its race from more candidates at once, which pays
   // as soon as more than a handful of entries are kept.
   int group = replace ? (k <= 16 ? 16 : (k <= 32 ? 32 : 64)) : (k <= 4 ? 16 : 64);
-  if (const char* forced = std::getenv("DGS_WEIGHTED_GROUP")) {  // test hook: 16, 32 or 64
-    const int f = std::atoi(forced);
-    if ((f == 16 || f == 32 || f == 64) && (replace || k <= f)) group = f;
+  if (const int64_t f = debug_option(DGS_DEBUG_WEIGHTED_GROUP)) {  // test hook: 16, 32 or 64
+    if ((f == 16 || f == 32 || f == 64) && (replace || k <= f)) group = int(f);
   }
   if (group == 16)
     launch_groups<IdT, 16>(seeds, n_seeds, a, indices, probs, k, replace, rng_seed, rng_stream, out_rows, out_cols, st);

@@ -2,6 +2,7 @@
 (oppo_bench/single_node/utils/chunktensor_sampler.py) at world size 1, without
 DGL: a block is a plain record instead of a DGLBlock.
 """
+import threading
 from collections import deque, namedtuple
 
 import torch
@@ -12,8 +13,20 @@ Block = namedtuple("Block", ["src_local", "dst_local", "num_src", "num_dst", "sr
 
 
 def set_rng_state(seed, stream=0):
-    """Seeds the sampling generator; the stream advances by one per sampling call."""
+    """Seeds the process-wide sampling generator; its stream advances by one per sampled hop.
+    Samplers made with `seed=` keep their own state and do not touch this one."""
     torch.ops.dgs_ops._CAPI_set_rng_state(int(seed), int(stream))
+
+
+def set_gather_buffer_cap(nbytes):
+    """Largest worst-case feature buffer the fused operators allocate before a batch's sizes are
+    known (default 2 GiB).  Above it a batch waits for its frontier size and gathers into exactly
+    that many rows: memory stays bounded, the host blocks a little earlier."""
+    torch.ops.dgs_ops._CAPI_set_gather_buffer_cap(int(nbytes))
+
+
+# guards the process-wide generator while a sampler with its own state borrows it for a per-hop call
+_rng_lock = threading.Lock()
 
 
 def create_dgs_communicator(group_size=1, local_group=None):
@@ -71,17 +84,34 @@ class ChunkTensorSampler:
     64 (`fused=False` forces the per-hop operators; both give identical results).  With
     `chunk_probs` (a float32 ChunkTensor of edge weights) every hop picks by weight, as
     upstream does (:97-100).
+
+    With `seed` the sampler owns its random state: batch number b (counted per sampler, or given
+    as `batch=` to submit / sample_blocks) draws hop h from stream `b * len(fanouts) + h` of that
+    seed, whatever other samplers or host threads do.  Without it the process-wide generator of
+    set_rng_state is used, as upstream's single global state.
     """
 
     FUSED_MAX_FANOUT = 64
 
-    def __init__(self, fanouts, chunk_indptr, chunk_indices, chunk_probs=None, replace=False, fused=True):
+    def __init__(self, fanouts, chunk_indptr, chunk_indices, chunk_probs=None, replace=False, fused=True,
+                 seed=None):
         self.chunk_indptr = chunk_indptr
         self.chunk_indices = chunk_indices
         self.chunk_probs = chunk_probs
         self.fanouts = list(fanouts)
         self.replace = replace
         self.fused = fused and all(0 <= f <= self.FUSED_MAX_FANOUT for f in self.fanouts)
+        self.seed = None if seed is None else int(seed)
+        self._batches = 0
+        self._count_lock = threading.Lock()
+
+    def _first_stream(self, batch):
+        """Stream of the first hop of a batch drawn from the sampler's own state."""
+        if batch is None:
+            with self._count_lock:
+                batch = self._batches
+                self._batches += 1
+        return int(batch) * len(self.fanouts)
 
     @staticmethod
     def _blocks(seeds, frontiers, srcs, dsts):
@@ -91,15 +121,27 @@ class ChunkTensorSampler:
             seeds = frontier
         return blocks
 
-    def sample_blocks(self, g, seed_nodes, exclude_eids=None):
+    def sample_blocks(self, g, seed_nodes, exclude_eids=None, batch=None):
         """Returns (input_nodes, seed_nodes, blocks); `g` is unused, as upstream.  Host-side
         seed_nodes (what upstream's DataLoader passes) are uploaded by the operator itself."""
-        if self.fused and self.chunk_probs is not None:
-            return self.submit(g, seed_nodes).result()
+        if self.fused and (self.chunk_probs is not None or self.seed is not None):
+            return self.submit(g, seed_nodes, batch=batch).result()
+        if self.seed is not None:  # per-hop operators draw from the process-wide state: lend it ours
+            with _rng_lock:
+                saved = torch.ops.dgs_ops._CAPI_get_rng_state()
+                torch.ops.dgs_ops._CAPI_set_rng_state(self.seed, self._first_stream(batch))
+                try:
+                    return self._sample_blocks_per_hop(seed_nodes)
+                finally:
+                    torch.ops.dgs_ops._CAPI_set_rng_state(*saved)
         if self.fused:
             frontiers, srcs, dsts, seeds = torch.ops.dgs_ops._CAPI_sample_blocks(
                 seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace)
             return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts)
+        return self._sample_blocks_per_hop(seed_nodes)
+
+    def _sample_blocks_per_hop(self, seed_nodes):
+        """The upstream loop itself (chunktensor_sampler.py:93-118), one operator call per step."""
         seeds = seed_nodes.cuda()
         blocks = []
         frontier = seeds
@@ -116,7 +158,7 @@ class ChunkTensorSampler:
             seeds = frontier
         return frontier, seed_nodes, blocks
 
-    def submit(self, g, seed_nodes, chunk_features=None):
+    def submit(self, g, seed_nodes, chunk_features=None, batch=None):
         """Enqueues a batch on the current stream and returns at once (fused path only).  Batches
         submitted on different streams overlap on the GPU: one batch's gather is bound by HBM
         bandwidth, the next batch's sampling by memory transactions, and they share the machine
@@ -124,7 +166,11 @@ class ChunkTensorSampler:
         if not self.fused:
             raise RuntimeError("submit() needs the fused path: every fanout <= 64")
         hop_fanouts = list(reversed(self.fanouts))
-        if self.chunk_probs is not None:
+        if self.seed is not None:
+            handle = torch.ops.dgs_ops._CAPI_sample_blocks_submit(
+                seed_nodes, self.chunk_indptr, self.chunk_indices, self.chunk_probs, hop_fanouts, self.replace,
+                chunk_features, self.seed, self._first_stream(batch))
+        elif self.chunk_probs is not None:
             handle = torch.ops.dgs_ops._CAPI_sample_blocks_weighted_begin(
                 seed_nodes, self.chunk_indptr, self.chunk_indices, self.chunk_probs, hop_fanouts, self.replace,
                 chunk_features)
@@ -144,7 +190,7 @@ class ChunkTensorSampler:
         if not self.fused:
             frontier, _, blocks = self.sample_blocks(g, seed_nodes)
             return frontier, seed_nodes, blocks, chunk_features._CAPI_index(frontier)
-        if self.chunk_probs is not None:
+        if self.chunk_probs is not None or self.seed is not None:
             return self.submit(g, seed_nodes, chunk_features).result()
         frontiers, srcs, dsts, x, seeds = torch.ops.dgs_ops._CAPI_sample_blocks_and_index(
             seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
@@ -213,11 +259,17 @@ class BatchPipeline:
 
     def __call__(self, seed_batches):
         consumer = torch.cuda.current_stream()
-        for st in self.streams:
-            st.wait_stream(consumer)  # whatever produced the seeds and the stores comes first
         queue = deque()
         for i, seeds in enumerate(seed_batches):
-            with torch.cuda.stream(self.streams[i % len(self.streams)]):
+            st = self.streams[i % len(self.streams)]
+            # Seeds on the device may have been made just now on the caller's stream (a generator
+            # that builds them lazily, or uploads them without blocking): the batch's stream waits
+            # for that stream as it stands.  This also orders the batch behind everything else the
+            # caller has enqueued there, so seeds that should overlap with the caller's work are
+            # better passed as host tensors (the operator uploads them on the batch's own stream).
+            if i < len(self.streams) or (torch.is_tensor(seeds) and seeds.is_cuda):
+                st.wait_stream(consumer)
+            with torch.cuda.stream(st):
                 queue.append(self.sampler.submit(None, seeds, self.chunk_features))
             if len(queue) >= len(self.streams):
                 yield self._hand_out(queue.popleft(), consumer)

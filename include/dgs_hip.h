@@ -43,6 +43,17 @@ const char* dgs_last_error(void);
 const char* dgs_status_name(dgs_status s);
 /* ABI version of this header (bumped on incompatible change). */
 int dgs_abi_version(void);
+/*
+ * Test hooks, process-wide: force code paths that small test inputs would not reach by
+ * themselves.  Results never depend on them.  Not for production use.
+ *   DGS_DEBUG_FORCE_SPLIT_TABLE  non-zero: dgs_sample_blocks without a node table uses the
+ *                                id-array + value-array hash table also where ids would fit
+ *                                the packed one
+ *   DGS_DEBUG_WEIGHTED_GROUP     16, 32 or 64: lanes per row of the weighted per-hop fill
+ *                                (0: chosen from num_picks)
+ */
+enum { DGS_DEBUG_FORCE_SPLIT_TABLE = 0, DGS_DEBUG_WEIGHTED_GROUP = 1 };
+dgs_status dgs_debug_set(int32_t option, int64_t value);
 
 /* ------------------------------------------------------------------------ */
 /* Two-tier positional store (ChunkTensor)                                   */
@@ -121,12 +132,18 @@ enum {
  * Replaces IndexFromChunkTensorCUDA / LocalIndex... / HostIndex...
  * (src/cuda/index_with_chunk_tensor.cu:9-53, :110-128/:170-194, :150-168/:223-247).
  * A row that straddles the device/host boundary is resolved per element, like
- * chunk_tensor_wrapper::At (src/chunk_tensor.h:33-42).  `out` holds
- * n * row_elems elements.  index values are not range-checked.
+ * chunk_tensor_wrapper::At (src/chunk_tensor.h:33-42), also for DGS_TIER_HOST
+ * (the reference's HostAt, src/chunk_tensor.h:56-58, reaches in front of the host
+ * slice for such a row).  `out` holds n * row_elems elements.
+ * Index values are checked before they address anything (the reference does not
+ * check, src/cuda/index_with_chunk_tensor.cu:16-23): a row outside the store, or
+ * with DGS_TIER_DEVICE / DGS_TIER_HOST a row the tier does not hold whole, is not
+ * read; its output row is zero bytes and *bad_index (device-visible int64, may be
+ * NULL, never cleared by the library) is set to 1 when the kernel runs.
  */
 dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
                            int32_t index_bytes, int64_t n, void* out,
-                           int32_t tier, void* stream);
+                           int32_t tier, int64_t* bad_index, void* stream);
 
 /*
  * Same gather with the row count read from device memory when the kernel runs:
@@ -138,7 +155,7 @@ dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
 dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
                                int32_t index_bytes, int64_t n_max,
                                const int64_t* n_rows_dev, void* out, int32_t tier,
-                               void* stream);
+                               int64_t* bad_index, void* stream);
 
 /*
  * Stable partition of an index list into (device-resident rows, host-resident
@@ -183,8 +200,11 @@ dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
  *   indices  : view of E ids, elem_bytes == id_bytes
  *   nnz_dev  : device int64[2]; [0] receives the number of emitted edges,
  *              [1] flags: bit 0 = some row has degree >= 2^32, bit 1 = some
- *              row has degree > num_picks > 2048 without replacement.  Flagged
+ *              seed id is not a row of the graph (the reference does not check;
+ *              here the id is tested before it addresses indptr).  Flagged
  *              rows emit nothing; the caller reports DGS_ERR_RANGE.
+ *              Every num_picks is served, as by the reference's reservoir
+ *              kernel (src/cuda/rowwise_sampling.cu:42-99).
  *   workspace: dgs_sample_workspace_bytes(n_seeds) bytes, 256-byte aligned,
  *              shared by the count and the fill of the same hop
  *
@@ -338,7 +358,11 @@ typedef struct dgs_block_out {
  *   sizes_dev              : device int64[3 * n_hops + 1]:
  *                            [0 .. n_hops]                 seeds of hop h (h = n_hops: final frontier size)
  *                            [n_hops + 1 .. 2 n_hops]      edges of hop h
- *                            [2 n_hops + 1 .. 3 n_hops]    non-zero if a row of hop h had degree >= 2^32
+ *                            [2 n_hops + 1 .. 3 n_hops]    error bits of hop h: 1 a row had degree >= 2^32 or
+ *                                                          offsets outside the edge array, 2 a seed id is
+ *                                                          not a row of the graph, 4 a picked neighbour id
+ *                                                          is not a node (each checked before it addresses
+ *                                                          anything; such rows emit nothing)
  *   sizes_host / ticket    : optional (both or neither).  sizes_host is pinned host memory
  *                            that the device can write (hipHostMalloc); the kernels mirror
  *                            sizes_dev into it, and *sizes_ticket marks the point on `stream`
@@ -448,6 +472,11 @@ dgs_status dgs_ticket_record(void* stream, void** ticket);
 dgs_status dgs_ticket_stream_wait(void* stream, void* ticket);
 dgs_status dgs_ticket_wait(void* ticket);
 dgs_status dgs_ticket_release(void* ticket);
+/*
+ * *idle = 1 when everything enqueued on `stream` so far has finished (also when the handle no
+ * longer names a live stream: a destroyed stream has drained), else 0.  Never blocks.
+ */
+dgs_status dgs_stream_query(void* stream, int32_t* idle);
 
 #ifdef __cplusplus
 }

@@ -33,7 +33,7 @@ def test_struct_layouts_match_the_header():
     pkg = load_pkg()
     assert ctypes.sizeof(pkg.capi.View) == 40      # 2 pointers + 2 int64 + 2 int32
     assert ctypes.sizeof(pkg.capi.Segments) == 8 * 8 + 8 * 8 + 8
-    assert pkg.capi.lib.dgs_abi_version() == 1
+    assert pkg.capi.lib.dgs_abi_version() == 2
 
 
 def test_store_split_matches_oracle(oracle):

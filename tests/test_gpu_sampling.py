@@ -76,10 +76,205 @@ def test_sample_edge_cases(pkg, oracle):
     # no seeds at all
     r, c, flags = capi.sample_neighbors(_dev(seeds[:0]), capi.tensor_view(ip), capi.tensor_view(ix), 5, False, 1, 2)
     assert r.numel() == 0 and c.numel() == 0 and flags == 0
-    # fanout above the LDS limit with a row that would need sampling: flagged, row skipped
     r, c, flags = capi.sample_neighbors(_dev(np.array([5], dtype=np.int64)), capi.tensor_view(ip),
                                         capi.tensor_view(ix), 3000, False, 1, 2, two_step=True)
-    assert flags == 0 and r.numel() == 300  # deg 300 <= k: plain copy, nothing to flag
+    assert flags == 0 and r.numel() == 300  # deg 300 <= k: plain copy
+
+
+@pytest.mark.parametrize("id_dtype", [np.int64, np.int32])
+def test_sample_any_fanout_without_replacement(pkg, oracle, id_dtype):
+    # fanouts above what fits the on-chip kept set, on rows that need sampling (upstream's
+    # reservoir kernel takes any num_picks, src/cuda/rowwise_sampling.cu:42-99)
+    capi = pkg.capi
+    deg = np.array([5000, 10, 3001, 3000, 0, 2999, 9000, 2050], dtype=np.int64)
+    indptr = np.zeros(deg.size + 1, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    rng = np.random.default_rng(12)
+    indices = rng.integers(0, 10 ** 6, size=int(indptr[-1])).astype(id_dtype)
+    ip, ix = _dev(indptr), _dev(indices)
+    seeds = np.array([0, 2, 1, 6, 3, 4, 5, 7, 0], dtype=id_dtype)
+    for k in (3000, 2049, 4500):
+        want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, k, False, 0xC0FFEE, 3)
+        for two_step in (False, True):
+            r, c, flags = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, False,
+                                                0xC0FFEE, 3, two_step=two_step)
+            assert flags == 0
+            assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c), (k, two_step)
+        # picks of a sampled row are distinct positions: the row's ids are distinct with high probability,
+        # so check through positions recovered from a row whose neighbour ids are its positions
+    ix2 = _dev(np.concatenate([np.arange(d) for d in deg]).astype(id_dtype))
+    r, c, _ = capi.sample_neighbors(_dev(seeds[:1]), capi.tensor_view(ip), capi.tensor_view(ix2), 3000, False, 9, 9)
+    got = _np(c)
+    assert got.size == 3000 and np.unique(got).size == 3000 and got.min() >= 0 and got.max() < 5000
+    r, c = pkg.ops._CAPI_sample_neighbors(_dev(seeds), ip, _dev(indices), 3000, False)
+    assert r.numel() == sum(min(int(deg[s]), 3000) for s in seeds)
+
+
+def test_seed_ids_outside_the_graph_are_refused(pkg, oracle, graph):
+    # a seed id is checked before it addresses indptr: its row emits nothing, the call is flagged,
+    # the operators raise
+    capi = pkg.capi
+    indptr, indices = graph
+    n = indptr.size - 1
+    ip, ix = _dev(indptr), _dev(indices)
+    good = np.array([5, 17, n - 1, 0], dtype=np.int64)
+    for bad_id in (-1, n, n + 12345, 2 ** 40, -2 ** 50):
+        seeds = np.concatenate([good[:2], [bad_id], good[2:]]).astype(np.int64)
+        want_r, want_c = oracle.sample_neighbors(good, indptr, indices, 6, False, 3, 1)
+        r, c, flags = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), 6, False, 3, 1)
+        assert flags == 2
+        assert np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)  # the other rows are as ever
+        with pytest.raises(RuntimeError, match="seed id"):
+            pkg.ops._CAPI_sample_neighbors(_dev(seeds), ip, ix, 6, False)
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    probs = pkg.create_chunktensor(torch.rand(indices.size) + 0.1, 1, 1 << 40)
+    for sampler in (pkg.ChunkTensorSampler([4, 3], ip_ct, ix_ct), pkg.ChunkTensorSampler([4, 3], ip_ct, ix_ct, fused=False),
+                    pkg.ChunkTensorSampler([4, 3], ip_ct, ix_ct, probs)):
+        for bad_id in (-1, n, 2 ** 33):
+            seeds = torch.tensor([3, bad_id, 9])
+            with pytest.raises(RuntimeError, match="seed id"):
+                sampler.sample_blocks(None, seeds)
+        f, _, _ = sampler.sample_blocks(None, torch.tensor([3, 9]))  # and the sampler still works
+        assert f[:2].tolist() == [3, 9]
+    # int32 ids; hash-table path of the C ABI (no node table)
+    seeds32 = _dev(np.array([1, -5, 2], dtype=np.int32))
+    ix32 = _dev(indices.astype(np.int32))
+    hops, _, flags = capi.sample_blocks(seeds32, capi.tensor_view(ip), capi.tensor_view(ix32), [3, 2], False, 1, 0)
+    assert flags[0] == 2 and flags[1] == 0
+
+
+def test_neighbour_ids_outside_the_graph_are_refused(pkg):
+    # a graph whose edge array holds an id that is no node: with the direct node table the id would
+    # address the table, so it is checked first and the call raises
+    n = 1000
+    rng = np.random.default_rng(4)
+    deg = rng.integers(1, 9, size=n)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    for bad_id in (n, -1, 2 ** 35, -7):
+        indices = rng.integers(0, n, size=int(indptr[-1])).astype(np.int64)
+        indices[indptr[10]] = bad_id  # first neighbour of node 10
+        ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+        ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+        sampler = pkg.ChunkTensorSampler([8, 8], ip_ct, ix_ct)
+        with pytest.raises(RuntimeError, match="neighbour id"):
+            sampler.sample_blocks(None, torch.tensor([10, 11]))
+    # degree and offset checks: an indptr entry pointing past the edge array
+    bad_ptr = indptr.copy()
+    bad_ptr[21:] += 10 ** 9
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(bad_ptr), 1, 1 << 40)
+    with pytest.raises(RuntimeError, match="offsets outside"):
+        pkg.ChunkTensorSampler([8], ip_ct, ix_ct).sample_blocks(None, torch.tensor([30]))
+
+
+def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph):
+    # when the worst-case feature buffer exceeds the cap the operator waits for the frontier size
+    # and gathers into exactly that many rows
+    indptr, indices = graph
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    feats = torch.randn((20000, 48))
+    ft = pkg.create_chunktensor(feats, 1, 1 << 40, cache_rate=0.4)
+    rng = np.random.default_rng(19)
+    seeds = torch.from_numpy(rng.integers(0, 20000, size=600))
+    sampler = pkg.ChunkTensorSampler([9, 6], ip_ct, ix_ct)
+    default_cap = pkg.ops._CAPI_get_gather_buffer_cap()
+    assert default_cap == 2 << 30
+    results = []
+    try:
+        for cap in (default_cap, 0, 600 * 7 * 10 * 48 * 4 - 1, 600 * 7 * 10 * 48 * 4):
+            pkg.set_gather_buffer_cap(cap)
+            pkg.set_rng_state(8, 8)
+            torch.cuda.reset_peak_memory_stats()
+            before = torch.cuda.memory_allocated()
+            f, _, blocks, x = sampler.sample_blocks_and_index(None, seeds, ft)
+            peak = torch.cuda.max_memory_allocated() - before
+            results.append((f.cpu(), x.cpu(), peak, x.untyped_storage().nbytes()))
+            streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+            got = list(pkg.BatchPipeline(sampler, ft, 2, streams=streams)([seeds, seeds.cuda(), seeds]))
+            assert all(torch.equal(g[3].cpu(), feats[g[0].cpu()]) for g in got)
+    finally:
+        pkg.set_gather_buffer_cap(default_cap)
+    o_frontier, _, _ = oracle.sample_blocks(seeds.numpy(), indptr, indices, [9, 6], False, 8, 8)
+    for f, x, _, _ in results:
+        assert np.array_equal(f.numpy(), o_frontier) and torch.equal(x, feats[f])
+    worst = 600 * 7 * 10 * 48 * 4
+    assert results[0][3] == worst and results[3][3] == worst            # ahead of the sizes: worst case
+    assert results[1][3] == results[1][0].numel() * 48 * 4 == results[2][3]  # capped: exactly the frontier
+    assert results[1][2] < results[0][2]
+
+
+def test_samplers_with_their_own_generator(pkg, oracle, graph):
+    # a sampler made with seed= draws batch b from its own streams whatever other threads do
+    import threading
+    indptr, indices = graph
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    rng = np.random.default_rng(2)
+    fanouts = [5, 4]
+    batches = [rng.integers(0, 20000, size=400).astype(np.int64) for _ in range(12)]
+    samplers = [pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, seed=1000 + t) for t in range(3)]
+    samplers.append(pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, seed=2000, fused=False))
+    results = [dict() for _ in samplers]
+    errors = []
+    pkg.set_rng_state(555, 5)
+
+    def work(t):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for i, b in enumerate(batches):
+                    results[t][i] = samplers[t].sample_blocks(None, torch.from_numpy(b))
+        except Exception as e:
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(len(samplers))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for t, sampler in enumerate(samplers):
+        for i, b in enumerate(batches):
+            want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, fanouts, False, sampler.seed, 2 * i)
+            assert np.array_equal(_np(results[t][i][0]), want_f), (t, i)
+            _check_blocks(results[t][i][2], want_blocks)
+    assert pkg.ops._CAPI_get_rng_state() == [555, 5]  # the process-wide generator was left as it was
+    # an explicit batch number names the streams
+    f, _, _ = samplers[0].sample_blocks(None, torch.from_numpy(batches[3]), batch=7)
+    want_f, _, _ = oracle.sample_blocks(batches[3], indptr, indices, fanouts, False, 1000, 14)
+    assert np.array_equal(_np(f), want_f)
+
+
+def test_node_tables_move_to_new_streams(pkg, oracle, graph):
+    # streams that come and go (one per epoch, say): once four streams have sampled from a graph,
+    # a new stream takes over the table of a stream that has nothing left to run
+    indptr, indices = graph
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    sampler = pkg.ChunkTensorSampler([6, 5, 4], ip_ct, ix_ct, seed=77)
+    rng = np.random.default_rng(6)
+    seeds = rng.integers(0, 20000, size=500).astype(np.int64)
+    want = [oracle.sample_blocks(seeds, indptr, indices, [6, 5, 4], False, 77, 3 * b)[0] for b in range(4)]
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    for epoch in range(9):
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            for b in range(4):
+                f, _, _ = sampler.sample_blocks(None, torch.from_numpy(seeds), batch=b)
+                assert np.array_equal(_np(f), want[b]), (epoch, b)
+        st.synchronize()
+    # busy streams are left alone: batches in flight on six streams at once
+    streams = [torch.cuda.Stream() for _ in range(6)]
+    pending = []
+    for i, st in enumerate(streams * 2):
+        with torch.cuda.stream(st):
+            pending.append(sampler.submit(None, _dev(seeds), batch=i % 4))
+    for i, p in enumerate(pending):
+        assert np.array_equal(_np(p.result()[0]), want[i % 4])
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() - base <= 4 * 8 * (indptr.size - 1) + (64 << 20)
 
 
 def test_sample_with_chunk_tensor_tiers(pkg, oracle, graph):
@@ -227,7 +422,7 @@ def test_fused_sample_blocks_parity(pkg, oracle, id_dtype, ptr_dtype, fanouts, r
         assert torch.equal(x.cpu(), feats[torch.from_numpy(o_frontier).long()])
 
 
-def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph, monkeypatch):
+def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph):
     capi = pkg.capi
     indptr, indices = graph
     ip, ix = _dev(indptr), _dev(indices)
@@ -240,10 +435,7 @@ def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph, monkeypat
     epoch = 0
     # hash table in the workspace (packed, then split slots), then the persistent node table twice
     for mode in ("packed", "split", "direct", "direct"):
-        if mode == "split":
-            monkeypatch.setenv("DGS_FORCE_SPLIT_TABLE", "1")
-        else:
-            monkeypatch.delenv("DGS_FORCE_SPLIT_TABLE", raising=False)
+        capi.check(capi.lib.dgs_debug_set(capi.DEBUG_FORCE_SPLIT_TABLE, int(mode == "split")))
         kw = {}
         if mode == "direct":
             epoch += 1

@@ -102,11 +102,12 @@ def test_split_local_host_index(pkg, oracle):
         o_loc, o_rem, o_host = oracle.split_index(idx.numpy(), s["threshold"], s["device_elems"], dim)
         assert np.array_equal(loc.cpu().numpy(), o_loc) and np.array_equal(host.cpu().numpy(), o_host)
         assert rem.numel() == 0 and o_rem.size == 0
-    # tier-specific gathers on rows wholly inside their tier
-    loc = loc[loc < 150]
+    # tier-specific gathers on the lists split_index made: the host list holds row 150, which
+    # straddles the boundary (its first five elements are in the device slice)
+    assert (host == 150).any() and not (loc >= 150).any()
     assert torch.equal(ct._CAPI_local_index(loc).cpu(), full[loc.cpu()])
-    host = host[host > 150]
     assert torch.equal(ct._CAPI_host_index(host).cpu(), full[host.cpu()])
+    ct._CAPI_synchronize_and_check()
     # int32 ids
     idx32 = torch.randint(0, rows, (777,), generator=g, dtype=torch.int32)
     loc, _, host = ct._CAPI_split_index(idx32.cuda())
@@ -154,5 +155,52 @@ def test_errors_raise_instead_of_aborting(pkg):
         ct._CAPI_index(torch.zeros(3, device="cuda"))  # float index
     capi = pkg.capi
     v = capi.tensor_view(torch.zeros(8, device="cuda"))
-    assert capi.lib.dgs_gather_rows(v, 1, None, 3, 1, None, 0, None) == capi.DGS_ERR_INVALID
+    assert capi.lib.dgs_gather_rows(v, 1, None, 3, 1, None, 0, None, None) == capi.DGS_ERR_INVALID
     assert b"index width" in capi.lib.dgs_last_error()
+
+
+def test_gather_refuses_row_ids_outside_the_store(pkg):
+    # ids are checked before they address anything: bad rows come back as zeros, the flag word is
+    # set, good rows are untouched by it
+    capi = pkg.capi
+    rows, dim = 300, 25
+    full = torch.randn((rows, dim))
+    cap = 100 * dim * 4  # rows 0..99 in HBM, 100..299 in host memory, no straddling row
+    st = capi.Store(rows * dim, 4, cap)
+    st.load(full)
+    flag = torch.zeros(1, dtype=torch.int64, device="cuda")
+    good = torch.tensor([0, 299, 100, 99, 150], device="cuda")
+    out = capi.gather_rows(st.view, dim, good, torch.float32, bad_index=flag)
+    assert flag.item() == 0 and torch.equal(out.cpu(), full[good.cpu()])
+    for dtype in (torch.int64, torch.int32):
+        idx = torch.tensor([5, -1, 299, 300, 2 ** 31 - 1, 120, -2 ** 31], dtype=dtype, device="cuda")
+        ok = torch.tensor([True, False, True, False, False, True, False])
+        flag.zero_()
+        out = capi.gather_rows(st.view, dim, idx, torch.float32, bad_index=flag).cpu()
+        assert flag.item() == 1
+        assert torch.equal(out[ok], full[idx.cpu().long()[ok]]) and (out[~ok] == 0).all()
+    idx = torch.tensor([2 ** 40, 7, -2 ** 62], device="cuda")
+    out = capi.gather_rows(st.view, dim, idx, torch.float32).cpu()  # no flag word: rows are just zero-filled
+    assert torch.equal(out[1], full[7]) and (out[0] == 0).all() and (out[2] == 0).all()
+    # a tier-specific gather refuses rows of the other tier
+    for tier, idx, ok in ((capi.TIER_DEVICE, [3, 100, 99, 299], [True, False, True, False]),
+                          (capi.TIER_HOST, [100, 99, 299, 0], [True, False, True, False])):
+        flag.zero_()
+        ids = torch.tensor(idx, device="cuda")
+        out = capi.gather_rows(st.view, dim, ids, torch.float32, tier=tier, bad_index=flag).cpu()
+        ok = torch.tensor(ok)
+        assert flag.item() == 1 and torch.equal(out[ok], full[ids.cpu()[ok]]) and (out[~ok] == 0).all()
+    st.close()
+    # the operator: the store remembers, and says so at its next call
+    ct = pkg.ChunkTensor([rows, dim], torch.float32, cap)
+    ct._CAPI_load_from_tensor(full)
+    x = ct._CAPI_index(torch.tensor([1, rows, 2], device="cuda"))
+    assert (x[1] == 0).all().item() and torch.equal(x[2].cpu(), full[2])
+    with pytest.raises(RuntimeError, match="outside the store"):
+        ct._CAPI_synchronize_and_check()
+    ct._CAPI_synchronize_and_check()  # reported once
+    ct._CAPI_local_index(torch.tensor([100], device="cuda"))
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="outside the store"):
+        ct._CAPI_index(torch.tensor([1], device="cuda"))
+    assert torch.equal(ct._CAPI_index(torch.tensor([1], device="cuda")).cpu(), full[1:2])

@@ -83,11 +83,12 @@ def test_weighted_row_lengths_around_the_wave_width(pkg, oracle):
 
 
 @pytest.mark.parametrize("group", ["16", "32", "64"])
-def test_weighted_every_group_width(pkg, oracle, graph, group, monkeypatch):
+def test_weighted_every_group_width(pkg, oracle, graph, group, request):
     # the library picks the lanes-per-row from num_picks; the hook forces each width (and with it
     # each long-row threshold) over the same inputs
-    monkeypatch.setenv("DGS_WEIGHTED_GROUP", group)
     capi = pkg.capi
+    capi.check(capi.lib.dgs_debug_set(capi.DEBUG_WEIGHTED_GROUP, int(group)))
+    request.addfinalizer(lambda: capi.lib.dgs_debug_set(capi.DEBUG_WEIGHTED_GROUP, 0))
     indptr, indices, probs = graph
     rng = np.random.default_rng(int(group))
     seeds = rng.integers(0, 20000, size=4000).astype(np.int64)
