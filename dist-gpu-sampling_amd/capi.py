@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libdgs_hip.so")
 
 DGS_OK, DGS_ERR_INVALID, DGS_ERR_HIP, DGS_ERR_WORKSPACE, DGS_ERR_UNSUPPORTED, DGS_ERR_RANGE = range(6)
 TIER_ANY, TIER_DEVICE, TIER_HOST = 0, 1, 2
-DEBUG_FORCE_SPLIT_TABLE, DEBUG_WEIGHTED_GROUP = 0, 1
+DEBUG_FORCE_SPLIT_TABLE, DEBUG_WEIGHTED_GROUP, DEBUG_GATHER_LDS_BYTES, DEBUG_SAMPLER_GRID_CAP = 0, 1, 2, 3
 MAX_SEGMENTS = 8
 
 c_i64, c_i32, c_u64, c_u32, c_vp, c_sz = (ctypes.c_int64, ctypes.c_int32, ctypes.c_uint64, ctypes.c_uint32,

@@ -152,12 +152,16 @@ __device__ __forceinline__ PhiloxWords philox4x32_10(uint32_t c0, uint32_t c1, u
   return PhiloxWords{{c0, c1, c2, c3}};
 }
 
-// Draw j of `row`, reduced to [0, n) (1 <= n < 2^32): multiply-shift with rejection over
-// the block's four words, the last accepted unconditionally.
-__device__ __forceinline__ uint32_t philox_bounded(uint64_t seed, uint32_t stream, int64_t row,
-                                                   uint32_t j, uint32_t n) {
-  const PhiloxWords p = philox4x32_10(j, stream, uint32_t(uint64_t(row)), uint32_t(uint64_t(row) >> 32),
-                                      uint32_t(seed), uint32_t(seed >> 32));
+// The Philox block of draw j of `row`: depends on nothing but the ids, so a kernel can compute it
+// while the loads that tell the range of the draw are still in flight.
+__device__ __forceinline__ PhiloxWords philox_draw_words(uint64_t seed, uint32_t stream, int64_t row, uint32_t j) {
+  return philox4x32_10(j, stream, uint32_t(uint64_t(row)), uint32_t(uint64_t(row) >> 32), uint32_t(seed),
+                       uint32_t(seed >> 32));
+}
+
+// A draw's block reduced to [0, n) (1 <= n < 2^32): multiply-shift with rejection over the
+// block's four words, the last accepted unconditionally.
+__device__ __forceinline__ uint32_t philox_reduce(const PhiloxWords& p, uint32_t n) {
   uint64_t m = uint64_t(p.w[0]) * n;
   if (uint32_t(m) < n) {  // rare: only now is the rejection threshold needed
     const uint32_t t = (0u - n) % n;
@@ -168,6 +172,12 @@ __device__ __forceinline__ uint32_t philox_bounded(uint64_t seed, uint32_t strea
     }
   }
   return uint32_t(m >> 32);
+}
+
+// Draw j of `row`, reduced to [0, n).
+__device__ __forceinline__ uint32_t philox_bounded(uint64_t seed, uint32_t stream, int64_t row,
+                                                   uint32_t j, uint32_t n) {
+  return philox_reduce(philox_draw_words(seed, stream, row, j), n);
 }
 
 }  // namespace dgs

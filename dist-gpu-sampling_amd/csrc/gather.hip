@@ -139,14 +139,16 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
     if (n_dev != nullptr && blocks > kMaxDynGrid) blocks = kMaxDynGrid;
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;
     const uint32_t magic = cpr > 1 ? uint32_t((uint64_t(1) << 32) / uint64_t(cpr)) + 1u : 0u;
+    int64_t lds = debug_option(DGS_DEBUG_GATHER_LDS_BYTES);
+    lds = lds < 0 ? 0 : (lds > 65536 ? 65536 : lds);
     if (blocks < tiles)
       hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, true>), dim3(uint32_t(blocks)),
-                         dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
+                         dim3(kGatherThreads), uint32_t(lds), st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
                          magic, static_cast<const IndexT*>(index), total_chunks, n_dev, row_lo, row_hi,
                          bad_index, static_cast<char*>(out));
     else
       hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, false>), dim3(uint32_t(blocks)),
-                         dim3(kGatherThreads), 0, st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
+                         dim3(kGatherThreads), uint32_t(lds), st, dev, host, thr_bytes, row_bytes, uint32_t(cpr),
                          magic, static_cast<const IndexT*>(index), total_chunks, n_dev, row_lo, row_hi,
                          bad_index, static_cast<char*>(out));
   } else {

@@ -20,13 +20,14 @@ __host__ __device__ inline int64_t pick_count(int64_t deg, int64_t k, bool repla
 //   deg >  k (Floyd):   slot s draws t in [0, deg-k+s] and keeps it unless a lower slot
 //                       already kept t, in which case it keeps deg-k+s (which no lower slot
 //                       can hold); the slots are resolved in order with __shfl / __ballot.
+// `words` is the Philox block of draw l of the row (philox_draw_words), which the caller may have
+// computed before the degree was known.
 template <int G>
 __device__ __forceinline__ bool pick_position(uint32_t deg, int k, bool replace, int l, int group_lane0,
-                                              uint64_t rng_seed, uint32_t rng_stream, int64_t row,
-                                              uint32_t* pos) {
+                                              const PhiloxWords& words, uint32_t* pos) {
   if (replace) {
     if (deg == 0 || l >= k) return false;
-    *pos = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), deg);
+    *pos = philox_reduce(words, deg);
     return true;
   }
   if (deg <= uint32_t(k)) {
@@ -36,7 +37,7 @@ __device__ __forceinline__ bool pick_position(uint32_t deg, int k, bool replace,
   constexpr uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << (G & 63)) - 1);
   const uint32_t top = deg - uint32_t(k) + uint32_t(l);
   uint32_t cand = 0xffffffffu;
-  if (l < k) cand = philox_bounded(rng_seed, rng_stream, row, uint32_t(l), top + 1u);
+  if (l < k) cand = philox_reduce(words, top + 1u);
   uint32_t kept = cand;
   for (int s = 1; s < k; ++s) {
     const uint32_t c = __shfl(cand, s, G);
@@ -45,6 +46,14 @@ __device__ __forceinline__ bool pick_position(uint32_t deg, int k, bool replace,
   }
   *pos = kept;
   return l < k;
+}
+
+template <int G>
+__device__ __forceinline__ bool pick_position(uint32_t deg, int k, bool replace, int l, int group_lane0,
+                                              uint64_t rng_seed, uint32_t rng_stream, int64_t row,
+                                              uint32_t* pos) {
+  return pick_position<G>(deg, k, replace, l, group_lane0, philox_draw_words(rng_seed, rng_stream, row, uint32_t(l)),
+                          pos);
 }
 
 }  // namespace dgs

@@ -33,6 +33,11 @@
 // Off the critical path, as surplus blocks of later launches: per-row pick counts are
 // scanned per 256-row tile, and the packed edge list (src_local, dst_local) is written
 // (rank of a pick = rank recorded at its id's smallest position).
+//
+// These kernels are chains of dependent memory accesses, so what a thread will need is requested
+// as early as its address is known: a hop's length lives in device memory, but every buffer has
+// its worst-case size, so a thread asks for its own elements (inside the buffer whatever the
+// length turns out to be) together with the length and only then decides whether they count.
 #include <type_traits>
 
 #include "common.h"
@@ -61,10 +66,15 @@ constexpr int64_t kInlineTiles = 2048;         // above this a separate scan lau
 // graph deduplicates heavily).  Grids are capped and blocks stride over the virtual block index,
 // so a mostly empty worst case costs a few loop trips instead of 10^5 empty blocks.
 constexpr int64_t kGridCap = 16384;
-inline uint32_t capped_grid(int64_t virtual_blocks) {
-  return uint32_t(virtual_blocks < 1 ? 1 : (virtual_blocks > kGridCap ? kGridCap : virtual_blocks));
+inline int64_t grid_cap() {
+  const int64_t forced = debug_option(DGS_DEBUG_SAMPLER_GRID_CAP);
+  return forced > 0 ? forced : kGridCap;
 }
-inline bool is_capped(int64_t virtual_blocks) { return virtual_blocks > kGridCap; }
+inline uint32_t capped_grid(int64_t virtual_blocks) {
+  const int64_t cap = grid_cap();
+  return uint32_t(virtual_blocks < 1 ? 1 : (virtual_blocks > cap ? cap : virtual_blocks));
+}
+inline bool is_capped(int64_t virtual_blocks) { return virtual_blocks > grid_cap(); }
 // Kernels come in two flavours: STRIDE = false runs exactly one virtual block per block (the
 // common, uncapped launch, with no loop in the instruction stream), STRIDE = true strides.
 #define DGS_FOR_VIRTUAL_BLOCKS(vb, total)                                                       \
@@ -72,10 +82,15 @@ inline bool is_capped(int64_t virtual_blocks) { return virtual_blocks > kGridCap
 
 struct Hop {
   const void* seeds;        // seed ids: caller's seeds (hop 0) or the frontier array
-  const int64_t* n_seeds;   // device scalar (ignored when n_seeds_host >= 0)
+  // The three device scalars below are read without a test in front of them, so that the reads
+  // leave together with a thread's first own reads: the pointers name readable words in every
+  // hop, also where the value is not used (hop 0 takes its count from n_seeds_host and has no
+  // previous hop).
+  const int64_t* n_seeds;   // device scalar: seeds of this hop (used when n_seeds_host < 0)
   int64_t n_seeds_host;     // hop 0: the caller's count; later hops: -1
   int64_t* n_seeds_out;     // hop 0: where to publish n_seeds on the device
-  const int64_t* prev_nnz;  // device scalar: edges of the previous hop (NULL in hop 0)
+  const int64_t* prev_nnz;      // device scalar: edges of the previous hop
+  const int64_t* prev_n_seeds;  // device scalar: seeds of the previous hop
   int64_t* n_unique;        // device scalar: frontier size after this hop
   int64_t* nnz;             // device scalar: edges of this hop
   int64_t* flags;           // device scalar: bit 0 degree, bit 1 seed id, bit 2 picked id of a bad row
@@ -99,14 +114,18 @@ struct Hop {
   void* dst_local;          // out [nnz]
   int64_t s_max;
   int64_t pos_base;         // first position of this hop (P_h)
+  int64_t len_max;          // positions of this hop in the worst case: (hop 0: s_max) + s_max * k
   int32_t k;
   int32_t index;            // hop number
   uint32_t rng_stream;
   int32_t pad_;
 };
 
+// (written without a conditional so that the read is not moved behind a test)
 __device__ __forceinline__ int64_t seeds_of(const Hop& h) {
-  return h.n_seeds_host >= 0 ? h.n_seeds_host : *h.n_seeds;
+  const int64_t on_device = *h.n_seeds;
+  const int64_t use_device = h.n_seeds_host >> 63;  // all ones when the count lives on the device
+  return (on_device & use_device) | (h.n_seeds_host & ~use_device);
 }
 // the first seed_part positions of hop 0 are the caller's seeds themselves
 __device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h.index == 0 ? s : 0; }
@@ -155,9 +174,9 @@ __device__ __forceinline__ void offsets_tile(const Hop& h, int tile) {
   __syncthreads();
   const int64_t s = seeds_of(h);
   const int64_t i = int64_t(tile) * kRowTile + threadIdx.x;
+  const uint32_t rc = i < h.s_max ? h.row_cnt[i] : 0u;  // requested together with s
   int c = 0;
   if (i < s) {
-    const uint32_t rc = h.row_cnt[i];
     if (is_bad_row(rc)) atomicOr(&bad, 1 << (kBadRow - rc)); else c = int(rc);
   }
   int total;
@@ -175,33 +194,38 @@ __device__ __forceinline__ void offsets_tile(const Hop& h, int tile) {
 template <typename IdT, typename TableT>
 __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, int64_t b) {
   __shared__ int64_t lds[kBlock / kWave];
-  const int64_t s = seeds_of(h);
-  const int64_t tiles = (s + kRowTile - 1) / kRowTile;
   const int k = h.k;
   if (k == 0) return;
   const int64_t tile = b / k;
   const int chunk = int(b - tile * k);
-  if (tile >= tiles) return;
-  int64_t prefix;
-  if (h.tile_off) {
-    prefix = h.tile_off[tile];
-  } else {
-    int64_t part = 0;
-    for (int64_t j = threadIdx.x; j < tile; j += kBlock) part += h.tile_sum[j];
-    prefix = block_sum<kBlock, int64_t>(part, lds);
-  }
   const int t = chunk * kBlock + threadIdx.x;  // padded pick inside the tile
   const int r = t / k;
   const int l = t - r * k;
   const int64_t i = tile * kRowTile + r;
-  if (r >= kRowTile || i >= s) return;
-  const uint32_t rc = h.row_cnt[i];
-  if (is_bad_row(rc) || uint32_t(l) >= rc) return;
-  const int64_t o = prefix + h.row_off[i] + l;
-  const int64_t p = h.pos_base + seed_part(h, s) + i * k + l;
-  static_cast<IdT*>(h.src_local)[o] = IdT(rank_of(h, table, p, h.slot[p]));
-  static_cast<IdT*>(h.dst_local)[o] =
-      h.index == 0 ? IdT(rank_of(h, table, h.pos_base + i, h.slot[h.pos_base + i])) : IdT(i);
+  // the hop's length and this thread's own row and pick, requested together
+  const int64_t s = seeds_of(h);
+  const bool mine = r < kRowTile && i < h.s_max;
+  // (hop 0's seed part is the caller's count, a kernel argument: p hangs on no load)
+  const int64_t p = h.pos_base + (h.index == 0 ? h.n_seeds_host : 0) + i * k + l;
+  uint32_t rc = 0, off = 0, word = 0, seed_word = 0;
+  if (mine) {
+    rc = h.row_cnt[i];
+    off = h.row_off[i];
+    word = h.slot[p];
+    if (h.index == 0) seed_word = h.slot[h.pos_base + i];
+  }
+  int64_t part = 0;
+  if (h.tile_off) {
+    if (threadIdx.x == 0) part = h.tile_off[tile];
+  } else {
+    for (int64_t j = threadIdx.x; j < tile; j += kBlock) part += h.tile_sum[j];
+  }
+  if (tile * kRowTile >= s) return;  // whole blocks leave together
+  const int64_t prefix = block_sum<kBlock, int64_t>(part, lds);
+  if (!mine || i >= s || is_bad_row(rc) || uint32_t(l) >= rc) return;
+  const int64_t o = prefix + off + l;
+  static_cast<IdT*>(h.src_local)[o] = IdT(rank_of(h, table, p, word));
+  static_cast<IdT*>(h.dst_local)[o] = h.index == 0 ? IdT(rank_of(h, table, h.pos_base + i, seed_word)) : IdT(i);
 }
 
 inline int64_t relabel_blocks(int64_t s_max, int k) {
@@ -245,10 +269,12 @@ __device__ __forceinline__ bool emit_pick(const Hop& h, const TableT& table, con
 // the previous hop tells: if more than a fifth of its picks were not new ids, look first.
 // (hop 0 has no history: look first only when it is big enough for contention to matter)
 __device__ __forceinline__ bool look_before_insert(const Hop& h, int64_t s) {
-  if (h.prev_nnz == nullptr) return s * h.k >= (int64_t(1) << 17);
   const int64_t picked = *h.prev_nnz;
-  const int64_t fresh = s - *(h.n_seeds - 1);  // ids the previous hop added to the frontier
-  return fresh * 5 < picked * 4;
+  const int64_t fresh = s - *h.prev_n_seeds;  // ids the previous hop added to the frontier
+  const bool first_hop = h.index == 0;
+  const bool big = s * h.k >= (int64_t(1) << 17);
+  const bool repeats = fresh * 5 < picked * 4;
+  return bool((int(first_hop) & int(big)) | (int(!first_hop) & int(repeats)));
 }
 
 // One virtual block of the fill launch: 256 / G seed rows.
@@ -256,15 +282,20 @@ template <typename IdT, typename PtrT, typename TableT, int G>
 __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT& table,
                                           const TierView<PtrT>& indptr, const TierView<IdT>& indices,
                                           bool replace, uint64_t rng_seed) {
-  const int64_t s = seeds_of(h);
-  if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
   const int64_t gid = vb * kBlock + threadIdx.x;
   const int64_t i = gid / G;
   const int l = int(gid % G);
+  // the hop's length, what the previous hop found, and this group's seed id, requested together
+  // (the seed list has room for s_max ids whatever the length turns out to be)
+  const IdT seed = i < h.s_max ? static_cast<const IdT*>(h.seeds)[i] : IdT(0);
+  const int64_t s = seeds_of(h);
+  const bool look_first = look_before_insert(h, s);
+  if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
   if (i >= s) return;  // whole groups leave together
   const int group_lane0 = (threadIdx.x & (kWave - 1)) - l;
-  const IdT seed = static_cast<const IdT*>(h.seeds)[i];
   const int64_t row = int64_t(seed);
+  // this lane's random block hangs on the ids only: computed while the offsets are on their way
+  const PhiloxWords words = philox_draw_words(rng_seed, h.rng_stream, row, uint32_t(l));
   // nothing is addressed by an id or an offset before it has been checked
   const bool seed_ok = row_in_range(indptr, row) && table.holds(seed);
   int64_t b = 0, deg64 = 0;
@@ -275,7 +306,6 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   const bool bad = deg64 < 0 || deg64 > 0xffffffffLL || b < 0 || b + deg64 > indices.n;
   const uint32_t deg = bad ? 0u : uint32_t(deg64);
   const int k = h.k;
-  const bool look_first = look_before_insert(h, s);
   if (l == 0 && h.index == 0) {  // the caller's seeds open the mapping list; flag() decides their first bits
     bool first;
     uint32_t displaced;
@@ -283,7 +313,7 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
         seed_ok ? table.insert_min(seed, uint32_t(h.pos_base + i), &first, &displaced) : kInvalidSlot;
   }
   uint32_t pos;
-  const bool have = pick_position<G>(deg, k, replace, l, group_lane0, rng_seed, h.rng_stream, row, &pos);
+  const bool have = pick_position<G>(deg, k, replace, l, group_lane0, words, &pos);
   bool pick_ok = true;
   if (l < k) pick_ok = emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, have, b + pos, look_first);
   constexpr uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << (G & 63)) - 1);
@@ -335,6 +365,7 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
                                                    const TierView<float>& probs, uint64_t rng_seed) {
   const Group<kWave> g;
   const int64_t s = seeds_of(h);
+  const bool look_first = look_before_insert(h, s);
   if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
   const int k = h.k;
   const int lanes = weighted_row_lanes(k);
@@ -362,7 +393,6 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
     bad = deg64 < 0 || deg64 > 0xffffffffLL || b < 0 || b + deg64 > indices.n;
     deg = bad ? 0u : uint32_t(deg64);
   }
-  const bool look_first = look_before_insert(h, s);
   if (i < s && l == 0 && h.index == 0) {
     bool first_seen;
     uint32_t displaced;
@@ -457,24 +487,31 @@ template <typename IdT, typename TableT>
 __device__ __forceinline__ void flag_tile(const Hop& h, int64_t tile, const TableT& table) {
   __shared__ int lds[kBlock / kWave];
   const int64_t s = seeds_of(h);
-  const int64_t len = seed_part(h, s) + s * h.k;
   const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
+  // this thread's slot words and lost marks, requested together with the hop's length
+  uint32_t w[kPosItems];
+  uint8_t gone[kPosItems];
+#pragma unroll
+  for (int j = 0; j < kPosItems; ++j) {
+    const bool inside = base + j < h.len_max;
+    w[j] = inside ? h.slot[h.pos_base + base + j] : kInvalidSlot;
+    gone[j] = inside && h.index != 0 ? h.lost[h.pos_base + base + j] : uint8_t(0);
+  }
+  const int64_t len = seed_part(h, s) + s * h.k;
   int c = 0;
   if (tile * kPosTile < len) {
 #pragma unroll
     for (int j = 0; j < kPosItems; ++j) {
       const int64_t rel = base + j;
-      if (rel < len) {
+      if (rel < len && w[j] != kInvalidSlot) {
         const int64_t p = h.pos_base + rel;
-        const uint32_t w = h.slot[p];
-        if (w == kInvalidSlot) continue;
         if (h.index == 0) {
-          if (table.value(w) == uint32_t(p)) {
-            h.slot[p] = w | kFirstBit;
+          if (table.value(w[j]) == uint32_t(p)) {
+            h.slot[p] = w[j] | kFirstBit;
             ++c;
           }
-        } else if (w & kFirstBit) {
-          if (h.lost[p]) h.slot[p] = w & ~kFirstBit; else ++c;
+        } else if (w[j] & kFirstBit) {
+          if (gone[j]) h.slot[p] = w[j] & ~kFirstBit; else ++c;
         }
       }
     }
@@ -494,73 +531,74 @@ __global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_bl
   }
 }
 
-// Separate scans for very long tile lists (one block).
-__global__ __launch_bounds__(1024) void pos_scan_kernel(Hop h) {
-  const int64_t s = seeds_of(h);
-  const int64_t tiles = (seed_part(h, s) + s * h.k + kPosTile - 1) / kPosTile;
+// Separate scans for very long tile lists (one block), over the worst-case tile counts (the
+// counts of tiles beyond the hop's real length are zero).
+__global__ __launch_bounds__(1024) void pos_scan_kernel(Hop h, int64_t pos_tiles) {
   int64_t sum;
-  single_block_scan<1024, int, int64_t>(h.pos_cnt, h.pos_off, tiles, &sum);
+  single_block_scan<1024, int, int64_t>(h.pos_cnt, h.pos_off, pos_tiles, &sum);
 }
-__global__ __launch_bounds__(1024) void tile_scan_kernel(Hop h) {
-  const int64_t tiles = (seeds_of(h) + kRowTile - 1) / kRowTile;
+__global__ __launch_bounds__(1024) void tile_scan_kernel(Hop h, int64_t row_tiles) {
   int64_t sum;
-  single_block_scan<1024, int, int64_t>(h.tile_sum, h.tile_off, tiles, &sum);
+  single_block_scan<1024, int, int64_t>(h.tile_sum, h.tile_off, row_tiles, &sum);
 }
 
 // One virtual block of the compact launch: the first occurrences of one 1024-position tile.
+// `pos_tiles` / `row_tiles` are the worst-case tile counts the flag launch covered: the counts of
+// tiles beyond the hop's real length are zero there, so sums may run over all of them.
 template <typename IdT, typename TableT>
-__device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, const TableT& table) {
+__device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, int64_t pos_tiles, int64_t row_tiles,
+                                             const TableT& table) {
   __shared__ int64_t lds64[kBlock / kWave];
   __shared__ int lds[kBlock / kWave];
+  // the hop's length, this thread's slot words and its share of the tile counts, requested together
   const int64_t s = seeds_of(h);
-  const int64_t len = seed_part(h, s) + s * h.k;
-  const int64_t tiles = (len + kPosTile - 1) / kPosTile;
-  const int64_t rank0 = first_rank(h, s);
-  if (tile >= tiles && tile != 0) return;
-  // first occurrences in the tiles before this one (block 0 also needs the grand total)
-  int64_t before = 0, all = 0;
+  const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
+  uint32_t w[kPosItems];
+#pragma unroll
+  for (int j = 0; j < kPosItems; ++j) w[j] = base + j < h.len_max ? h.slot[h.pos_base + base + j] : kInvalidSlot;
+  // first occurrences in the tiles before this one (block 0 needs the grand total instead)
+  int64_t part = 0;
   if (h.pos_off) {
-    before = tile < tiles ? h.pos_off[tile] : 0;
-    if (tile == 0 && tiles > 0) all = h.pos_off[tiles - 1] + h.pos_cnt[tiles - 1];
+    if (threadIdx.x == 0) part = tile == 0 ? h.pos_off[pos_tiles - 1] + h.pos_cnt[pos_tiles - 1] : h.pos_off[tile];
   } else {
-    const int64_t upto = tile == 0 ? tiles : tile;
-    int64_t part = 0;
+    const int64_t upto = tile == 0 ? pos_tiles : tile;
     for (int64_t j = threadIdx.x; j < upto; j += kBlock) part += h.pos_cnt[j];
-    part = block_sum<kBlock, int64_t>(part, lds64);
-    if (tile == 0) all = part; else before = part;
   }
+  int64_t edges = 0;
+  int bad = 0;
   if (tile == 0) {
-    // this hop's lengths, written even when there is nothing to do: frontier size, edge count
-    // (row tiles were scanned by the surplus blocks of the flag launch) and error flag
-    const int64_t row_tiles = (s + kRowTile - 1) / kRowTile;
-    int64_t edges = 0;
-    int bad = 0;
     for (int64_t j = threadIdx.x; j < row_tiles; j += kBlock) {
       edges += h.tile_sum[j];
       bad |= h.tile_flag[j];
     }
+  }
+  const int64_t len = seed_part(h, s) + s * h.k;
+  const int64_t rank0 = first_rank(h, s);
+  if (tile != 0 && tile * kPosTile >= len) return;  // whole blocks leave together
+  part = block_sum<kBlock, int64_t>(part, lds64);
+  if (tile == 0) {
+    // this hop's lengths, written even when there is nothing to do: frontier size, edge count
+    // (row tiles were scanned by the surplus blocks of the flag launch) and error bits
     edges = block_sum<kBlock, int64_t>(edges, lds64);
     bad = block_or<kBlock>(bad, lds);
     if (threadIdx.x == 0) {
-      *h.n_unique = rank0 + all;
+      *h.n_unique = rank0 + part;
       *h.nnz = edges;
       *h.flags = bad;
       if (h.host_sizes) {
         if (h.index == 0) h.host_sizes[0] = s;
-        h.host_sizes[h.index + 1] = rank0 + all;
+        h.host_sizes[h.index + 1] = rank0 + part;
         h.host_sizes[h.n_hops + 1 + h.index] = edges;
         h.host_sizes[2 * h.n_hops + 1 + h.index] = bad;
       }
     }
+    if (len <= 0) return;
   }
-  if (tile >= tiles) return;
-  const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
-  uint32_t w[kPosItems];
+  const int64_t before = tile == 0 ? 0 : part;
   int c = 0;
 #pragma unroll
   for (int j = 0; j < kPosItems; ++j) {
-    w[j] = base + j < len ? h.slot[h.pos_base + base + j] : kInvalidSlot;
-    if (w[j] == kInvalidSlot) w[j] = 0;  // bit 31 clear: not a first occurrence
+    if (base + j >= len || w[j] == kInvalidSlot) w[j] = 0;  // bit 31 clear: not a first occurrence
     c += (w[j] & kFirstBit) != 0;
   }
   int total;
@@ -576,8 +614,9 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, const T
 }
 
 template <typename IdT, typename TableT, bool STRIDE>
-__global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, int64_t pos_tiles, TableT table) {
-  DGS_FOR_VIRTUAL_BLOCKS(vb, pos_tiles) compact_tile<IdT, TableT>(h, vb, table);
+__global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, int64_t blocks, int64_t pos_tiles,
+                                                             int64_t row_tiles, TableT table) {
+  DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) compact_tile<IdT, TableT>(h, vb, pos_tiles, row_tiles, table);
 }
 
 template <typename IdT, typename TableT, bool STRIDE>
@@ -671,6 +710,7 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
     v.pos_off = pos_tiles > size_t(kInlineTiles) ? c.take<int64_t>(pos_tiles) : nullptr;
     v.s_max = p.s_max[h];
     v.pos_base = pos_base;
+    v.len_max = int64_t(len);
     v.k = int32_t(fanouts[h]);
     v.index = h;
     if (hops) hops[h] = v;
@@ -765,20 +805,20 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
                          dim3(kBlock), 0, st, cur, pos_tiles, row_tiles, table);
     DGS_LAUNCH_CHECK();
     if (cur.pos_off) {
-      hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
+      hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur, pos_tiles);
       DGS_LAUNCH_CHECK();
     }
     if (cur.tile_off) {
-      hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
+      hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, cur, row_tiles);
       DGS_LAUNCH_CHECK();
     }
     const int64_t compact_blocks = pos_tiles > 0 ? pos_tiles : 1;  // block 0 always writes the lengths
     if (is_capped(compact_blocks))
       hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT, true>), dim3(capped_grid(compact_blocks)), dim3(kBlock),
-                         0, st, cur, compact_blocks, table);
+                         0, st, cur, compact_blocks, pos_tiles, row_tiles, table);
     else
       hipLaunchKernelGGL((hop_compact_kernel<IdT, TableT, false>), dim3(capped_grid(compact_blocks)), dim3(kBlock),
-                         0, st, cur, compact_blocks, table);
+                         0, st, cur, compact_blocks, pos_tiles, row_tiles, table);
     DGS_LAUNCH_CHECK();
   }
   // every length is final here: mark the point the caller may wait for
@@ -911,7 +951,8 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
     t.n_seeds = sizes_dev + h;
     t.n_seeds_host = h == 0 ? n_seeds : -1;
     t.n_seeds_out = h == 0 ? sizes_dev : nullptr;
-    t.prev_nnz = h == 0 ? nullptr : sizes_dev + n_hops + h;  // edges of hop h - 1
+    t.prev_nnz = sizes_dev + n_hops + (h == 0 ? 1 : h);  // edges of hop h - 1 (hop 0: any readable word)
+    t.prev_n_seeds = sizes_dev + (h == 0 ? 0 : h - 1);
     t.n_unique = sizes_dev + h + 1;
     t.nnz = sizes_dev + n_hops + 1 + h;
     t.flags = sizes_dev + 2 * n_hops + 1 + h;

@@ -51,8 +51,17 @@ int dgs_abi_version(void);
  *                                the packed one
  *   DGS_DEBUG_WEIGHTED_GROUP     16, 32 or 64: lanes per row of the weighted per-hop fill
  *                                (0: chosen from num_picks)
+ *   DGS_DEBUG_GATHER_LDS_BYTES   bytes of (unused) LDS that every block of the row gather
+ *                                reserves, 0..65536: bounds how many of its blocks share a CU
+ *   DGS_DEBUG_SAMPLER_GRID_CAP   > 0: most blocks a launch of dgs_sample_blocks may have
+ *                                (larger launches loop over their blocks)
  */
-enum { DGS_DEBUG_FORCE_SPLIT_TABLE = 0, DGS_DEBUG_WEIGHTED_GROUP = 1 };
+enum {
+  DGS_DEBUG_FORCE_SPLIT_TABLE = 0,
+  DGS_DEBUG_WEIGHTED_GROUP = 1,
+  DGS_DEBUG_GATHER_LDS_BYTES = 2,
+  DGS_DEBUG_SAMPLER_GRID_CAP = 3
+};
 dgs_status dgs_debug_set(int32_t option, int64_t value);
 
 /* ------------------------------------------------------------------------ */

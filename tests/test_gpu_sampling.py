@@ -628,3 +628,28 @@ def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph):
         pkg.BatchPipeline(sampler, x_ct, 0)
     with pytest.raises(RuntimeError):
         list(pkg.BatchPipeline(pkg.ChunkTensorSampler([100], ip_ct, ix_ct), x_ct)([_dev(batches[0])]))
+
+
+@pytest.mark.parametrize("cap", [1, 7, 300])
+def test_fused_sampler_under_a_small_grid_cap(pkg, oracle, graph, cap, request):
+    # every launch of the fused sampler loops over its blocks when there are more than the cap:
+    # the results do not depend on the cap
+    capi = pkg.capi
+    indptr, indices = graph
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    probs = (np.random.default_rng(1).random(indices.size) + 0.05).astype(np.float32)
+    pr_ct = pkg.create_chunktensor(torch.from_numpy(probs), 1, 1 << 40)
+    feats = torch.randn((20000, 12))
+    ft = pkg.create_chunktensor(feats, 1, 1 << 40)
+    rng = np.random.default_rng(cap)
+    seeds = rng.integers(0, 20000, size=1500).astype(np.int64)
+    capi.check(capi.lib.dgs_debug_set(capi.DEBUG_SAMPLER_GRID_CAP, cap))
+    request.addfinalizer(lambda: capi.lib.dgs_debug_set(capi.DEBUG_SAMPLER_GRID_CAP, 0))
+    for weights, fanouts, replace in ((None, [12, 6, 3], False), (None, [20, 9], True), (probs, [5, 4], False)):
+        sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, None if weights is None else pr_ct, replace=replace, seed=5)
+        f, _, blocks, x = sampler.sample_blocks_and_index(None, torch.from_numpy(seeds), ft)
+        want_f, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, replace, 5, 0, probs=weights)
+        assert np.array_equal(_np(f), want_f)
+        _check_blocks(blocks, want_blocks)
+        assert torch.equal(x.cpu(), feats[f.cpu()])
