@@ -65,9 +65,7 @@ def build_torch(force=True):
           "-I" + os.path.join(rocm, "include"),
           "-o", TORCH_LIB, src,
           "-L" + HERE, "-ldgs_hip", "-L" + os.path.join(tdir, "lib"),
-          "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
-          # torch's stream guard is header-only and calls the HIP runtime directly
-          "-L" + os.path.join(rocm, "lib"), "-lamdhip64",
+          "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
           "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"])
     return TORCH_LIB
 

@@ -22,7 +22,6 @@
 //     dereferenced (upstream does not check, src/cuda/index_with_chunk_tensor.cu:16-23):
 //     sampling raises; a gather zero-fills the row and the store raises at its next call.
 #include <c10/hip/HIPFunctions.h>
-#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/custom_class.h>
@@ -538,14 +537,6 @@ class PendingBlocks : public torch::CustomClassHolder {
   PendingBlocks() = default;
   ~PendingBlocks() override {
     if (ticket_ != nullptr) dgs_ticket_wait(ticket_);  // never leave a ticket behind
-    if (gather_ticket_ != nullptr) dgs_ticket_release(gather_ticket_);
-  }
-
-  // Makes the current stream wait for the batch's feature gather when that ran on a stream of
-  // its own (nothing to do otherwise: the gather then sits on the stream the batch was submitted
-  // on, like everything else of the batch).
-  void WaitGather() {
-    if (gather_ticket_ != nullptr) check(dgs_ticket_stream_wait(current_stream(), gather_ticket_));
   }
 
   BlocksResult Finish() {
@@ -580,8 +571,7 @@ class PendingBlocks : public torch::CustomClassHolder {
                                                  const c10::intrusive_ptr<ChunkTensor>& features,
                                                  const c10::intrusive_ptr<ChunkTensor>& probs =
                                                      c10::intrusive_ptr<ChunkTensor>(),
-                                                 const std::pair<uint64_t, uint32_t>* own_rng = nullptr,
-                                                 const c10::optional<c10::Stream>& gather_stream = c10::nullopt) {
+                                                 const std::pair<uint64_t, uint32_t>* own_rng = nullptr) {
     const int32_t w = id_width(seeds_in, "seeds");
     if (features) features->CheckErrors();
     if (probs) TORCH_CHECK(probs->dtype() == torch::kFloat32, "probs store must be float32, got ", probs->dtype());
@@ -641,32 +631,13 @@ class PendingBlocks : public torch::CustomClassHolder {
     if (features) {
       const auto xopt = torch::TensorOptions().dtype(features->dtype()).device(dev);
       const int64_t row_bytes = features->elem_stride() * static_cast<int64_t>(c10::elementSize(features->dtype()));
-      // The gather runs on the batch's own stream, or on a stream of its own behind the point
-      // where the frontier is final: the batch's stream is then free for its remaining edge lists
-      // and for the next batch, and the gathers of successive batches never compete with each
-      // other for memory bandwidth while the (latency-bound) sampling of other batches runs beside them.
-      void* gst = st;
-      c10::optional<c10::hip::HIPStreamMasqueradingAsCUDA> gs;
-      if (gather_stream.has_value()) {
-        gs.emplace(*gather_stream);
-        gst = gs->stream();
-        check(dgs_ticket_stream_wait(gst, p->ticket_));
-        // the gather reads these on its own stream: their memory must not be reused before it has run
-        p->all_.record_stream(gs->unwrap());
-        sizes_dev.record_stream(gs->unwrap());
-      }
       if (seeds_max[hops] * row_bytes <= g_gather_buffer_cap.load()) {
         // the lengths are final at the ticket; the gather is enqueued before anybody waits for
         // them, into a buffer for the worst case of which the result is a prefix
-        if (gs.has_value()) {
-          c10::hip::HIPStreamGuardMasqueradingAsCUDA on_gather_stream(gs->unwrap());
-          p->x_ = torch::empty({seeds_max[hops], features->elem_stride()}, xopt);  // from that stream's pool
-        } else {
-          p->x_ = torch::empty({seeds_max[hops], features->elem_stride()}, xopt);
-        }
+        p->x_ = torch::empty({seeds_max[hops], features->elem_stride()}, xopt);
         p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
                                                 seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops,
-                                                p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), gst);
+                                                p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
       } else {
         // the worst case would be too large a buffer (it grows with the product of the fanouts,
         // the frontier does not): wait for the frontier's size and gather into exactly that many
@@ -675,16 +646,10 @@ class PendingBlocks : public torch::CustomClassHolder {
         p->ticket_ = nullptr;
         check(dgs_ticket_wait(t));
         const int64_t rows = p->pinned_.data_ptr<int64_t>()[hops];
-        if (gs.has_value()) {
-          c10::hip::HIPStreamGuardMasqueradingAsCUDA on_gather_stream(gs->unwrap());
-          p->x_ = torch::empty({rows, features->elem_stride()}, xopt);
-        } else {
-          p->x_ = torch::empty({rows, features->elem_stride()}, xopt);
-        }
+        p->x_ = torch::empty({rows, features->elem_stride()}, xopt);
         p->gather_status_ = dgs_gather_rows(features->view(), features->elem_stride(), p->all_.data_ptr(), w, rows,
-                                            p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), gst);
+                                            p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
       }
-      if (gs.has_value()) check(dgs_ticket_record(gst, &p->gather_ticket_));
     }
     return p;
   }
@@ -693,7 +658,6 @@ class PendingBlocks : public torch::CustomClassHolder {
   int hops_ = 0;
   bool finished_ = false;
   void* ticket_ = nullptr;
-  void* gather_ticket_ = nullptr;  // end of the gather when it runs on a stream of its own
   dgs_status gather_status_ = DGS_OK;
   torch::Tensor pinned_, seeds_, all_, x_;
   std::vector<torch::Tensor> src_, dst_;
@@ -755,28 +719,21 @@ c10::intrusive_ptr<PendingBlocks> SampleBlocksWeightedBegin(torch::Tensor seeds,
 // Any of the *_begin operators with the generator state passed in: the hops draw from streams
 // rng_stream, rng_stream + 1, ... of seed rng_seed and the process-wide generator is left alone,
 // so a caller that keeps its own counter gets the same picks whatever other threads do.
-// `rng` is empty (the process-wide generator) or [seed, first stream]; `gather_stream` is empty
-// (the gather runs on the current stream) or the [stream_id, device_index, device_type] of the
-// torch stream that runs the feature gather of this batch.
+// The general form of the *_begin operators: `probs` and `features` are optional, `rng` is empty
+// (the process-wide generator) or [seed, first stream].
 c10::intrusive_ptr<PendingBlocks> SampleBlocksSubmit(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr,
                                                      c10::intrusive_ptr<ChunkTensor> indices,
                                                      c10::optional<c10::intrusive_ptr<ChunkTensor>> probs,
                                                      std::vector<int64_t> fanouts, bool replace,
                                                      c10::optional<c10::intrusive_ptr<ChunkTensor>> features,
-                                                     std::vector<int64_t> rng, std::vector<int64_t> gather_stream) {
+                                                     std::vector<int64_t> rng) {
   TORCH_CHECK(rng.empty() || rng.size() == 2, "sample_blocks_submit: rng is [] or [seed, stream]");
-  TORCH_CHECK(gather_stream.empty() || gather_stream.size() == 3,
-              "sample_blocks_submit: gather_stream is [] or [stream_id, device_index, device_type]");
   std::pair<uint64_t, uint32_t> own{0, 0};
   if (!rng.empty()) own = {static_cast<uint64_t>(rng[0]), static_cast<uint32_t>(rng[1])};
-  c10::optional<c10::Stream> gs;
-  if (!gather_stream.empty())
-    gs = c10::Stream::unpack3(gather_stream[0], static_cast<c10::DeviceIndex>(gather_stream[1]),
-                              static_cast<c10::DeviceType>(gather_stream[2]));
   return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace,
                               features.has_value() ? *features : c10::intrusive_ptr<ChunkTensor>(),
                               probs.has_value() ? *probs : c10::intrusive_ptr<ChunkTensor>(),
-                              rng.empty() ? nullptr : &own, gs);
+                              rng.empty() ? nullptr : &own);
 }
 
 // Largest worst-case feature buffer (bytes) the fused operators allocate ahead of the sizes.
@@ -826,9 +783,7 @@ TORCH_LIBRARY(dgs_classes, m) {
       // not in upstream: waits for the current stream, then raises if a gather met a bad row id
       .def("_CAPI_synchronize_and_check", &ChunkTensor::SynchronizeAndCheck);
   // not in upstream: a sample_blocks call in flight
-  m.class_<PendingBlocks>("PendingBlocks")
-      .def("_CAPI_finish", &PendingBlocks::Finish)
-      .def("_CAPI_wait_gather", &PendingBlocks::WaitGather);
+  m.class_<PendingBlocks>("PendingBlocks").def("_CAPI_finish", &PendingBlocks::Finish);
 }
 
 TORCH_LIBRARY(dgs_ops, m) {

@@ -58,21 +58,14 @@ def create_chunktensor(tensor, num_gpus, available_mem, cache_rate=1.0, root_ran
 class PendingBatch:
     """A batch whose kernels are enqueued (ChunkTensorSampler.submit).  result() waits until the
     batch's sizes are known and returns what sample_blocks / sample_blocks_and_index return; the
-    last kernels of the batch may still be running on the stream it was submitted on (and its
-    feature gather on the gather stream, if one was given), so a consumer on another stream
-    orders itself after them with `batch.order_before(consumer)`."""
+    last kernels of the batch may still be running on the stream it was submitted on, so a consumer
+    on another stream orders itself after that stream (`consumer.wait_stream(batch.stream)`)."""
 
     def __init__(self, handle, seed_nodes, with_features, stream):
         self._handle = handle
         self._seed_nodes = seed_nodes
         self._with_features = with_features
         self.stream = stream
-
-    def order_before(self, consumer):
-        """Makes the stream `consumer` wait for everything the batch has enqueued."""
-        consumer.wait_stream(self.stream)
-        with torch.cuda.stream(consumer):
-            self._handle._CAPI_wait_gather()
 
     def result(self):
         frontiers, srcs, dsts, x, seeds = self._handle._CAPI_finish()
@@ -165,24 +158,18 @@ class ChunkTensorSampler:
             seeds = frontier
         return frontier, seed_nodes, blocks
 
-    def submit(self, g, seed_nodes, chunk_features=None, batch=None, gather_stream=None):
+    def submit(self, g, seed_nodes, chunk_features=None, batch=None):
         """Enqueues a batch on the current stream and returns at once (fused path only).  Batches
-        submitted on different streams overlap on the GPU: sampling is a chain of short kernels
-        bound by memory latency, and several such chains run side by side at no cost to each
-        other.  With `gather_stream` the feature gather of the batch (bound by HBM bandwidth) is
-        enqueued on that stream instead, behind the point where the frontier is final: the
-        gathers of successive batches then run one after the other while the sampling of later
-        batches proceeds beside them.  Results come from PendingBatch.result(), in any order."""
+        submitted on different streams overlap on the GPU: the short kernels of one batch's first
+        hops fill the gaps between the large kernels of another.  Results come from
+        PendingBatch.result(), in any order."""
         if not self.fused:
             raise RuntimeError("submit() needs the fused path: every fanout <= 64")
         hop_fanouts = list(reversed(self.fanouts))
         rng = [] if self.seed is None else [self.seed, self._first_stream(batch)]
-        gs = []
-        if gather_stream is not None and chunk_features is not None:
-            gs = [gather_stream.stream_id, gather_stream.device_index, gather_stream.device_type]
         handle = torch.ops.dgs_ops._CAPI_sample_blocks_submit(
             seed_nodes, self.chunk_indptr, self.chunk_indices, self.chunk_probs, hop_fanouts, self.replace,
-            chunk_features, rng, gs)
+            chunk_features, rng)
         return PendingBatch(handle, seed_nodes, chunk_features is not None, torch.cuda.current_stream())
 
     def sample_blocks_and_index(self, g, seed_nodes, chunk_features):
@@ -205,10 +192,9 @@ _pipeline_streams = []
 
 
 def pipeline_streams(n):
-    """The first n of the streams that BatchPipeline objects run on by default: the first one
-    runs the feature gathers, the others sample.  They are shared by all pipelines of the
-    process: a graph keeps one node table per stream that ever sampled from it (at most four),
-    so pipelines that come and go should not each bring new streams."""
+    """The first n of the streams that BatchPipeline objects run on by default.  They are shared by
+    all pipelines of the process: a graph keeps one node table per stream that ever sampled from
+    it (at most four), so pipelines that come and go should not each bring new streams."""
     while len(_pipeline_streams) < n:
         _pipeline_streams.append(torch.cuda.Stream())
     return _pipeline_streams[:n]
@@ -229,26 +215,18 @@ class BatchPipeline:
     that stream behind it; a consumer that works on the batch's own stream needs nothing, and the
     allocator can reuse the batch's buffers as soon as they are dropped (measured on a 288 MB
     feature block per batch: 5 % more batches per second).
-    By default all pipelines share pipeline_streams(inflight + 1): one stream for the feature
-    gathers (`gather_stream`; pass False to keep each batch's gather on the batch's own stream)
-    and `inflight` streams that sample.
+    By default all pipelines share pipeline_streams(inflight).
     Streams of one pipeline should sit on different hardware queues to overlap; the first
     four streams a process makes do.
     """
 
-    def __init__(self, sampler, chunk_features=None, inflight=2, streams=None, hand_over=True, gather_stream=None):
+    def __init__(self, sampler, chunk_features=None, inflight=2, streams=None, hand_over=True):
         self.hand_over = hand_over
         if inflight < 1:
             raise ValueError("inflight must be at least 1")
         self.sampler = sampler
         self.chunk_features = chunk_features
-        if gather_stream is False or chunk_features is None or inflight == 1:
-            self.gather_stream = None  # a single batch in flight gains nothing from a second stream
-        elif gather_stream is None or gather_stream is True:
-            self.gather_stream = pipeline_streams(1)[0]
-        else:
-            self.gather_stream = gather_stream
-        self.streams = list(streams) if streams is not None else pipeline_streams(inflight + 1)[1:]
+        self.streams = list(streams) if streams is not None else pipeline_streams(inflight)
         if not self.streams:
             raise ValueError("no streams to run on")
 
@@ -256,7 +234,7 @@ class BatchPipeline:
         out = pending.result()
         if not self.hand_over:
             return out
-        pending.order_before(consumer)
+        consumer.wait_stream(pending.stream)
         tensors = [out[0]]
         for b in out[2]:
             tensors += [b.src_local, b.dst_local]
@@ -282,7 +260,7 @@ class BatchPipeline:
             if i < len(self.streams) or (torch.is_tensor(seeds) and seeds.is_cuda):
                 st.wait_stream(consumer)
             with torch.cuda.stream(st):
-                queue.append(self.sampler.submit(None, seeds, self.chunk_features, gather_stream=self.gather_stream))
+                queue.append(self.sampler.submit(None, seeds, self.chunk_features))
             if len(queue) >= len(self.streams):
                 yield self._hand_out(queue.popleft(), consumer)
         while queue:
