@@ -57,7 +57,7 @@ SIGNATURES = {
     "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
     "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_workspace_bytes": (c_sz, [c_i64]),
-    "dgs_sample_count": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_count": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_fill": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_u64, c_u32, c_vp, c_vp,
                                        c_vp, c_sz, c_vp]),
     "dgs_sample_neighbors": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32,
@@ -69,7 +69,8 @@ SIGNATURES = {
     "dgs_sample_neighbors_weighted": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, View, c_i64, c_i32, c_u64,
                                                      c_u32, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_unique_relabel_workspace_bytes": (c_sz, [c_i64, c_i32]),
-    "dgs_unique_relabel": (ctypes.c_int, [Segments, Segments, c_i32, c_vp, c_vp, Segments, c_vp, c_sz, c_vp]),
+    "dgs_unique_relabel": (ctypes.c_int, [Segments, Segments, c_i32, c_i32, c_vp, c_vp, c_vp, ctypes.POINTER(c_vp),
+                                          Segments, c_vp, c_sz, c_vp]),
     "dgs_sample_blocks_plan": (ctypes.c_int, [c_i64, ctypes.POINTER(c_i64), c_i32, ctypes.POINTER(c_i64),
                                               ctypes.POINTER(c_i64)]),
     "dgs_sample_blocks_workspace_bytes": (c_sz, [c_i64, ctypes.POINTER(c_i64), c_i32, c_i32]),
@@ -201,7 +202,7 @@ def sample_neighbors(seeds, indptr_view, indices_view, num_picks, replace, rng_s
     w = seeds.element_size()
     if two_step:
         check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
-                                   ws.data_ptr(), nb, stream_ptr()))
+                                   None, ws.data_ptr(), nb, stream_ptr()))
         cnt, flags = read_i64(nnz, 2)
         rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
         cols = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
@@ -242,7 +243,7 @@ def sample_neighbors_weighted(seeds, indptr_view, indices_view, probs_view, num_
     w = seeds.element_size()
     if two_step:
         check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
-                                   ws.data_ptr(), nb, stream_ptr()))
+                                   None, ws.data_ptr(), nb, stream_ptr()))
         cnt, flags = read_i64(nnz, 2)
         rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
         cols = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
@@ -268,20 +269,24 @@ def renumber_csc(indptr, indices, order, rank, new_indptr):
     return out
 
 
-def unique_relabel(mapping, requiring):
-    """Returns (unique, [relabelled ...])."""
+def unique_relabel(mapping, requiring, packed_table=True):
+    """Returns (unique, [relabelled ...]).  With `packed_table` 8-byte ids are tried in the one-word
+    slots first and the call is repeated with the two-array table if an id does not fit."""
     dev = mapping[0].device
     dt = mapping[0].dtype
     n = sum(t.numel() for t in mapping)
     unique = torch.empty(n, dtype=dt, device=dev)
     outs = [torch.empty_like(t) for t in requiring]
-    num = torch.empty(1, dtype=torch.int64, device=dev)
+    num = torch.empty(2, dtype=torch.int64, device=dev)
     w = mapping[0].element_size()
     nb = lib.dgs_unique_relabel_workspace_bytes(n, w)
     ws = _ws(nb, dev)
-    check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, unique.data_ptr(), num.data_ptr(),
-                                 segments(outs), ws.data_ptr(), nb, stream_ptr()))
-    u = read_i64(num, 1)[0]
+    for packed in ((1, 0) if packed_table else (0,)):
+        check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, packed, unique.data_ptr(),
+                                     num.data_ptr(), None, None, segments(outs), ws.data_ptr(), nb, stream_ptr()))
+        u, overflow = read_i64(num, 2)
+        if not overflow:
+            break
     return unique[:u], outs
 
 

@@ -345,17 +345,25 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
   if (one_shot) {
     rows = torch::empty({n * num_picks}, seeds.options());
     cols = torch::empty({n * num_picks}, seeds.options());
-    if (probs != nullptr)
-      check(dgs_sample_neighbors_weighted(seeds.data_ptr(), w, n, indptr, indices, *probs, num_picks, replace,
-                                          rng.first, rng.second, rows.data_ptr(), cols.data_ptr(),
-                                          nnz_dev.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
-    else
-      check(dgs_sample_neighbors(seeds.data_ptr(), w, n, indptr, indices, num_picks, replace, rng.first,
-                                 rng.second, rows.data_ptr(), cols.data_ptr(), nnz_dev.data_ptr<int64_t>(),
-                                 ws.data_ptr(), ws_bytes, st));
-    len = read_back(nnz_dev, 2);
-  } else {
+    // count (which mirrors the length into pinned memory), a ticket, then the fill: the host waits
+    // for the ticket only, and the fill is still running when the operator returns
+    thread_local torch::Tensor pinned =
+        torch::empty({2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
     check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(),
+                           pinned.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
+    void* ticket = nullptr;
+    check(dgs_ticket_record(st, &ticket));
+    const dgs_status fill_status =
+        probs != nullptr
+            ? dgs_sample_fill_weighted(seeds.data_ptr(), w, n, indices, *probs, num_picks, replace, rng.first,
+                                       rng.second, rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st)
+            : dgs_sample_fill(seeds.data_ptr(), w, n, indices, num_picks, replace, rng.first, rng.second,
+                              rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st);
+    check(dgs_ticket_wait(ticket));
+    check(fill_status);
+    len.assign(pinned.data_ptr<int64_t>(), pinned.data_ptr<int64_t>() + 2);
+  } else {
+    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(), nullptr,
                            ws.data_ptr(), ws_bytes, st));
     len = read_back(nnz_dev, 2);
     rows = torch::empty({len[0]}, seeds.options());
@@ -514,12 +522,27 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> TensorRelabel(std::vector<
     }
   }
   torch::Tensor unique = torch::empty({n}, opt);
-  torch::Tensor num_unique = torch::empty({1}, opt.dtype(torch::kInt64));
+  torch::Tensor counts = torch::empty({2}, opt.dtype(torch::kInt64));
   const size_t ws_bytes = dgs_unique_relabel_workspace_bytes(n, w);
   torch::Tensor ws = device_bytes(ws_bytes, dev);
-  check(dgs_unique_relabel(map_seg, req_seg, w, unique.data_ptr(), num_unique.data_ptr<int64_t>(), out_seg,
-                           ws.data_ptr(), ws_bytes, current_stream()));
-  const int64_t u = read_back(num_unique, 1)[0];
+  // The kernels mirror the counts into pinned memory as soon as they are final, and the host
+  // waits for that point only: the kernels that write `unique` and the relabelled ids are still
+  // running when the operator returns (its results are ordered on the stream as always).
+  thread_local torch::Tensor pinned =
+      torch::empty({2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+  int64_t* counts_host = pinned.data_ptr<int64_t>();
+  // 8-byte ids first go into one-word slots (one atomic per id); an id of 2^32 - 1 or more voids
+  // that attempt and the call is repeated with the two-array table
+  int64_t u = 0;
+  for (const int32_t packed : {1, 0}) {
+    void* ticket = nullptr;
+    check(dgs_unique_relabel(map_seg, req_seg, w, packed, unique.data_ptr(), counts.data_ptr<int64_t>(), counts_host,
+                             &ticket, out_seg, ws.data_ptr(), ws_bytes, current_stream()));
+    check(dgs_ticket_wait(ticket));
+    u = counts_host[0];
+    if (counts_host[1] == 0) break;
+    TORCH_CHECK(packed != 0, "tensor_relabel: the table rejected an id");
+  }
   return std::make_tuple(unique.narrow(0, 0, u), relabelled.split_with_sizes(sizes, 0));
 }
 

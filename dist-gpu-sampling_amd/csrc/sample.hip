@@ -92,7 +92,8 @@ __global__ __launch_bounds__(kTile) void sample_count_kernel(
 __global__ __launch_bounds__(1024) void sample_scan_kernel(const int64_t* __restrict__ tile_sum,
                                                            int64_t* __restrict__ tile_off,
                                                            const int* __restrict__ tile_flag,
-                                                           int64_t tiles, int64_t* __restrict__ nnz_dev) {
+                                                           int64_t tiles, int64_t* __restrict__ nnz_dev,
+                                                           int64_t* __restrict__ nnz_host) {
   __shared__ int any_flag;
   if (threadIdx.x == 0) any_flag = 0;
   __syncthreads();
@@ -105,6 +106,10 @@ __global__ __launch_bounds__(1024) void sample_scan_kernel(const int64_t* __rest
   if (threadIdx.x == 0) {
     nnz_dev[0] = sum;
     nnz_dev[1] = any_flag;
+    if (nnz_host) {  // pinned host memory: the caller reads the length without a copy
+      nnz_host[0] = sum;
+      nnz_host[1] = any_flag;
+    }
   }
 }
 
@@ -260,7 +265,7 @@ __global__ __launch_bounds__(kTile) void fill_wave_global_kernel(
 
 template <typename IdT, typename PtrT>
 dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr, int64_t k, bool replace,
-                     const SampleWorkspace& w, int64_t* nnz_dev, hipStream_t st) {
+                     const SampleWorkspace& w, int64_t* nnz_dev, int64_t* nnz_host, hipStream_t st) {
   const int64_t tiles = (n_seeds + kTile - 1) / kTile;
   if (tiles > 0) {
     hipLaunchKernelGGL((sample_count_kernel<IdT, PtrT>), dim3(uint32_t(tiles)), dim3(kTile), 0, st,
@@ -269,7 +274,7 @@ dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr,
     DGS_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL(sample_scan_kernel, dim3(1), dim3(1024), 0, st, w.tile_sum, w.tile_off, w.tile_flag,
-                     tiles, nnz_dev);
+                     tiles, nnz_dev, nnz_host);
   DGS_LAUNCH_CHECK();
   return DGS_OK;
 }
@@ -324,8 +329,8 @@ DGS_API size_t dgs_sample_workspace_bytes(int64_t n_seeds) {
 }
 
 DGS_API dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
-                                    int64_t num_picks, int32_t replace, int64_t* nnz_dev, void* workspace,
-                                    size_t workspace_bytes, void* stream) {
+                                    int64_t num_picks, int32_t replace, int64_t* nnz_dev, int64_t* nnz_host,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
   using namespace dgs;
   dgs_status s = check_sample_args("sample_count", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
   if (s != DGS_OK) return s;
@@ -337,10 +342,10 @@ DGS_API dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t
   sample_workspace_layout(n_seeds, workspace, &w);
   const bool rep = replace != 0;
   if (id_bytes == 8)
-    return indptr.elem_bytes == 8 ? run_count<int64_t, int64_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, st)
-                                  : run_count<int64_t, int32_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, st);
-  return indptr.elem_bytes == 8 ? run_count<int32_t, int64_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, st)
-                                : run_count<int32_t, int32_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, st);
+    return indptr.elem_bytes == 8 ? run_count<int64_t, int64_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st)
+                                  : run_count<int64_t, int32_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st);
+  return indptr.elem_bytes == 8 ? run_count<int32_t, int64_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st)
+                                : run_count<int32_t, int32_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st);
 }
 
 DGS_API dgs_status dgs_sample_fill(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indices,
@@ -368,7 +373,7 @@ DGS_API dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes, int
                                         int32_t replace, uint64_t rng_seed, uint32_t rng_stream,
                                         void* out_rows, void* out_cols, int64_t* nnz_dev, void* workspace,
                                         size_t workspace_bytes, void* stream) {
-  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, num_picks, replace, nnz_dev, workspace,
+  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, num_picks, replace, nnz_dev, nullptr, workspace,
                                   workspace_bytes, stream);
   if (s != DGS_OK) return s;
   return dgs_sample_fill(seeds, id_bytes, n_seeds, indices, num_picks, replace, rng_seed, rng_stream, out_rows,

@@ -219,7 +219,11 @@ dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
  *
  * dgs_sample_count is the degree/count/scan half (the reference's sub_indptr,
  * rowwise_sampling_with_chunk_tensor.cu:127-156): it leaves the per-row
- * offsets in the workspace and the edge count in nnz_dev.
+ * offsets in the workspace and the edge count in nnz_dev, and mirrors nnz_dev
+ * into nnz_host when that is given (int64[2] of pinned host memory that the
+ * device can write; NULL: no mirror): a caller that records a ticket behind
+ * this call, enqueues the fill and then waits for the ticket reads the length
+ * while the fill still runs.
  * dgs_sample_fill is the COO fill (:15-111, :158-180); out_rows / out_cols
  * must hold nnz ids.  dgs_sample_neighbors runs both; its outputs must hold
  * n_seeds * num_picks ids (the worst case), so no length is read back between
@@ -228,7 +232,7 @@ dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
 size_t dgs_sample_workspace_bytes(int64_t n_seeds);
 dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t n_seeds,
                             dgs_view indptr, int64_t num_picks, int32_t replace,
-                            int64_t* nnz_dev, void* workspace,
+                            int64_t* nnz_dev, int64_t* nnz_host, void* workspace,
                             size_t workspace_bytes, void* stream);
 dgs_status dgs_sample_fill(const void* seeds, int32_t id_bytes, int64_t n_seeds,
                            dgs_view indices, int64_t num_picks, int32_t replace,
@@ -324,16 +328,29 @@ typedef struct dgs_segments {
  * out[t][i] = position of requiring[t][i] in unique, or -1 when absent.
  * Replaces TensorRelabelCUDA / Unique / Relabel / RelabelHashmap
  * (src/cuda/tensor_reindex.cu:11-205).
+ *   packed_table   : 8-byte ids only.  Non-zero: the table keeps id and position in one 64-bit
+ *                    slot (one atomic per id instead of two), which holds ids below 2^32 - 1; an
+ *                    id beyond that sets counts_dev[1] and voids the call's results (call again
+ *                    with 0).  Zero: id array + value array, any id >= 0.
  *   unique_out     : device, capacity sum(mapping.len) ids
- *   num_unique_dev : device int64[1]
+ *   counts_dev     : device int64[2]: [0] number of distinct ids, [1] non-zero if an id did not
+ *                    fit the packed table
+ *   counts_host / counts_ticket : optional (both or neither).  counts_host is pinned host memory
+ *                    that the device can write; the kernels mirror counts_dev into it, and
+ *                    *counts_ticket marks the point on `stream` after which it is complete:
+ *                    before `unique_out` and `out` are written, so that a caller can wait for the
+ *                    count (dgs_ticket_wait) while those kernels still run.  Saves the reference's
+ *                    blocking read at the end (src/cuda/tensor_reindex.cu:129).
  *   out            : device arrays, out.len must equal requiring.len
- * ids must be >= 0 (-1 is the empty-slot marker, as in the reference).
+ * Mapping ids must be >= 0 (-1 is the empty-slot marker, as in the reference); a requiring id that
+ * is negative or not in the mapping list gives -1.
  * sum(mapping.len) must be <= 2^30.
  */
 size_t dgs_unique_relabel_workspace_bytes(int64_t n_mapping, int32_t id_bytes);
 dgs_status dgs_unique_relabel(dgs_segments mapping, dgs_segments requiring,
-                              int32_t id_bytes, void* unique_out,
-                              int64_t* num_unique_dev, dgs_segments out,
+                              int32_t id_bytes, int32_t packed_table, void* unique_out,
+                              int64_t* counts_dev, int64_t* counts_host,
+                              void** counts_ticket, dgs_segments out,
                               void* workspace, size_t workspace_bytes,
                               void* stream);
 

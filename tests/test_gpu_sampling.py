@@ -653,3 +653,31 @@ def test_fused_sampler_under_a_small_grid_cap(pkg, oracle, graph, cap, request):
         assert np.array_equal(_np(f), want_f)
         _check_blocks(blocks, want_blocks)
         assert torch.equal(x.cpu(), feats[f.cpu()])
+
+
+def test_unique_relabel_ids_beyond_32_bits(pkg, oracle):
+    # 8-byte ids are first tried in one-word table slots; an id of 2^32 - 1 or more sends the call
+    # to the two-array table.  Ids that only differ above bit 31 must not be confused, present or not.
+    rng = np.random.default_rng(40)
+    small = rng.integers(0, 5000, size=4000).astype(np.int64)
+    for big in (2 ** 32 - 1, 2 ** 32 + 7, 2 ** 40 + 3):
+        mapping = [small[:1000].copy(), np.concatenate([small[1000:], [big, 7, big + 2 ** 32]]).astype(np.int64)]
+        requiring = [np.array([7, 7 + 2 ** 32, big, -1, -5, 2 ** 62, 4999, big - 2 ** 32], dtype=np.int64), mapping[1]]
+        want_u, want_outs = oracle.unique_relabel(mapping, requiring)
+        want_first = want_outs[0].copy()
+        in_map = np.isin(requiring[0], np.concatenate(mapping))
+        assert (want_first[~in_map] == -1).all()
+        u, outs = pkg.capi.unique_relabel([_dev(p) for p in mapping], [_dev(p) for p in requiring])
+        assert np.array_equal(_np(u), want_u)
+        for a, b in zip(outs, want_outs):
+            assert np.array_equal(_np(a), b)
+        u, outs = pkg.ops._CAPI_tensor_relabel([_dev(p) for p in mapping], [_dev(p) for p in requiring])
+        assert np.array_equal(_np(u), want_u)
+        for a, b in zip(outs, want_outs):
+            assert np.array_equal(_np(a), b)
+    # ids that all fit: the packed attempt stands, and an id absent from the mapping that aliases a
+    # present one in its low 32 bits is still absent
+    mapping = [small]
+    requiring = [np.array([small[0], small[0] + 2 ** 32, -1], dtype=np.int64)]
+    u, outs = pkg.capi.unique_relabel([_dev(p) for p in mapping], [_dev(p) for p in requiring])
+    assert _np(outs[0]).tolist() == [0, -1, -1]
