@@ -24,9 +24,33 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per gathered 400-byte row of workload c1, from rocprofv3 FETCH_SIZE (x2.0 after
-# calibration against a plain copy) and WRITE_SIZE (x1.0): 378.3 MB + 288.2 MB per 719,002 rows
-C1_GATHER_TRAFFIC_BYTES_PER_ROW = (378.3e6 + 288.2e6) / 719002.0
+GATHER_SOURCE = os.path.join(ROOT, "dist-gpu-sampling_amd", "csrc", "gather.hip")
+GATHER_TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gather_flat_kernel_c1_pmc.txt")
+
+
+def measured_gather_traffic():
+    """HBM bytes per gathered 400-byte row of workload c1, as the committed counter summary holds
+    them (rocprofv3 FETCH_SIZE and WRITE_SIZE, scaled by a plain copy of known size), together
+    with where they come from.  The summary names the version of the gather source it was taken
+    on; for any other version the reading says nothing and (None, why) is returned."""
+    import hashlib
+    import re
+    try:
+        text = open(GATHER_TRAFFIC_SUMMARY).read()
+        source_hash = hashlib.sha256(open(GATHER_SOURCE, "rb").read()).hexdigest()[:16]
+    except OSError as err:
+        return None, f"no counter summary to read ({err.filename})"
+    per_row = re.search(r"^traffic_bytes_per_row\s*=\s*([0-9.]+)", text, re.M)
+    taken_on = re.search(r"^gather_source_sha256_16\s*=\s*([0-9a-f]{16})", text, re.M)
+    name = os.path.relpath(GATHER_TRAFFIC_SUMMARY, ROOT)
+    if not per_row or not taken_on:
+        return None, f"{name} holds no traffic_bytes_per_row / gather_source_sha256_16 lines"
+    if taken_on.group(1) != source_hash:
+        return None, (f"{name} was taken on gather.hip {taken_on.group(1)}, this run has {source_hash}: "
+                      "counters not re-taken for this kernel")
+    return float(per_row.group(1)), (f"{name} (gather.hip {source_hash}): counter bytes per gathered row "
+                                     "x this run's rows; not a counter reading of this run")
+
 
 WORKLOADS = {
     # benchmark configuration 1: the one the headline metric is quoted on
@@ -142,6 +166,11 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0, probs=None
     total = t_sample + t_gather
     gather_bytes = rows * (2 * feats.shape[1] * feats.element_size() + 8)
     return {"value": edges / total, "unit": "edges/s", "cores": threads, "kind": "port",
+            "host_cpus": os.cpu_count(), "omp_threads": threads, "torch_threads": torch.get_num_threads(),
+            "threads_per_leg": {"sampling": f"{threads} (OpenMP over the seed rows)",
+                                "unique/relabel": "1 (the identity-hash table with sequential inserts, as "
+                                                  "upstream's algorithm orders them)",
+                                "gather": f"{torch.get_num_threads()} (torch.index_select)"},
             "sample": f"{done} batches of {cfg['batch']} seeds, fanouts {cfg['fanouts']}, same graph/features "
                       f"({total:.1f} s of CPU work): oracle sampling+relabel, torch.index_select gather",
             "sample_edges_per_s": edges / t_sample, "gather_GBps": gather_bytes / t_gather / 1e9,
@@ -205,6 +234,28 @@ def run_batches(sampler, seed_batches, features, inflight, consume=lambda r: Non
         return [consume(sampler.sample_blocks_and_index(None, b, features)) for b in seed_batches]
     pipeline = sys.modules[type(sampler).__module__].BatchPipeline(sampler, features, inflight, hand_over=hand_over)
     return [consume(r) for r in pipeline(seed_batches)]
+
+
+def table_access_rates(dgs, slots, n_ops, reps=10):
+    """Random 8-byte accesses per second this GPU serves on a table of `slots` slots, by kind:
+    the library's probe kernel (one access per thread, nothing else), timed with events on the
+    stream it is launched on.  The fused sampler does one atomicMin with return per pick on a
+    table of one slot per node, so these are the rates that bound it."""
+    capi = dgs.capi
+    table = torch.full((slots,), -1, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(1, dtype=torch.int64, device="cuda")
+    out = {"slots": slots, "table_bytes": 8 * slots, "accesses_per_launch": n_ops, "unit": "G accesses/s"}
+    for name, op in (("load", capi.PROBE_LOAD), ("store", capi.PROBE_STORE),
+                     ("atomic_min_with_return", capi.PROBE_ATOMIC_MIN),
+                     ("atomic_min_no_return", capi.PROBE_ATOMIC_MIN_NO_RETURN)):
+        salt = [0]
+        def once():
+            salt[0] += 1
+            capi.probe_table(op, table, n_ops, salt[0], sink)
+        t = time_call(once, reps)
+        out[name] = n_ops / t / 1e9
+        out[name + "_us"] = 1e6 * t
+    return out
 
 
 def time_call(fn, reps):
@@ -420,8 +471,6 @@ def main():
     dgs.set_rng_state(20240602, 0)
 
     inflight = args.inflight if sampler.fused else 1
-    run_batches(sampler, batches[:args.warmup], ct_feats, inflight)
-    torch.cuda.synchronize()
     if args.calibrate_copy_mib > 0:
         src = torch.empty(args.calibrate_copy_mib << 18, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)
@@ -429,36 +478,35 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    def keep(r):  # sizes, the frontier ids (for the gather leg below) and the destination ids of the widest hop
-        return ({"frontier": r[0].numel(),
-                 "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]}, r[0], r[2][0].dst_ids)
+    def sizes(r):  # what the timed loops keep of a batch: its lengths; every buffer is dropped at once
+        return {"frontier": r[0].numel(),
+                "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]}
 
-    results = run_batches(sampler, batches[args.warmup:], ct_feats, inflight, keep)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    stats = [r[0] for r in results]
-    frontiers = [r[1] for r in results]
-    widest_hop_seeds = results[-1][2]
-    del results
-    # one batch at a time on one stream: what a single batch takes from call to result
-    dgs.set_rng_state(20240602, 0)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_batches(sampler, batches[args.warmup:], ct_feats, 1)
-    torch.cuda.synchronize()
-    ms_latency = 1e3 * (time.perf_counter() - t0) / args.steps
-    # batches in flight again, each handed over to the calling stream (made to wait for the batch,
-    # buffers recorded there): what a consumer on another stream than the batch's own sees
-    ms_handed_over = None
-    if inflight > 1:
-        run_batches(sampler, batches[:args.warmup], ct_feats, inflight, hand_over=True)
+    def timed_steps(smp, seed_batches, n_inflight, hand_over=False):
+        """W untimed warm-up batches, then exactly K batches between two synchronisations."""
+        run_batches(smp, seed_batches[:args.warmup], ct_feats, n_inflight, sizes, hand_over)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        run_batches(sampler, batches[args.warmup:], ct_feats, inflight, hand_over=True)
+        res = run_batches(smp, seed_batches[args.warmup:], ct_feats, n_inflight, sizes, hand_over)
         torch.cuda.synchronize()
-        ms_handed_over = 1e3 * (time.perf_counter() - t0) / args.steps
+        return time.perf_counter() - t0, res
+
+    # the headline: `inflight` batches on the GPU at any time, seeds already in HBM, each batch
+    # left on the stream it ran on
+    elapsed, stats = timed_steps(sampler, batches, inflight)
+    repeats = [1e3 * timed_steps(sampler, batches, inflight)[0] / args.steps for _ in range(3)]
+    # one batch at a time on one stream: what a single batch takes from call to result
+    ms_latency = 1e3 * timed_steps(sampler, batches, 1)[0] / args.steps
+    # batches in flight again, each handed over to the calling stream (made to wait for the batch,
+    # buffers recorded there): what a consumer on another stream than the batch's own sees
+    ms_handed_over = 1e3 * timed_steps(sampler, batches, inflight, True)[0] / args.steps if inflight > 1 else None
+    # seeds as upstream's DataLoader passes them: pageable host tensors, uploaded by the operator
+    ms_host_seeds = 1e3 * timed_steps(sampler, batches_cpu, inflight)[0] / args.steps
+    # what an unmodified upstream harness runs: per hop one sampling operator and one relabel
+    # operator (each returns tensors of exact length, so each waits for its lengths), then _CAPI_index
+    per_hop = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, ct_probs, replace=cfg["replace"],
+                                     fused=False)
+    ms_per_hop_ops = 1e3 * timed_steps(per_hop, batches, 1)[0] / args.steps
 
     # Stage split and the dominant kernel's duration, on the same batches: events on torch's
     # current stream (the one the C ABI launches on) around the sampler call and around the
@@ -468,10 +516,16 @@ def main():
     for i in range(args.warmup):
         sampler.sample_blocks(None, batches[i])
     torch.cuda.synchronize()
+    frontiers = []
+    stage_stats = []
     for i in range(args.steps):
         events[i][0].record()
-        sampler.sample_blocks(None, batches[args.warmup + i])
+        r = sampler.sample_blocks(None, batches[args.warmup + i])
         events[i][1].record()
+        frontiers.append(r[0])
+        stage_stats.append(sizes(r))
+        widest_hop_seeds = r[2][0].dst_ids
+    del r
     torch.cuda.synchronize()
     gather_ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(args.steps)]
     for i in range(args.steps):  # queued back to back: the GPU never waits for the host
@@ -479,18 +533,28 @@ def main():
         x = ct_feats._CAPI_index(frontiers[i])
         gather_ev[i][1].record()
     torch.cuda.synchronize()
+    del x, frontiers
+
+    def total_bytes(all_stats):
+        bs = bu = bg = 0
+        for s in all_stats:
+            a, b, c = algorithmic_bytes(s, cfg["feat_dim"], feat_bytes)
+            bs, bu, bg = bs + a, bu + b, bg + c
+        return bs, bu, bg
 
     ms_step = 1e3 * elapsed / args.steps
     ms_sample = float(np.mean([e[0].elapsed_time(e[1]) for e in events]))
     ms_gather = float(np.mean([e[0].elapsed_time(e[1]) for e in gather_ev]))
     edges = sum(sum(h[1] for h in s["hops"]) for s in stats)
     rows = sum(s["frontier"] for s in stats)
-    bs = bu = bg = 0
-    for s in stats:
-        a, b, c = algorithmic_bytes(s, cfg["feat_dim"], feat_bytes)
-        bs, bu, bg = bs + a, bu + b, bg + c
-    gather_gbps = bg / args.steps / (ms_gather * 1e-3) / 1e9
+    bs, bu, bg = total_bytes(stats)
+    stage_edges = sum(sum(h[1] for h in s["hops"]) for s in stage_stats)
+    stage_rows = sum(s["frontier"] for s in stage_stats)
+    sbs, sbu, sbg = total_bytes(stage_stats)  # the batches of the stage-split runs (same seeds, their own picks)
+    gather_gbps = sbg / args.steps / (ms_gather * 1e-3) / 1e9
+    sampler_gbps = (sbs + sbu) / args.steps / (ms_sample * 1e-3) / 1e9
     step_gbps = (bs + bu + bg) / elapsed / 1e9
+    traffic_per_row, traffic_source = measured_gather_traffic() if args.workload in ("c1", "c1w") else (None, None)
 
     out = {
         "metric": "sampled edges/s (sampling + relabel + feature gather per batch), 1 MI355X",
@@ -509,10 +573,22 @@ def main():
                                f"features {cfg['feat_dtype']} x{cfg['feat_dim']}, all in HBM, batch {cfg['batch']} "
                                f"uniform seeds, fanouts {cfg['fanouts']} without replacement"
                                f"{', weighted by a float32 weight per edge' if cfg.get('weighted') else ''}, then gather",
-                   "fanouts": cfg["fanouts"], "batch": cfg["batch"], "batches_in_flight": inflight},
+                   "fanouts": cfg["fanouts"], "batch": cfg["batch"], "batches_in_flight": inflight,
+                   "timed": "value / ms_per_step: the fused operator (_CAPI_sample_blocks_submit, sampling + "
+                            "relabel of every hop + gather per batch), seeds resident in HBM, "
+                            f"{inflight} batches in flight on as many streams, each batch left on its own stream"},
+        "ms_per_step_repeats": repeats,
         "ms_per_batch_alone": ms_latency,
         "ms_per_step_handed_over": ms_handed_over,
-        "sample_edges_per_s": edges / args.steps / (ms_sample * 1e-3),
+        "ms_per_step_host_seeds": ms_host_seeds,
+        "ms_per_step_per_hop_ops": ms_per_hop_ops,
+        "timings": {"ms_per_step_repeats": "the timed region run three more times (spread)",
+                    "ms_per_batch_alone": "one batch at a time, one stream, call to result",
+                    "ms_per_step_handed_over": "as the headline, each batch handed to the calling stream",
+                    "ms_per_step_host_seeds": "as the headline, seeds passed as pageable host tensors",
+                    "ms_per_step_per_hop_ops": "upstream's own loop: _CAPI_sample_neighbors_with_chunk_tensor + "
+                                               "_CAPI_tensor_relabel per hop, then _CAPI_index, one batch at a time"},
+        "sample_edges_per_s": stage_edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
         "ms_sample_relabel": ms_sample,
         "ms_gather": ms_gather,
@@ -523,10 +599,27 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gather_flat_kernel (ChunkTensor._CAPI_index)",
                      "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gather_gbps / HBM_PEAK_GBPS,
-                     "traffic": (C1_GATHER_TRAFFIC_BYTES_PER_ROW * rows / args.steps) if args.workload in ("c1", "c1w") else None,
-                     "algorithmic_bytes": bg / args.steps, "avg_launch_us": 1e3 * ms_gather},
+                     "traffic": None if traffic_per_row is None else traffic_per_row * stage_rows / args.steps,
+                     "traffic_source": traffic_source,
+                     "algorithmic_bytes": sbg / args.steps, "avg_launch_us": 1e3 * ms_gather},
+        "stages": [
+            {"stage": "sampling + relabel of every hop (fused sampler kernels, one batch alone on one stream)",
+             "bound": "hbm", "achieved": sampler_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": sampler_gbps / HBM_PEAK_GBPS, "algorithmic_bytes": (sbs + sbu) / args.steps,
+             "avg_us": 1e3 * ms_sample},
+            {"stage": "feature gather of the last frontier (gather_flat_kernel)",
+             "bound": "hbm", "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": gather_gbps / HBM_PEAK_GBPS, "algorithmic_bytes": sbg / args.steps,
+             "avg_us": 1e3 * ms_gather},
+            {"stage": "whole step as timed for the headline", "bound": "hbm", "achieved": step_gbps,
+             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS,
+             "algorithmic_bytes": (bs + bu + bg) / args.steps, "avg_us": 1e3 * ms_step},
+        ],
         "graph_gen_s": t_gen,
     }
+    if args.workload != "c0":
+        # one access per pick of the widest hop, on a table the size of the sampler's node table
+        out["table_access_rates"] = table_access_rates(dgs, cfg["nodes"], int(max(h[1] for h in stats[0]["hops"])))
     if cfg.get("weighted"):
         # the weighted fill of the widest hop alone: its input is every weight of every sampled row
         ops = torch.ops.dgs_ops

@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libdgs_hip.so")
 DGS_OK, DGS_ERR_INVALID, DGS_ERR_HIP, DGS_ERR_WORKSPACE, DGS_ERR_UNSUPPORTED, DGS_ERR_RANGE = range(6)
 TIER_ANY, TIER_DEVICE, TIER_HOST = 0, 1, 2
 DEBUG_FORCE_SPLIT_TABLE, DEBUG_WEIGHTED_GROUP, DEBUG_GATHER_LDS_BYTES, DEBUG_SAMPLER_GRID_CAP = 0, 1, 2, 3
+PROBE_LOAD, PROBE_STORE, PROBE_ATOMIC_MIN, PROBE_ATOMIC_MIN_NO_RETURN = 0, 1, 2, 3
 MAX_SEGMENTS = 8
 
 c_i64, c_i32, c_u64, c_u32, c_vp, c_sz = (ctypes.c_int64, ctypes.c_int32, ctypes.c_uint64, ctypes.c_uint32,
@@ -44,6 +45,7 @@ SIGNATURES = {
     "dgs_status_name": (ctypes.c_char_p, [ctypes.c_int]),
     "dgs_abi_version": (ctypes.c_int, []),
     "dgs_debug_set": (ctypes.c_int, [c_i32, c_i64]),
+    "dgs_debug_probe_table": (ctypes.c_int, [c_i32, c_vp, c_i64, c_i64, c_u64, c_vp, c_vp]),
     "dgs_store_split": (ctypes.c_int, [c_i64, c_i32, c_i64, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)]),
     "dgs_store_create": (ctypes.c_int, [c_i64, c_i32, c_i64, ctypes.POINTER(c_vp)]),
     "dgs_store_destroy": (ctypes.c_int, [c_vp]),
@@ -168,6 +170,12 @@ def read_i64(dev_tensor, count):
     host = torch.empty(count, dtype=torch.int64).pin_memory()
     check(lib.dgs_read_back(host.data_ptr(), dev_tensor.data_ptr(), 8 * count, stream_ptr()))
     return host.tolist()
+
+
+def probe_table(op, table, n_ops, salt, sink):
+    """dgs_debug_probe_table on torch's current stream: n_ops random 8-byte accesses of kind `op`
+    to `table` (an int64 device tensor); `sink` is an int64 device tensor of one element."""
+    check(lib.dgs_debug_probe_table(op, table.data_ptr(), table.numel(), n_ops, salt, sink.data_ptr(), stream_ptr()))
 
 
 def gather_rows(view, row_elems, index, dtype, tier=TIER_ANY, bad_index=None):

@@ -46,53 +46,86 @@ __device__ __forceinline__ const char* resolve(const char* dev, const char* host
 // chunk c -> row c / cpr, column c % cpr; the division runs on a block-local
 // 32-bit offset with a precomputed reciprocal (exact while
 // (cpr + kChunksPerBlock) * cpr < 2^32, guaranteed by kMaxFlatChunksPerRow).
-// Rows [row_lo, row_hi) are the ones the launch may read.
+// Rows [row_lo, row_hi) are the ones the launch may read; the range is not empty.
+//
+// The kChunksPerBlock output chunks from chunk c0 on (c0 < total_chunks); returns whether an
+// index outside [row_lo, row_hi) was met.
+// Three passes, each over all of the thread's chunks, so that nothing but the row ids, then
+// nothing but the chunks themselves, is alive across the waits: the row ids (all requested
+// before any is used), the loads, the stores.
+template <int VEC, int TIER, typename IndexT>
+__device__ __forceinline__ bool gather_tile(const char* __restrict__ dev, const char* __restrict__ host,
+                                            int64_t thr_bytes, int64_t row_bytes, uint32_t cpr, uint32_t magic,
+                                            const IndexT* __restrict__ index, int64_t total_chunks, int64_t row_lo,
+                                            int64_t row_hi, char* __restrict__ out, int64_t c0) {
+  using C = typename Chunk<VEC>::type;
+  bool bad = false;
+  const int64_t row0 = c0 / cpr;
+  const uint32_t rem0 = uint32_t(c0 - row0 * cpr);
+  const IndexT* __restrict__ index0 = index + row0;
+  int64_t src[kGatherUnroll];
+  uint32_t off[kGatherUnroll];  // byte offset of the chunk inside its row
+#pragma unroll
+  for (int u = 0; u < kGatherUnroll; ++u) {
+    const uint32_t t = u * kGatherThreads + threadIdx.x;
+    const uint32_t lc = rem0 + t;
+    const uint32_t q = cpr == 1 ? lc : __umulhi(lc, magic);
+    off[u] = (lc - q * cpr) * uint32_t(VEC);
+    src[u] = c0 + t < total_chunks ? int64_t(index0[q]) : row_lo;  // past the end: some row, never stored
+  }
+  // An id outside [row_lo, row_hi) is replaced by row_lo before it addresses anything (the
+  // launcher guarantees that row_lo is a row the tier holds), and what was read for it is
+  // dropped: no branch around the loads, so all of them are in flight together.
+  C val[kGatherUnroll];
+  bool in_range[kGatherUnroll];
+#pragma unroll
+  for (int u = 0; u < kGatherUnroll; ++u) {
+    in_range[u] = src[u] >= row_lo && src[u] < row_hi;
+    if (!in_range[u]) {
+      src[u] = row_lo;
+      bad |= c0 + u * kGatherThreads + threadIdx.x < total_chunks;
+    }
+    const int64_t g = src[u] * row_bytes + int64_t(off[u]);
+    val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
+  }
+#pragma unroll
+  for (int u = 0; u < kGatherUnroll; ++u)
+    if (!in_range[u]) val[u] = C(0);
+  char* __restrict__ o = out + (c0 + threadIdx.x) * VEC;
+#pragma unroll
+  for (int u = 0; u < kGatherUnroll; ++u) {
+    if (c0 + u * kGatherThreads + threadIdx.x < total_chunks)
+      __builtin_nontemporal_store(val[u], reinterpret_cast<C*>(o + int64_t(u) * kGatherThreads * VEC));
+  }
+  return bad;
+}
+
+// STRIDE: the grid is smaller than the tile count (capped launch) and blocks stride over the
+// tiles; otherwise a block has exactly one tile and no loop in its instruction stream.
 template <int VEC, int TIER, typename IndexT, bool STRIDE>
 __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, uint32_t cpr, uint32_t magic, const IndexT* __restrict__ index,
     int64_t total_chunks, const int64_t* __restrict__ n_rows_dev, int64_t row_lo, int64_t row_hi,
     int64_t* __restrict__ bad_index, char* __restrict__ out) {
-  using C = typename Chunk<VEC>::type;
-  bool bad = false;
   if (n_rows_dev) total_chunks = *n_rows_dev * cpr;  // row count decided on the device
-  // STRIDE: the grid is smaller than the tile count (capped launch), blocks stride over the tiles
-  for (int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock; c0 < total_chunks;
-       c0 += STRIDE ? int64_t(gridDim.x) * kChunksPerBlock : total_chunks) {
-    const int64_t row0 = c0 / cpr;
-    const uint32_t rem0 = uint32_t(c0 - row0 * cpr);
-
-    C val[kGatherUnroll];
-    bool ok[kGatherUnroll];
-#pragma unroll
-    for (int u = 0; u < kGatherUnroll; ++u) {
-      const uint32_t t = u * kGatherThreads + threadIdx.x;
-      ok[u] = c0 + t < total_chunks;
-      if (ok[u]) {
-        const uint32_t lc = rem0 + t;
-        const uint32_t q = cpr == 1 ? lc : __umulhi(lc, magic);
-        const uint32_t col = lc - q * cpr;
-        const int64_t src_row = int64_t(index[row0 + q]);
-        if (src_row >= row_lo && src_row < row_hi) {
-          const int64_t g = src_row * row_bytes + int64_t(col) * VEC;
-          val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
-        } else {
-          val[u] = C(0);
-          bad = true;
-        }
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < kGatherUnroll; ++u) {
-      const uint32_t t = u * kGatherThreads + threadIdx.x;
-      if (ok[u]) __builtin_nontemporal_store(val[u], reinterpret_cast<C*>(out + (c0 + t) * VEC));
-    }
+  bool bad = false;
+  if (STRIDE) {
+    for (int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock; c0 < total_chunks;
+         c0 += int64_t(gridDim.x) * kChunksPerBlock)
+      bad |= gather_tile<VEC, TIER, IndexT>(dev, host, thr_bytes, row_bytes, cpr, magic, index, total_chunks, row_lo,
+                                            row_hi, out, c0);
+  } else {
+    const int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock;
+    if (c0 < total_chunks)
+      bad = gather_tile<VEC, TIER, IndexT>(dev, host, thr_bytes, row_bytes, cpr, magic, index, total_chunks, row_lo,
+                                           row_hi, out, c0);
   }
   if (bad && bad_index) *bad_index = 1;
 }
 
-// Rows wider than kMaxFlatChunksPerRow chunks: a block owns one segment of
-// kChunksPerBlock chunks of one row.
+// Rows wider than kMaxFlatChunksPerRow chunks, and any launch whose tier holds no whole row
+// (every id is refused): a block owns one segment of kChunksPerBlock chunks of one row.
 template <int VEC, int TIER, typename IndexT>
 __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
@@ -132,7 +165,7 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
   const int64_t row_hi = TIER == DGS_TIER_DEVICE ? thr_bytes / row_bytes : n_rows;
   const char* dev = static_cast<const char*>(v.dev);
   const char* host = static_cast<const char*>(v.host);
-  if (cpr <= kMaxFlatChunksPerRow) {
+  if (cpr <= kMaxFlatChunksPerRow && row_lo < row_hi) {
     const int64_t total_chunks = n * cpr;
     const int64_t tiles = (total_chunks + kChunksPerBlock - 1) / kChunksPerBlock;
     int64_t blocks = tiles;

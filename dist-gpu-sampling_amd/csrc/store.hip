@@ -65,6 +65,50 @@ DGS_API dgs_status dgs_debug_set(int32_t option, int64_t value) {
   return DGS_OK;
 }
 
+namespace dgs {
+namespace {
+template <int OP>
+__global__ __launch_bounds__(256) void probe_table_kernel(unsigned long long* __restrict__ table, uint64_t slots,
+                                                          int64_t n_ops, uint64_t salt,
+                                                          unsigned long long* __restrict__ sink) {
+  const int64_t j = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (j >= n_ops) return;
+  uint64_t x = uint64_t(j) * 0x9E3779B97F4A7C15ull + salt;
+  x ^= x >> 31;
+  x *= 0xBF58476D1CE4E5B9ull;
+  x ^= x >> 29;
+  unsigned long long* slot = table + x % slots;  // always inside the table
+  unsigned long long seen = ~0ull;
+  if (OP == DGS_PROBE_LOAD) seen = __builtin_nontemporal_load(slot);
+  if (OP == DGS_PROBE_STORE) *slot = static_cast<unsigned long long>(j);
+  if (OP == DGS_PROBE_ATOMIC_MIN) seen = atomicMin(slot, static_cast<unsigned long long>(j) | (salt << 40));
+  if (OP == DGS_PROBE_ATOMIC_MIN_NO_RETURN) atomicMin(slot, static_cast<unsigned long long>(j) | (salt << 40));
+  if (seen == 0x0123456789abcdefull) *sink = seen;  // keeps the value alive; practically never taken
+}
+}  // namespace
+}  // namespace dgs
+
+DGS_API dgs_status dgs_debug_probe_table(int32_t op, void* table, int64_t slots, int64_t n_ops, uint64_t salt,
+                                         void* sink, void* stream) {
+  using namespace dgs;
+  DGS_REQUIRE(op >= DGS_PROBE_LOAD && op <= DGS_PROBE_ATOMIC_MIN_NO_RETURN, DGS_ERR_INVALID, "probe: unknown op %d", op);
+  DGS_REQUIRE(table != nullptr && sink != nullptr && slots > 0, DGS_ERR_INVALID, "probe: null table or no slots");
+  DGS_REQUIRE(n_ops >= 0 && n_ops <= (int64_t(1) << 38), DGS_ERR_INVALID, "probe: n_ops=%lld", (long long)n_ops);
+  if (n_ops == 0) return DGS_OK;
+  const dim3 grid(uint32_t((n_ops + 255) / 256)), block(256);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  auto* t = static_cast<unsigned long long*>(table);
+  auto* k = static_cast<unsigned long long*>(sink);
+  switch (op) {
+    case DGS_PROBE_LOAD: hipLaunchKernelGGL(probe_table_kernel<DGS_PROBE_LOAD>, grid, block, 0, st, t, uint64_t(slots), n_ops, salt, k); break;
+    case DGS_PROBE_STORE: hipLaunchKernelGGL(probe_table_kernel<DGS_PROBE_STORE>, grid, block, 0, st, t, uint64_t(slots), n_ops, salt, k); break;
+    case DGS_PROBE_ATOMIC_MIN: hipLaunchKernelGGL(probe_table_kernel<DGS_PROBE_ATOMIC_MIN>, grid, block, 0, st, t, uint64_t(slots), n_ops, salt, k); break;
+    default: hipLaunchKernelGGL(probe_table_kernel<DGS_PROBE_ATOMIC_MIN_NO_RETURN>, grid, block, 0, st, t, uint64_t(slots), n_ops, salt, k); break;
+  }
+  DGS_LAUNCH_CHECK();
+  return DGS_OK;
+}
+
 DGS_API dgs_status dgs_store_split(int64_t total_elems, int32_t elem_bytes, int64_t capacity_bytes,
                                    int64_t* device_elems, int64_t* host_elems) {
   DGS_REQUIRE(total_elems >= 0, DGS_ERR_INVALID, "store: negative element count %lld",

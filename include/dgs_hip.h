@@ -64,6 +64,23 @@ enum {
 };
 dgs_status dgs_debug_set(int32_t option, int64_t value);
 
+/*
+ * Measurement aid, no counterpart in the reference: `n_ops` threads each touch one 8-byte
+ * slot of `table` (`slots` of them, device memory), slot = a hash of (thread index, salt)
+ * reduced modulo `slots`, with
+ *   DGS_PROBE_LOAD        a load,
+ *   DGS_PROBE_STORE       a store of the thread's index,
+ *   DGS_PROBE_ATOMIC_MIN  an atomicMin with the old value returned (what the fused sampler does
+ *                         once per pick on its node table),
+ *   DGS_PROBE_ATOMIC_MIN_NO_RETURN  the same without using the old value.
+ * What the loads and atomics returned is folded into *sink (8 bytes of device memory) so that
+ * nothing is optimised away.  Timed by the caller (events on `stream`), it gives the rate at
+ * which this GPU serves random 8-byte accesses of each kind: the bound of the table kernels.
+ */
+enum { DGS_PROBE_LOAD = 0, DGS_PROBE_STORE = 1, DGS_PROBE_ATOMIC_MIN = 2, DGS_PROBE_ATOMIC_MIN_NO_RETURN = 3 };
+dgs_status dgs_debug_probe_table(int32_t op, void* table, int64_t slots, int64_t n_ops, uint64_t salt,
+                                 void* sink, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Two-tier positional store (ChunkTensor)                                   */
 /* ------------------------------------------------------------------------ */

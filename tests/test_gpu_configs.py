@@ -123,10 +123,11 @@ def _check_properties(pkg, indptr, indices, seeds, fanouts, replace, frontier, b
 
 
 def _run_case(pkg, oracle, indptr, indices, feats, feat_capacity, seeds, fanouts, replace, oracle_parity=True,
-              graph_capacity=1 << 62):
+              graph_capacity=1 << 62, ct_x=None):
     ct_ip = _store_from_device(pkg, indptr, graph_capacity)
     ct_ix = _store_from_device(pkg, indices, graph_capacity)
-    ct_x = _store_from_device(pkg, feats, feat_capacity)
+    if ct_x is None:
+        ct_x = _store_from_device(pkg, feats, feat_capacity)
     sampler = pkg.ChunkTensorSampler(fanouts, ct_ip, ct_ix, replace=replace)
     pkg.set_rng_state(20240601, 0)
     frontier, _, blocks, x = sampler.sample_blocks_and_index(None, seeds, ct_x)
@@ -202,11 +203,10 @@ def test_config2_large_graph_int32_ids_bf16(pkg, oracle):
     _free()
 
 
-def test_config3_two_tier_features(pkg, oracle):
-    # the large graph's shape at 1/8 scale with f32 x256 features: the top 40% of rows (ids are
-    # assigned in decreasing in-degree) in HBM, the rest in pinned host memory; 8192 seeds, [20, 15, 10]
+def _config3(pkg, oracle, n, e):
+    """The large graph's shape with f32 x256 features: the top 40% of rows (ids are assigned in
+    decreasing in-degree) in HBM, the rest in pinned host memory; int32 ids, 8192 seeds, [20, 15, 10]."""
     gen = torch.Generator(device="cuda").manual_seed(20240604)
-    n, e = 13_882_494, 201_960_734
     deg = _powerlaw_degrees(n, e, 30_000, 0.05, gen)
     deg = torch.sort(deg, descending=True).values  # hottest rows first
     indptr, indices = _csc_uniform_sources(n, deg, torch.int32, gen)
@@ -216,20 +216,40 @@ def test_config3_two_tier_features(pkg, oracle):
         feats[a: a + (1 << 22)].normal_(generator=gen)
     hot_rows = int(n * 0.4)
     capacity = hot_rows * 256 * 4 + 4 * 100  # the boundary falls inside a row
+    host_bytes = n * 256 * 4 - capacity
+    try:
+        ct_x = _store_from_device(pkg, feats, capacity)
+    except RuntimeError as err:  # the one thing that depends on the machine: pinning the host slice
+        del indptr, indices, feats
+        _free()
+        pytest.skip(f"the {host_bytes / 1e9:.1f} GB host slice could not be allocated as pinned memory: {err}")
     seeds = torch.randint(0, n, (8192,), generator=gen, device="cuda", dtype=torch.int32)
-    rows, edges = _run_case(pkg, oracle, indptr, indices, feats, capacity, seeds, [20, 15, 10], False)
+    rows, edges = _run_case(pkg, oracle, indptr, indices, feats, capacity, seeds, [20, 15, 10], False, ct_x=ct_x)
     assert rows > 1_000_000
-    # tier-specific gathers on the partitioned frontier give the same rows
-    ct_x = _store_from_device(pkg, feats, capacity)
+    # tier-specific gathers on the partitioned frontier give the same rows (the straddling row
+    # hot_rows counts as a host row)
     idx = torch.randint(0, n, (200_000,), generator=gen, device="cuda")
+    idx[:3] = torch.tensor([hot_rows - 1, hot_rows, hot_rows + 1], device="cuda")
     local, remote, host = ct_x._CAPI_split_index(idx)
     assert remote.numel() == 0 and local.numel() + host.numel() == idx.numel()
     assert torch.equal(local, idx[idx < hot_rows]) and torch.equal(host, idx[idx >= hot_rows])
-    host_only = host[host > hot_rows]
     assert torch.equal(ct_x._CAPI_local_index(local), feats[local])
-    assert torch.equal(ct_x._CAPI_host_index(host_only), feats[host_only])
+    assert torch.equal(ct_x._CAPI_host_index(host), feats[host])
     del indptr, indices, feats, ct_x
     _free()
+    return rows, edges
+
+
+def test_config3_two_tier_features(pkg, oracle):
+    # 1/8 of the full size: 5.7 GB in HBM, 8.5 GB pinned
+    _config3(pkg, oracle, 13_882_494, 201_960_734)
+
+
+@pytest.mark.timeout(900)
+def test_config3_two_tier_features_full_size(pkg, oracle):
+    # 111,059,956 nodes / 1,615,685,872 edges, 113.7 GB of features: 45.5 GB in HBM, 68.2 GB pinned
+    rows, edges = _config3(pkg, oracle, 111_059_956, 1_615_685_872)
+    assert rows > 2_000_000 and edges > rows - 8192
 
 
 def _rmat_csc(scale, e, gen):
