@@ -236,7 +236,7 @@ def run_batches(sampler, seed_batches, features, inflight, consume=lambda r: Non
     return [consume(r) for r in pipeline(seed_batches)]
 
 
-def table_access_rates(dgs, slots, n_ops, reps=10):
+def table_access_rates(dgs, slots, n_ops, reps=50):
     """Random 8-byte accesses per second this GPU serves on a table of `slots` slots, by kind:
     the library's probe kernel (one access per thread, nothing else), timed with events on the
     stream it is launched on.  The fused sampler does one atomicMin with return per pick on a
@@ -248,11 +248,15 @@ def table_access_rates(dgs, slots, n_ops, reps=10):
     for name, op in (("load", capi.PROBE_LOAD), ("store", capi.PROBE_STORE),
                      ("atomic_min_with_return", capi.PROBE_ATOMIC_MIN),
                      ("atomic_min_no_return", capi.PROBE_ATOMIC_MIN_NO_RETURN)):
-        salt = [0]
-        def once():
-            salt[0] += 1
-            capi.probe_table(op, table, n_ops, salt[0], sink)
-        t = time_call(once, reps)
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        capi.probe_table(op, table, n_ops, 0, sink)
+        torch.cuda.synchronize()
+        begin.record()
+        for rep in range(reps):  # back to back, so that the gaps around a single short launch do not count
+            capi.probe_table(op, table, n_ops, 1 + rep, sink)
+        end.record()
+        torch.cuda.synchronize()
+        t = begin.elapsed_time(end) * 1e-3 / reps
         out[name] = n_ops / t / 1e9
         out[name + "_us"] = 1e6 * t
     return out
@@ -361,19 +365,21 @@ def run_large(args, dgs):
     inflight = args.inflight if cfg["hbm_rows"] >= 1.0 else 1
     run_batches(sampler, seeds[:args.warmup], ct_x, inflight)
     torch.cuda.synchronize()
-    edges = rows = 0
-    frontiers = []
+    frontiers = []  # the first few, for the gather leg below; of the other batches only the lengths are kept
+    def keep(r):
+        if len(frontiers) < 8:
+            frontiers.append(r[0])
+        return r[0].numel(), sum(b.src_local.numel() for b in r[2])
+    resident = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
     t0 = time.perf_counter()
-    results = run_batches(sampler, seeds[args.warmup:], ct_x, inflight,
-                          lambda r: (r[0], sum(b.src_local.numel() for b in r[2])))
+    results = run_batches(sampler, seeds[args.warmup:], ct_x, inflight, keep)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    for frontier, n_edges in results:
-        edges += n_edges
-        rows += frontier.numel()
-        if len(frontiers) < 8:
-            frontiers.append(frontier)
-    del results
+    peak_batch_bytes = torch.cuda.max_memory_allocated() - resident
+    rows = sum(r[0] for r in results)
+    edges = sum(r[1] for r in results)
+    frontier = frontiers[-1]
     row_bytes = dim * eb
     # the gather alone, once per kept frontier (a repeat of the same rows would be served by the
     # 256 MB last-level cache), events on the launching stream, queued back to back
@@ -401,6 +407,10 @@ def run_large(args, dgs):
                    "batches_in_flight": inflight},
         "avg_frontier_rows": rows / args.steps, "avg_edges_per_batch": edges / args.steps,
         "gather_ms": 1e3 * t_mixed, "gather_GBps": gather_gbps, "graph_gen_s": t_gen,
+        # torch allocations of the batches in flight at their peak (outputs, workspaces, kept frontiers),
+        # beyond what was resident before the timed loop; the stores themselves are not torch memory
+        "peak_batch_bytes": peak_batch_bytes,
+        "gather_buffer_cap_bytes": int(torch.ops.dgs_ops._CAPI_get_gather_buffer_cap()),
     }
     if cfg["hbm_rows"] < 1.0:
         local, _, host_ids = ct_x._CAPI_split_index(frontier)
@@ -431,8 +441,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + sorted(LARGE))
     ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
-    ap.add_argument("--inflight", type=int, default=2,
+    ap.add_argument("--inflight", type=int, default=3,
                     help="batches in flight on as many streams (1 = one blocking call per batch)")
+    ap.add_argument("--gather-buffer-cap-gib", type=float, default=None,
+                    help="largest feature buffer the fused operator allocates ahead of a batch's sizes "
+                         "(the library's default when not given)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
@@ -446,6 +459,8 @@ def main():
 
     dgs = importlib.import_module("dist-gpu-sampling_amd")
     torch.cuda.set_device(0)
+    if args.gather_buffer_cap_gib is not None:
+        dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
     if args.workload in LARGE:
         return run_large(args, dgs)
     cfg = WORKLOADS[args.workload]
@@ -618,8 +633,9 @@ def main():
         "graph_gen_s": t_gen,
     }
     if args.workload != "c0":
-        # one access per pick of the widest hop, on a table the size of the sampler's node table
-        out["table_access_rates"] = table_access_rates(dgs, cfg["nodes"], int(max(h[1] for h in stats[0]["hops"])))
+        # on a table the size of the sampler's node table; eight times the picks of the widest hop per
+        # launch, so that a launch lasts long enough for the host's launch rate not to show
+        out["table_access_rates"] = table_access_rates(dgs, cfg["nodes"], 8 * int(max(h[1] for h in stats[0]["hops"])))
     if cfg.get("weighted"):
         # the weighted fill of the widest hop alone: its input is every weight of every sampled row
         ops = torch.ops.dgs_ops

@@ -23,6 +23,7 @@
 //     sampling raises; a gather zero-fills the row and the store raises at its next call.
 #include <c10/hip/HIPFunctions.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/StreamGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/custom_class.h>
 #include <torch/script.h>
@@ -566,7 +567,7 @@ class PendingBlocks : public torch::CustomClassHolder {
     TORCH_CHECK(!finished_, "PendingBlocks: already finished");
     finished_ = true;
     dgs_status ws_status = DGS_OK;
-    if (ticket_ != nullptr) {  // still null when Begin had to wait for the sizes itself
+    if (ticket_ != nullptr) {
       void* t = ticket_;
       ticket_ = nullptr;
       ws_status = dgs_ticket_wait(t);
@@ -583,8 +584,21 @@ class PendingBlocks : public torch::CustomClassHolder {
       src_[h] = src_[h].narrow(0, 0, sz[hops_ + 1 + h]);
       dst_[h] = dst_[h].narrow(0, 0, sz[hops_ + 1 + h]);
     }
-    if (x_.defined()) x_ = x_.narrow(0, 0, sz[hops_]);
-    return std::make_tuple(frontier, src_, dst_, x_.defined() ? x_ : torch::empty({0}, seeds_.options()), seeds_);
+    if (features_) {
+      const int64_t rows = sz[hops_];
+      if (rows <= x_rows_) {
+        x_ = x_.narrow(0, 0, rows);
+      } else {
+        // the frontier did not fit the capped buffer and the gather enqueued behind the last hop
+        // wrote nothing: gather now into exactly `rows` rows, on the stream the batch was begun on
+        // (the lengths are final, so the frontier is complete)
+        const c10::StreamGuard on_begin_stream(stream_);
+        x_ = torch::empty({rows, features_->elem_stride()}, x_.options());
+        check(dgs_gather_rows(features_->view(), features_->elem_stride(), all_.data_ptr(), width_, rows,
+                              x_.data_ptr(), DGS_TIER_ANY, features_->bad_index_word(), current_stream()));
+      }
+    }
+    return std::make_tuple(frontier, src_, dst_, features_ ? x_ : torch::empty({0}, seeds_.options()), seeds_);
   }
 
   static c10::intrusive_ptr<PendingBlocks> Begin(const torch::Tensor& seeds_in,
@@ -654,25 +668,22 @@ class PendingBlocks : public torch::CustomClassHolder {
     if (features) {
       const auto xopt = torch::TensorOptions().dtype(features->dtype()).device(dev);
       const int64_t row_bytes = features->elem_stride() * static_cast<int64_t>(c10::elementSize(features->dtype()));
-      if (seeds_max[hops] * row_bytes <= g_gather_buffer_cap.load()) {
-        // the lengths are final at the ticket; the gather is enqueued before anybody waits for
-        // them, into a buffer for the worst case of which the result is a prefix
-        p->x_ = torch::empty({seeds_max[hops], features->elem_stride()}, xopt);
+      // The lengths are final at the ticket; the gather is enqueued before anybody waits for them,
+      // into a buffer of which the result is a prefix: one for the worst case, or, where that would
+      // exceed the cap (the worst case grows with the product of the fanouts, the frontier does
+      // not), the largest the cap allows.  A frontier that does not fit such a buffer is left
+      // alone by the kernel and gathered in Finish, into exactly its size.
+      int64_t buffer_rows = seeds_max[hops];
+      if (buffer_rows * row_bytes > g_gather_buffer_cap.load()) buffer_rows = g_gather_buffer_cap.load() / row_bytes;
+      p->features_ = features;
+      p->width_ = w;
+      p->stream_ = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap();
+      p->x_rows_ = buffer_rows > 0 ? buffer_rows : -1;
+      p->x_ = torch::empty({buffer_rows, features->elem_stride()}, xopt);
+      if (buffer_rows > 0)
         p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
-                                                seeds_max[hops], sizes_dev.data_ptr<int64_t>() + hops,
+                                                buffer_rows, sizes_dev.data_ptr<int64_t>() + hops,
                                                 p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
-      } else {
-        // the worst case would be too large a buffer (it grows with the product of the fanouts,
-        // the frontier does not): wait for the frontier's size and gather into exactly that many
-        // rows, as upstream's exact-size output (src/cuda/index_with_chunk_tensor.cu:29-53)
-        void* t = p->ticket_;
-        p->ticket_ = nullptr;
-        check(dgs_ticket_wait(t));
-        const int64_t rows = p->pinned_.data_ptr<int64_t>()[hops];
-        p->x_ = torch::empty({rows, features->elem_stride()}, xopt);
-        p->gather_status_ = dgs_gather_rows(features->view(), features->elem_stride(), p->all_.data_ptr(), w, rows,
-                                            p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
-      }
     }
     return p;
   }
@@ -684,6 +695,12 @@ class PendingBlocks : public torch::CustomClassHolder {
   dgs_status gather_status_ = DGS_OK;
   torch::Tensor pinned_, seeds_, all_, x_;
   std::vector<torch::Tensor> src_, dst_;
+  // the feature gather: rows of the buffer it was enqueued into (-1: none), and what a second,
+  // exact gather in Finish needs
+  c10::intrusive_ptr<ChunkTensor> features_;
+  int64_t x_rows_ = -1;
+  int32_t width_ = 0;
+  c10::Stream stream_ = c10::Stream(c10::Stream::DEFAULT, c10::Device(c10::DeviceType::CPU, -1));
 };
 
 namespace {

@@ -191,7 +191,13 @@ __device__ __forceinline__ void offsets_tile(const Hop& h, int tile) {
 // One block per (256-row tile, 256 padded picks): writes the rows' edges at their packed
 // offsets.  src_local = rank of the picked id; dst_local = rank of the row's seed, which is
 // the row number itself except in hop 0, whose seeds may repeat.
-template <typename IdT, typename TableT>
+//
+// EARLY (here and in the other tile functions): the launch is about as large as the hop really
+// is, so a thread requests its own elements together with the hop's length and tests afterwards.
+// Without it the launch was sized for a worst case that may exceed the hop many times over
+// (and loops over its virtual blocks): the length is waited for first and blocks beyond it
+// leave without having read anything.
+template <typename IdT, typename TableT, bool EARLY>
 __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, int64_t b) {
   __shared__ int64_t lds[kBlock / kWave];
   const int k = h.k;
@@ -204,6 +210,7 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   const int64_t i = tile * kRowTile + r;
   // the hop's length and this thread's own row and pick, requested together
   const int64_t s = seeds_of(h);
+  if (!EARLY && tile * kRowTile >= s) return;
   const bool mine = r < kRowTile && i < h.s_max;
   // (hop 0's seed part is the caller's count, a kernel argument: p hangs on no load)
   const int64_t p = h.pos_base + (h.index == 0 ? h.n_seeds_host : 0) + i * k + l;
@@ -278,13 +285,15 @@ __device__ __forceinline__ bool look_before_insert(const Hop& h, int64_t s) {
 }
 
 // One virtual block of the fill launch: 256 / G seed rows.
-template <typename IdT, typename PtrT, typename TableT, int G>
+template <typename IdT, typename PtrT, typename TableT, int G, bool EARLY>
 __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT& table,
                                           const TierView<PtrT>& indptr, const TierView<IdT>& indices,
                                           bool replace, uint64_t rng_seed) {
   const int64_t gid = vb * kBlock + threadIdx.x;
   const int64_t i = gid / G;
   const int l = int(gid % G);
+  // a launch sized far beyond the hop: blocks past its end wait for nothing but the length
+  if (!EARLY && vb != 0 && vb * (kBlock / G) >= seeds_of(h)) return;
   // the hop's length, what the previous hop found, and this group's seed id, requested together
   // (the seed list has room for s_max ids whatever the length turns out to be)
   const IdT seed = i < h.s_max ? static_cast<const IdT*>(h.seeds)[i] : IdT(0);
@@ -335,9 +344,9 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
   const int64_t total = fill_blocks + relabel_count + clear_blocks;
   DGS_FOR_VIRTUAL_BLOCKS(vb, total) {
     if (vb < fill_blocks) {
-      fill_rows<IdT, PtrT, TableT, G>(h, vb, table, indptr, indices, replace, rng_seed);
+      fill_rows<IdT, PtrT, TableT, G, !STRIDE>(h, vb, table, indptr, indices, replace, rng_seed);
     } else if (vb < fill_blocks + relabel_count) {
-      relabel_tile<IdT, TableT>(prev, table, vb - fill_blocks);
+      relabel_tile<IdT, TableT, !STRIDE>(prev, table, vb - fill_blocks);
     } else {
       const int64_t i = (vb - fill_blocks - relabel_count) * kBlock + threadIdx.x;
       if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
@@ -444,7 +453,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(5, 8))) 
     if (vb < fill_blocks) {
       fill_rows_weighted<IdT, PtrT, TableT, REPLACE>(h, vb, table, indptr, indices, probs, rng_seed);
     } else if (vb < fill_blocks + relabel_count) {
-      relabel_tile<IdT, TableT>(prev, table, vb - fill_blocks);
+      relabel_tile<IdT, TableT, false>(prev, table, vb - fill_blocks);  // always a striding launch
     } else {
       const int64_t i = (vb - fill_blocks - relabel_count) * kBlock + threadIdx.x;
       if (i < clear_n16) clear_begin[i] = make_uint4(0u, 0u, 0u, 0u);
@@ -483,21 +492,26 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
 }
 
 // One virtual block of the flag launch: 1024 padded positions.
-template <typename IdT, typename TableT>
+template <typename IdT, typename TableT, bool EARLY>
 __device__ __forceinline__ void flag_tile(const Hop& h, int64_t tile, const TableT& table) {
   __shared__ int lds[kBlock / kWave];
   const int64_t s = seeds_of(h);
+  const int64_t len = seed_part(h, s) + s * h.k;
+  if (!EARLY && tile * kPosTile >= len) {
+    if (threadIdx.x == 0) h.pos_cnt[tile] = 0;
+    return;
+  }
   const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
-  // this thread's slot words and lost marks, requested together with the hop's length
+  // this thread's slot words and lost marks (EARLY: requested together with the hop's length)
+  const int64_t readable = EARLY ? h.len_max : len;
   uint32_t w[kPosItems];
   uint8_t gone[kPosItems];
 #pragma unroll
   for (int j = 0; j < kPosItems; ++j) {
-    const bool inside = base + j < h.len_max;
+    const bool inside = base + j < readable;
     w[j] = inside ? h.slot[h.pos_base + base + j] : kInvalidSlot;
     gone[j] = inside && h.index != 0 ? h.lost[h.pos_base + base + j] : uint8_t(0);
   }
-  const int64_t len = seed_part(h, s) + s * h.k;
   int c = 0;
   if (tile * kPosTile < len) {
 #pragma unroll
@@ -526,40 +540,46 @@ template <typename IdT, typename TableT, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_flag_kernel(Hop h, int64_t flag_blocks, int64_t row_tiles,
                                                           TableT table) {
   DGS_FOR_VIRTUAL_BLOCKS(vb, flag_blocks + row_tiles) {
-    if (vb < flag_blocks) flag_tile<IdT, TableT>(h, vb, table);
+    if (vb < flag_blocks) flag_tile<IdT, TableT, !STRIDE>(h, vb, table);
     else offsets_tile(h, int(vb - flag_blocks));
   }
 }
 
-// Separate scans for very long tile lists (one block), over the worst-case tile counts (the
-// counts of tiles beyond the hop's real length are zero).
-__global__ __launch_bounds__(1024) void pos_scan_kernel(Hop h, int64_t pos_tiles) {
-  int64_t sum;
-  single_block_scan<1024, int, int64_t>(h.pos_cnt, h.pos_off, pos_tiles, &sum);
+// Separate scans for very long tile lists (one block), over the tiles the hop really has.
+__device__ __forceinline__ int64_t real_pos_tiles(const Hop& h, int64_t s) {
+  return (seed_part(h, s) + s * h.k + kPosTile - 1) / kPosTile;
 }
-__global__ __launch_bounds__(1024) void tile_scan_kernel(Hop h, int64_t row_tiles) {
+__global__ __launch_bounds__(1024) void pos_scan_kernel(Hop h) {
   int64_t sum;
-  single_block_scan<1024, int, int64_t>(h.tile_sum, h.tile_off, row_tiles, &sum);
+  single_block_scan<1024, int, int64_t>(h.pos_cnt, h.pos_off, real_pos_tiles(h, seeds_of(h)), &sum);
+}
+__global__ __launch_bounds__(1024) void tile_scan_kernel(Hop h) {
+  int64_t sum;
+  single_block_scan<1024, int, int64_t>(h.tile_sum, h.tile_off, (seeds_of(h) + kRowTile - 1) / kRowTile, &sum);
 }
 
 // One virtual block of the compact launch: the first occurrences of one 1024-position tile.
 // `pos_tiles` / `row_tiles` are the worst-case tile counts the flag launch covered: the counts of
 // tiles beyond the hop's real length are zero there, so sums may run over all of them.
-template <typename IdT, typename TableT>
+template <typename IdT, typename TableT, bool EARLY>
 __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, int64_t pos_tiles, int64_t row_tiles,
                                              const TableT& table) {
   __shared__ int64_t lds64[kBlock / kWave];
   __shared__ int lds[kBlock / kWave];
-  // the hop's length, this thread's slot words and its share of the tile counts, requested together
+  // the hop's length, this thread's slot words and its share of the tile counts (EARLY: requested together)
   const int64_t s = seeds_of(h);
+  const int64_t len = seed_part(h, s) + s * h.k;
+  if (!EARLY && tile != 0 && tile * kPosTile >= len) return;
   const int64_t base = tile * kPosTile + threadIdx.x * kPosItems;
+  const int64_t readable = EARLY ? h.len_max : len;
   uint32_t w[kPosItems];
 #pragma unroll
-  for (int j = 0; j < kPosItems; ++j) w[j] = base + j < h.len_max ? h.slot[h.pos_base + base + j] : kInvalidSlot;
+  for (int j = 0; j < kPosItems; ++j) w[j] = base + j < readable ? h.slot[h.pos_base + base + j] : kInvalidSlot;
   // first occurrences in the tiles before this one (block 0 needs the grand total instead)
   int64_t part = 0;
-  if (h.pos_off) {
-    if (threadIdx.x == 0) part = tile == 0 ? h.pos_off[pos_tiles - 1] + h.pos_cnt[pos_tiles - 1] : h.pos_off[tile];
+  if (h.pos_off) {  // scanned by pos_scan_kernel over the hop's real tiles
+    const int64_t last = real_pos_tiles(h, s) - 1;
+    if (threadIdx.x == 0) part = tile != 0 ? h.pos_off[tile] : last >= 0 ? h.pos_off[last] + h.pos_cnt[last] : 0;
   } else {
     const int64_t upto = tile == 0 ? pos_tiles : tile;
     for (int64_t j = threadIdx.x; j < upto; j += kBlock) part += h.pos_cnt[j];
@@ -572,7 +592,6 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, int64_t
       bad |= h.tile_flag[j];
     }
   }
-  const int64_t len = seed_part(h, s) + s * h.k;
   const int64_t rank0 = first_rank(h, s);
   if (tile != 0 && tile * kPosTile >= len) return;  // whole blocks leave together
   part = block_sum<kBlock, int64_t>(part, lds64);
@@ -616,12 +635,12 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, int64_t
 template <typename IdT, typename TableT, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_compact_kernel(Hop h, int64_t blocks, int64_t pos_tiles,
                                                              int64_t row_tiles, TableT table) {
-  DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) compact_tile<IdT, TableT>(h, vb, pos_tiles, row_tiles, table);
+  DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) compact_tile<IdT, TableT, !STRIDE>(h, vb, pos_tiles, row_tiles, table);
 }
 
 template <typename IdT, typename TableT, bool STRIDE>
 __global__ __launch_bounds__(kBlock) void hop_relabel_kernel(Hop h, int64_t blocks, TableT table) {
-  DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) relabel_tile<IdT, TableT>(h, table, vb);
+  DGS_FOR_VIRTUAL_BLOCKS(vb, blocks) relabel_tile<IdT, TableT, !STRIDE>(h, table, vb);
 }
 
 __global__ void zero_sizes_kernel(int64_t* __restrict__ sizes, int n) {
@@ -805,11 +824,11 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
                          dim3(kBlock), 0, st, cur, pos_tiles, row_tiles, table);
     DGS_LAUNCH_CHECK();
     if (cur.pos_off) {
-      hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur, pos_tiles);
+      hipLaunchKernelGGL(pos_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
       DGS_LAUNCH_CHECK();
     }
     if (cur.tile_off) {
-      hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, cur, row_tiles);
+      hipLaunchKernelGGL(tile_scan_kernel, dim3(1), dim3(1024), 0, st, cur);
       DGS_LAUNCH_CHECK();
     }
     const int64_t compact_blocks = pos_tiles > 0 ? pos_tiles : 1;  // block 0 always writes the lengths

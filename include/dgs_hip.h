@@ -173,10 +173,12 @@ dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
 
 /*
  * Same gather with the row count read from device memory when the kernel runs:
- * `n_rows_dev` points to an int64 <= n_max; the launch is sized for n_max rows and
- * `out` must hold n_max rows.  Lets a caller enqueue the gather of a frontier whose
- * length a previous kernel on the same stream is still computing.  No counterpart in
- * the reference (which reads every length back to the host first).
+ * `n_rows_dev` points to an int64; the launch is sized for n_max rows and `out` must
+ * hold n_max rows.  A count above n_max (or below 0) gathers nothing at all, so a
+ * caller may offer a buffer smaller than the worst case and gather again, exactly,
+ * when the count turns out not to fit.  Lets a caller enqueue the gather of a frontier
+ * whose length a previous kernel on the same stream is still computing.  No
+ * counterpart in the reference (which reads every length back to the host first).
  */
 dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
                                int32_t index_bytes, int64_t n_max,

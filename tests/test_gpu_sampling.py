@@ -168,8 +168,9 @@ def test_neighbour_ids_outside_the_graph_are_refused(pkg):
 
 
 def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph):
-    # when the worst-case feature buffer exceeds the cap the operator waits for the frontier size
-    # and gathers into exactly that many rows
+    # when the worst-case feature buffer exceeds the cap the gather goes into the largest buffer the
+    # cap allows, and a frontier that does not fit even that is gathered once its size is known,
+    # into exactly that many rows
     indptr, indices = graph
     ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
     ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
@@ -182,7 +183,7 @@ def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph):
     assert default_cap == 2 << 30
     results = []
     try:
-        for cap in (default_cap, 0, 600 * 7 * 10 * 48 * 4 - 1, 600 * 7 * 10 * 48 * 4):
+        for cap in (default_cap, 0, 600 * 7 * 10 * 48 * 4 - 1, 600 * 7 * 10 * 48 * 4, 1000 * 48 * 4):
             pkg.set_gather_buffer_cap(cap)
             pkg.set_rng_state(8, 8)
             torch.cuda.reset_peak_memory_stats()
@@ -200,7 +201,10 @@ def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph):
         assert np.array_equal(f.numpy(), o_frontier) and torch.equal(x, feats[f])
     worst = 600 * 7 * 10 * 48 * 4
     assert results[0][3] == worst and results[3][3] == worst            # ahead of the sizes: worst case
-    assert results[1][3] == results[1][0].numel() * 48 * 4 == results[2][3]  # capped: exactly the frontier
+    rows = results[1][0].numel()
+    assert 1000 < rows < 600 * 7 * 10 - 1
+    assert results[1][3] == rows * 48 * 4 == results[4][3]  # nothing fits the cap: exactly the frontier, afterwards
+    assert results[2][3] == (600 * 7 * 10 - 1) * 48 * 4      # the frontier fits what the cap allows
     assert results[1][2] < results[0][2]
 
 
