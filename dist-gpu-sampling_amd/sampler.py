@@ -220,7 +220,7 @@ class BatchPipeline:
     four streams a process makes do.
     """
 
-    def __init__(self, sampler, chunk_features=None, inflight=2, streams=None, hand_over=True):
+    def __init__(self, sampler, chunk_features=None, inflight=3, streams=None, hand_over=True):
         self.hand_over = hand_over
         if inflight < 1:
             raise ValueError("inflight must be at least 1")
