@@ -204,3 +204,29 @@ def test_gather_refuses_row_ids_outside_the_store(pkg):
     with pytest.raises(RuntimeError, match="outside the store"):
         ct._CAPI_index(torch.tensor([1], device="cuda"))
     assert torch.equal(ct._CAPI_index(torch.tensor([1], device="cuda")).cpu(), full[1:2])
+
+
+def test_probe_table_touches_only_its_table(pkg):
+    # the measurement aid behind bench.py's table_access_rates: every kind of access stays inside
+    # the table, loads change nothing, stores and atomics leave thread indices behind
+    capi = pkg.capi
+    slots, n_ops = 1000, 5000
+    guard = torch.full((slots + 2,), -7, dtype=torch.int64, device="cuda")
+    table = guard[1:-1]
+    sink = torch.zeros(1, dtype=torch.int64, device="cuda")
+    table.fill_(torch.iinfo(torch.int64).max)
+    capi.probe_table(capi.PROBE_LOAD, table, n_ops, 3, sink)
+    assert (table == torch.iinfo(torch.int64).max).all()
+    capi.probe_table(capi.PROBE_ATOMIC_MIN, table, n_ops, 0, sink)
+    touched = table[table != torch.iinfo(torch.int64).max]
+    assert 900 < touched.numel() <= slots and int(touched.max()) < n_ops and int(touched.min()) >= 0
+    before = table.clone()
+    capi.probe_table(capi.PROBE_ATOMIC_MIN_NO_RETURN, table, n_ops, 0, sink)  # the same values again: no change
+    assert torch.equal(table, before)
+    table.fill_(-1)
+    capi.probe_table(capi.PROBE_STORE, table, n_ops, 1, sink)
+    stored = table[table != -1]
+    assert 900 < stored.numel() <= slots and int(stored.max()) < n_ops and int(stored.min()) >= 0
+    assert int(guard[0]) == -7 and int(guard[-1]) == -7
+    with pytest.raises(RuntimeError):
+        capi.probe_table(9, table, n_ops, 0, sink)
