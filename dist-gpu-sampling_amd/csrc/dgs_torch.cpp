@@ -632,7 +632,15 @@ class PendingBlocks : public torch::CustomClassHolder {
     p->hops_ = hops;
     // the kernels mirror the lengths into this call's own pinned words
     p->pinned_ = torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-    p->seeds_ = seeds_in.to(dev, /*non_blocking=*/true).contiguous().view({-1});
+    if (seeds_in.device().is_cpu() && !seeds_in.is_pinned() && n > 0) {
+      // pageable host seeds (what upstream's DataLoader passes): staged through pinned memory of
+      // this batch, so that the upload is a plain asynchronous copy the host does not wait for
+      p->staged_seeds_ = torch::empty({n}, seeds_in.options().pinned_memory(true));
+      p->staged_seeds_.copy_(seeds_in.contiguous().view({-1}));
+      p->seeds_ = p->staged_seeds_.to(dev, /*non_blocking=*/true);
+    } else {
+      p->seeds_ = seeds_in.to(dev, /*non_blocking=*/true).contiguous().view({-1});
+    }
     const auto opt = p->seeds_.options();
     p->src_.resize(hops);
     p->dst_.resize(hops);
@@ -694,6 +702,7 @@ class PendingBlocks : public torch::CustomClassHolder {
   void* ticket_ = nullptr;
   dgs_status gather_status_ = DGS_OK;
   torch::Tensor pinned_, seeds_, all_, x_;
+  torch::Tensor staged_seeds_;  // pinned copy of host seeds, alive until the batch is finished
   std::vector<torch::Tensor> src_, dst_;
   // the feature gather: rows of the buffer it was enqueued into (-1: none), and what a second,
   // exact gather in Finish needs
