@@ -230,3 +230,45 @@ def test_probe_table_touches_only_its_table(pkg):
     assert int(guard[0]) == -7 and int(guard[-1]) == -7
     with pytest.raises(RuntimeError):
         capi.probe_table(9, table, n_ops, 0, sink)
+
+
+def test_gather_of_a_tier_that_holds_no_whole_row(pkg):
+    # a device slice shorter than one row holds no row whole: a device-tier gather refuses every
+    # id (and reads nothing), the per-chunk gather still serves the straddling row exactly
+    capi = pkg.capi
+    rows, dim = 50, 24
+    full = torch.randn((rows, dim))
+    st = capi.Store(rows * dim, 4, 10 * 4)  # 10 of row 0's 24 elements in HBM
+    st.load(full)
+    flag = torch.zeros(1, dtype=torch.int64, device="cuda")
+    idx = torch.tensor([0, 1, 49, 7], device="cuda")
+    out = capi.gather_rows(st.view, dim, idx, torch.float32, tier=capi.TIER_DEVICE, bad_index=flag)
+    assert flag.item() == 1 and (out == 0).all().item()
+    flag.zero_()
+    out = capi.gather_rows(st.view, dim, idx, torch.float32, bad_index=flag)
+    assert flag.item() == 0 and torch.equal(out.cpu(), full[idx.cpu()])
+    out = capi.gather_rows(st.view, dim, idx, torch.float32, tier=capi.TIER_HOST, bad_index=flag)  # row 0 straddles
+    assert flag.item() == 0 and torch.equal(out.cpu(), full[idx.cpu()])
+    st.close()
+
+
+@pytest.mark.parametrize("dim", [25, 40000 * 4])  # the flattened kernel and the one for very wide rows
+def test_gather_dyn_leaves_a_buffer_alone_that_is_too_small(pkg, dim):
+    # dgs_gather_rows_dyn with a device-side row count above the rows the output holds writes
+    # nothing; with a count that fits it gathers exactly that many rows
+    capi = pkg.capi
+    rows = 64 if dim > 1000 else 4000
+    full = torch.randn((rows, dim))
+    st = capi.Store(rows * dim, 4, 1 << 40)
+    st.load(full)
+    n_max = 40
+    idx = torch.randint(0, rows, (100,), device="cuda")
+    out = torch.full((n_max + 1, dim), -3.0, device="cuda")
+    for count, written in ((41, 0), (100, 0), (-1, 0), (40, 40), (7, 7), (0, 0)):
+        out.fill_(-3.0)
+        n_dev = torch.tensor([count], dtype=torch.int64, device="cuda")
+        capi.check(capi.lib.dgs_gather_rows_dyn(st.view, dim, idx.data_ptr(), 8, n_max, n_dev.data_ptr(), out.data_ptr(),
+                                                capi.TIER_ANY, None, capi.stream_ptr()))
+        assert torch.equal(out[:written].cpu(), full[idx[:written].cpu()]), count
+        assert (out[written:] == -3.0).all().item(), count
+    st.close()
