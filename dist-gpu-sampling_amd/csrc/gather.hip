@@ -23,7 +23,7 @@ constexpr int kChunksPerBlock = kGatherThreads * kGatherUnroll;
 constexpr uint32_t kMaxFlatChunksPerRow = 32768;
 // A launch sized for a worst-case row count (dgs_gather_rows_dyn) is capped at this many blocks;
 // blocks stride over the tiles, so a mostly unused worst case does not cost 10^5 empty blocks.
-constexpr int64_t kMaxDynGrid = 65536;
+constexpr int64_t kMaxDynGrid = 32768;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
