@@ -131,6 +131,9 @@ __device__ __forceinline__ int64_t seeds_of(const Hop& h) {
 __device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h.index == 0 ? s : 0; }
 // rank of the first id this hop can add: later hops append behind their seeds
 __device__ __forceinline__ int64_t first_rank(const Hop& h, int64_t s) { return h.index == 0 ? 0 : s; }
+constexpr int kRelabelItems = 4;  // padded picks per thread in relabel_tile
+__host__ __device__ __forceinline__ int relabel_groups(int k) { return (k + kRelabelItems - 1) / kRelabelItems; }
+
 // rank of the id at position p, given p's slot word
 template <typename TableT>
 __device__ __forceinline__ uint32_t rank_of(const Hop& h, const TableT& table, int64_t p, uint32_t slot_word) {
@@ -188,8 +191,9 @@ __device__ __forceinline__ void offsets_tile(const Hop& h, int tile) {
   }
 }
 
-// One block per (256-row tile, 256 padded picks): writes the rows' edges at their packed
-// offsets.  src_local = rank of the picked id; dst_local = rank of the row's seed, which is
+// One block per (256-row tile, 4 x 256 padded picks): writes the rows' edges at their packed
+// offsets; a thread handles four picks, 256 apart, so that a wave has four times the loads in
+// flight and the launch a quarter of the waves.  src_local = rank of the picked id; dst_local = rank of the row's seed, which is
 // the row number itself except in hop 0, whose seeds may repeat.
 //
 // EARLY (here and in the other tile functions): the launch is about as large as the hop really
@@ -202,24 +206,34 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   __shared__ int64_t lds[kBlock / kWave];
   const int k = h.k;
   if (k == 0) return;
-  const int64_t tile = b / k;
-  const int chunk = int(b - tile * k);
-  const int t = chunk * kBlock + threadIdx.x;  // padded pick inside the tile
-  const int r = t / k;
-  const int l = t - r * k;
-  const int64_t i = tile * kRowTile + r;
-  // the hop's length and this thread's own row and pick, requested together
+  const int groups = relabel_groups(k);
+  const int64_t tile = b / groups;
+  const int group = int(b - tile * groups);
+  // the hop's length and this thread's own rows and picks, requested together
   const int64_t s = seeds_of(h);
   if (!EARLY && tile * kRowTile >= s) return;
-  const bool mine = r < kRowTile && i < h.s_max;
-  // (hop 0's seed part is the caller's count, a kernel argument: p hangs on no load)
-  const int64_t p = h.pos_base + (h.index == 0 ? h.n_seeds_host : 0) + i * k + l;
-  uint32_t rc = 0, off = 0, word = 0, seed_word = 0;
-  if (mine) {
-    rc = h.row_cnt[i];
-    off = h.row_off[i];
-    word = h.slot[p];
-    if (h.index == 0) seed_word = h.slot[h.pos_base + i];
+  // (hop 0's seed part is the caller's count, a kernel argument: positions hang on no load)
+  const int64_t p0 = h.pos_base + (h.index == 0 ? h.n_seeds_host : 0);
+  int64_t i[kRelabelItems], p[kRelabelItems];
+  int l[kRelabelItems];
+  bool mine[kRelabelItems];
+  uint32_t rc[kRelabelItems], off[kRelabelItems], word[kRelabelItems], seed_word[kRelabelItems];
+#pragma unroll
+  for (int j = 0; j < kRelabelItems; ++j) {
+    const int chunk = group * kRelabelItems + j;
+    const int t = chunk * kBlock + threadIdx.x;  // padded pick inside the tile
+    const int r = t / k;
+    l[j] = t - r * k;
+    i[j] = tile * kRowTile + r;
+    p[j] = p0 + i[j] * k + l[j];
+    mine[j] = chunk < k && i[j] < h.s_max;
+    rc[j] = off[j] = word[j] = seed_word[j] = 0;
+    if (mine[j]) {
+      rc[j] = h.row_cnt[i[j]];
+      off[j] = h.row_off[i[j]];
+      word[j] = h.slot[p[j]];
+      if (h.index == 0) seed_word[j] = h.slot[h.pos_base + i[j]];
+    }
   }
   int64_t part = 0;
   if (h.tile_off) {
@@ -228,15 +242,34 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
     for (int64_t j = threadIdx.x; j < tile; j += kBlock) part += h.tile_sum[j];
   }
   if (tile * kRowTile >= s) return;  // whole blocks leave together
+  // Rank of a pick = rank recorded at the smallest position of its id: its own position when it
+  // is a first occurrence, else the position the table holds.  Two rounds of loads, each issued
+  // for all of the thread's picks before any is used, and both before the block adds up its
+  // prefix (whose barrier nothing here has to wait behind).
+  bool live[kRelabelItems];
+  uint32_t at[kRelabelItems];
+#pragma unroll
+  for (int j = 0; j < kRelabelItems; ++j) {
+    live[j] = mine[j] && i[j] < s && !is_bad_row(rc[j]) && uint32_t(l[j]) < rc[j];
+    at[j] = uint32_t(p[j]);
+    if (live[j] && !(word[j] & kFirstBit)) at[j] = table.value(word[j]);
+  }
+  uint32_t rank[kRelabelItems];
+#pragma unroll
+  for (int j = 0; j < kRelabelItems; ++j) rank[j] = live[j] ? h.rank_at[at[j]] : 0u;
   const int64_t prefix = block_sum<kBlock, int64_t>(part, lds);
-  if (!mine || i >= s || is_bad_row(rc) || uint32_t(l) >= rc) return;
-  const int64_t o = prefix + off + l;
-  static_cast<IdT*>(h.src_local)[o] = IdT(rank_of(h, table, p, word));
-  static_cast<IdT*>(h.dst_local)[o] = h.index == 0 ? IdT(rank_of(h, table, h.pos_base + i, seed_word)) : IdT(i);
+#pragma unroll
+  for (int j = 0; j < kRelabelItems; ++j) {
+    if (!live[j]) continue;
+    const int64_t o = prefix + off[j] + l[j];
+    static_cast<IdT*>(h.src_local)[o] = IdT(rank[j]);
+    static_cast<IdT*>(h.dst_local)[o] =
+        h.index == 0 ? IdT(rank_of(h, table, h.pos_base + i[j], seed_word[j])) : IdT(i[j]);
+  }
 }
 
 inline int64_t relabel_blocks(int64_t s_max, int k) {
-  return ((s_max + kRowTile - 1) / kRowTile) * k;
+  return ((s_max + kRowTile - 1) / kRowTile) * relabel_groups(k);
 }
 
 // ---- critical path ------------------------------------------------------------------------
