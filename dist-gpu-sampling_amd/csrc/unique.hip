@@ -112,8 +112,8 @@ __global__ __launch_bounds__(1024) void unique_scan_kernel(const int* __restrict
 
 template <typename IdT, typename TableT>
 __global__ __launch_bounds__(kThreads) void compact_kernel(dgs_segments mapping, int64_t n,
-                                                           const uint32_t* __restrict__ slot,
-                                                           const int* __restrict__ tile_off, TableT table,
+                                                           uint32_t* __restrict__ slot,
+                                                           const int* __restrict__ tile_off,
                                                            IdT* __restrict__ unique_out) {
   __shared__ int lds[kThreads / kWave];
   const int64_t base = int64_t(blockIdx.x) * kTileIds + threadIdx.x * kItems;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(dgs_segments mapping,
   for (int j = 0; j < kItems; ++j) {
     if (s[j] & kFirstBit) {
       unique_out[rank] = seg_load<IdT>(mapping, base + j);
-      table.set_value(s[j] & ~kFirstBit, uint32_t(rank));
+      slot[base + j] = uint32_t(rank) | kFirstBit;  // a first occurrence's word now holds its rank
       ++rank;
     }
   }
@@ -152,7 +152,10 @@ struct SegmentAlias {
   int64_t mapping_begin[DGS_MAX_SEGMENTS];
 };
 
-// out[j] = rank of requiring[j], -1 when the id is not in the table.
+// out[j] = rank of requiring[j], -1 when the id is not in the table.  Ranks live in the slot
+// words of the first occurrences (a streamed array), the table keeps every id's smallest
+// position: an element that is itself a first occurrence of the mapping list needs no random
+// read at all, any other one reads the table entry and then that position's word.
 template <typename IdT, typename TableT>
 __global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring, int64_t m, TableT table,
                                                           const uint32_t* __restrict__ slot, SegmentAlias alias,
@@ -163,13 +166,20 @@ __global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring
   int64_t off;
   seg_locate(requiring, j, &seg, &off);
   uint32_t s;
+  bool holds_rank = false;  // s is the word of a first occurrence of the mapping list
   if (alias.mapping_begin[seg] >= 0) {
-    s = slot[alias.mapping_begin[seg] + off] & ~kFirstBit;
+    s = slot[alias.mapping_begin[seg] + off];
+    holds_rank = (s & kFirstBit) != 0;
+    s &= ~kFirstBit;
   } else {
     const IdT key = static_cast<const IdT*>(requiring.ptr[seg])[off];
     s = table.holds(key) ? table.find(key) : table.mask + 1;  // an id the table cannot hold is not in it
   }
-  static_cast<IdT*>(const_cast<void*>(out.ptr[seg]))[off] = s > table.mask ? IdT(-1) : IdT(table.value(s));
+  IdT rank;
+  if (holds_rank) rank = IdT(s);
+  else if (s > table.mask) rank = IdT(-1);
+  else rank = IdT(slot[table.value(s)] & ~kFirstBit);
+  static_cast<IdT*>(const_cast<void*>(out.ptr[seg]))[off] = rank;
 }
 
 // ---- small inputs: one block, the table in LDS -----------------------------------------------
@@ -372,7 +382,7 @@ dgs_status run_unique_relabel(const dgs_segments& mapping, int64_t n, const dgs_
   }
   if (n > 0) {
     hipLaunchKernelGGL((compact_kernel<IdT, TableT>), dim3(uint32_t(tiles)), dim3(kThreads), 0, st, mapping, n,
-                       w.slot, w.tile_off, table, static_cast<IdT*>(unique_out));
+                       w.slot, w.tile_off, static_cast<IdT*>(unique_out));
     DGS_LAUNCH_CHECK();
   }
   if (m > 0) {
