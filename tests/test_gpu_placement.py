@@ -105,4 +105,14 @@ def test_loading_factor_runs(pkg):
         f = pkg.loading_factor.compute_loading_factor(ct, n, d, 4, option, 8000.0 if option == "local" else 64.0,
                                                       valid_time_threshold_ms=0.02, valid_needed=2, log=lines.append)
         assert f > 0.5 and np.isfinite(f)   # nothing moves faster than the stated bandwidth allows (with slack)
+        # the factor is the mean over the logged sizes of measured time / (rows x row bytes / bandwidth)
+        import re
+        mine = [l for l in lines if l.startswith(option)][-2:]
+        bw = 8000.0 if option == "local" else 64.0
+        ratios = []
+        for l in mine:
+            rows = int(re.search(r": (\d+) rows", l).group(1))
+            measured_ms = float(re.search(r"measured ([0-9.]+) ms", l).group(1))  # printed to 0.001 ms
+            ratios.append(measured_ms / (rows * d * 4 / 1e9 / bw * 1e3))
+        assert abs(f - sum(ratios) / len(ratios)) < 0.1 * f
     assert len(lines) == 4
