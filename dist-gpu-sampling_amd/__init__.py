@@ -35,8 +35,10 @@ from .sampler import (  # noqa: E402
     create_chunktensor,
     create_dgs_communicator,
     get_available_memory,
+    pipeline_streams,
     set_gather_buffer_cap,
     set_rng_state,
+    streams_overlap,
 )
 
 from . import placement  # noqa: E402
@@ -46,4 +48,4 @@ ChunkTensor = torch.classes.dgs_classes.ChunkTensor
 ops = torch.ops.dgs_ops
 
 __all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "create_chunktensor",
-           "create_dgs_communicator", "get_available_memory", "set_rng_state", "set_gather_buffer_cap", "HIP_LIB", "TORCH_LIB"]
+           "create_dgs_communicator", "get_available_memory", "set_rng_state", "set_gather_buffer_cap", "pipeline_streams", "streams_overlap", "HIP_LIB", "TORCH_LIB"]

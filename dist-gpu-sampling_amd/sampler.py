@@ -191,12 +191,51 @@ class ChunkTensorSampler:
 _pipeline_streams = []
 
 
+def streams_overlap(a, b, scratch=None):
+    """Whether work on stream `b` can run while stream `a` is busy.  HIP spreads a process's streams
+    over a few hardware queues (four by default), and two streams that land on the same queue run
+    their kernels in submission order however independent they are.  Measured, not looked up: a
+    long fill is enqueued on `a`, a tiny one on `b`, and the host watches which finishes when."""
+    import time
+    if scratch is None:
+        scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB: a fill of some 300 us
+    tiny = torch.empty(64, dtype=torch.float32, device="cuda")
+    done_a, done_b = torch.cuda.Event(), torch.cuda.Event()
+    votes = 0
+    for _ in range(3):
+        torch.cuda.synchronize()
+        with torch.cuda.stream(a):
+            scratch.fill_(1.0)
+            done_a.record()
+        with torch.cuda.stream(b):
+            tiny.fill_(1.0)
+            done_b.record()
+        t0 = time.perf_counter()
+        done_b.synchronize()
+        t1 = time.perf_counter()
+        done_a.synchronize()
+        t2 = time.perf_counter()
+        votes += (t1 - t0) < 0.5 * (t2 - t0)
+    return votes >= 2
+
+
 def pipeline_streams(n):
     """The first n of the streams that BatchPipeline objects run on by default.  They are shared by
     all pipelines of the process: a graph keeps one node table per stream that ever sampled from
-    it (at most four), so pipelines that come and go should not each bring new streams."""
-    while len(_pipeline_streams) < n:
-        _pipeline_streams.append(torch.cuda.Stream())
+    it (at most four), so pipelines that come and go should not each bring new streams.
+    A new stream joins only if it overlaps with every stream already chosen (streams_overlap):
+    in a process that has made other streams before, freshly made ones may share a hardware queue.
+    After a few candidates without luck the next one is taken as it is."""
+    if len(_pipeline_streams) < n:
+        scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda") if _pipeline_streams or n > 1 else None
+        rejected = []  # kept alive until the choice is made, so that new candidates are new streams
+        while len(_pipeline_streams) < n:
+            candidate = torch.cuda.Stream()
+            if len(rejected) < 6 and not all(streams_overlap(s, candidate, scratch) for s in _pipeline_streams):
+                rejected.append(candidate)
+                continue
+            _pipeline_streams.append(candidate)
+        del scratch
     return _pipeline_streams[:n]
 
 

@@ -685,3 +685,18 @@ def test_unique_relabel_ids_beyond_32_bits(pkg, oracle):
     requiring = [np.array([small[0], small[0] + 2 ** 32, -1], dtype=np.int64)]
     u, outs = pkg.capi.unique_relabel([_dev(p) for p in mapping], [_dev(p) for p in requiring])
     assert _np(outs[0]).tolist() == [0, -1, -1]
+
+
+def test_pipeline_streams_do_not_share_a_hardware_queue(pkg):
+    # a process that has made streams before (here: six of them) still gets pipeline streams that
+    # run side by side; streams that share a hardware queue would run their batches one after the other
+    others = [torch.cuda.Stream() for _ in range(6)]
+    chosen = pkg.pipeline_streams(3)
+    assert len(chosen) == 3 and len({s.cuda_stream for s in chosen}) == 3
+    assert pkg.pipeline_streams(2) == chosen[:2] and pkg.pipeline_streams(3) == chosen   # shared by all pipelines
+    for i in range(3):
+        for j in range(3):
+            if i != j:
+                assert pkg.streams_overlap(chosen[i], chosen[j])
+    assert not pkg.streams_overlap(chosen[0], chosen[0])  # one stream runs in order
+    del others
