@@ -299,8 +299,9 @@ def unique_relabel(mapping, requiring, packed_table=True):
 
 
 def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_seed, first_stream,
-                  feature_view=None, feature_row_elems=None, feature_dtype=None, node_table=None, epoch=0):
-    """All hops in one call.  Returns [(frontier, src_local, dst_local) per hop], the gathered
+                  feature_view=None, feature_row_elems=None, feature_dtype=None, node_table=None, epoch=0,
+                  probs_view=None):
+    """All hops in one call (picks by the edge weights `probs_view` when given).  Returns [(frontier, src_local, dst_local) per hop], the gathered
     rows of the last frontier when a feature view is given, and the per-hop error flags.
     `node_table` is an int64 device tensor of dgs_node_table_bytes(n_nodes) bytes filled with -1."""
     hops = len(hop_fanouts)
@@ -319,12 +320,20 @@ def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_se
         bufs.append((s, d))
         outs[h] = BlockOut(s.data_ptr(), d.data_ptr())
     sizes = torch.empty(3 * hops + 1, dtype=torch.int64, device=seeds.device)
-    nb = lib.dgs_sample_blocks_workspace_bytes(n, fan, hops, w)
-    ws = _ws(nb, seeds.device)
-    check(lib.dgs_sample_blocks(seeds.data_ptr(), w, n, indptr_view, indices_view, fan, hops, int(replace),
-                                rng_seed, first_stream, node_table.data_ptr() if node_table is not None else None,
-                                epoch, frontier.data_ptr(), outs, sizes.data_ptr(), None, None, ws.data_ptr(), nb,
-                                stream_ptr()))
+    table_ptr = node_table.data_ptr() if node_table is not None else None
+    if probs_view is None:
+        nb = lib.dgs_sample_blocks_workspace_bytes(n, fan, hops, w)
+        ws = _ws(nb, seeds.device)
+        check(lib.dgs_sample_blocks(seeds.data_ptr(), w, n, indptr_view, indices_view, fan, hops, int(replace),
+                                    rng_seed, first_stream, table_ptr, epoch, frontier.data_ptr(), outs,
+                                    sizes.data_ptr(), None, None, ws.data_ptr(), nb, stream_ptr()))
+    else:
+        nb = lib.dgs_sample_blocks_weighted_workspace_bytes(n, fan, hops, w)
+        ws = _ws(nb, seeds.device)
+        check(lib.dgs_sample_blocks_weighted(seeds.data_ptr(), w, n, indptr_view, indices_view, probs_view, fan, hops,
+                                             int(replace), rng_seed, first_stream, table_ptr, epoch,
+                                             frontier.data_ptr(), outs, sizes.data_ptr(), None, None, ws.data_ptr(),
+                                             nb, stream_ptr()))
     x = None
     if feature_view is not None:
         x = torch.empty((smax[hops], feature_row_elems), dtype=feature_dtype, device=seeds.device)

@@ -230,27 +230,22 @@ class ChunkTensor : public torch::CustomClassHolder {
   std::unique_lock<std::mutex> enqueue_lock() { return std::unique_lock<std::mutex>(node_table_mutex_); }
   // When every table belongs to another stream, the caller takes over the one used longest ago
   // among those whose stream has nothing left to run (a stream that is no longer used, such as
-  // one made per epoch).  If all of them are busy: with `must_have` the table used longest ago is
-  // taken after waiting for the device to go idle, without it the caller gets no table.
-  std::pair<void*, uint32_t> node_table(void* stream, bool must_have = false) {
+  // one made per epoch).  If all of them are busy the caller gets no table and its call builds a
+  // hash table in its workspace.
+  std::pair<void*, uint32_t> node_table(void* stream) {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
     if (bytes == 0 || bytes > (size_t(8) << 30)) return {nullptr, 0u};
     auto it = node_tables_.find(stream);
     if (it == node_tables_.end()) {
       if (node_tables_.size() >= kMaxNodeTables) {
-        auto pick = node_tables_.end(), oldest = node_tables_.begin();
+        auto pick = node_tables_.end();
         for (auto jt = node_tables_.begin(); jt != node_tables_.end(); ++jt) {
-          if (jt->second.last_use < oldest->second.last_use) oldest = jt;
           int32_t idle = 0;
           check(dgs_stream_query(jt->first, &idle));
           if (idle && (pick == node_tables_.end() || jt->second.last_use < pick->second.last_use)) pick = jt;
         }
-        if (pick == node_tables_.end()) {
-          if (!must_have) return {nullptr, 0u};
-          c10::hip::device_synchronize();
-          pick = oldest;
-        }
+        if (pick == node_tables_.end()) return {nullptr, 0u};
         NodeTable taken = std::move(pick->second);
         node_tables_.erase(pick);
         // the memory came from another stream's pool: it must not be handed out again while
@@ -657,9 +652,7 @@ class PendingBlocks : public torch::CustomClassHolder {
     torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
     // host threads that sample from the same graph enqueue their calls one at a time
     const std::unique_lock<std::mutex> one_call_at_a_time = indptr->enqueue_lock();
-    const auto table = indptr->node_table(st, /*must_have=*/static_cast<bool>(probs));
-    TORCH_CHECK(!probs || table.first != nullptr,
-                "weighted sample_blocks needs a node table (fewer than 2^31 nodes): use the per-hop operators here");
+    const auto table = indptr->node_table(st);
     // the caller's own (seed, first stream) when given, else the next `hops` streams of the
     // process-wide generator
     const auto rng = own_rng != nullptr ? *own_rng : next_rng(static_cast<uint32_t>(hops));

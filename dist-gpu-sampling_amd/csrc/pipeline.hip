@@ -834,12 +834,9 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
       clear_n16 = last > first ? (last - first) / 16 : 0;
     }
     if (p.weighted) {
-      // only instantiated for the direct table: the entry point refuses weighted calls without one
-      if constexpr (std::is_same_v<TableT, DirectTable<IdT>>) {
-        const dgs_status ws = replace ? launch_fill_weighted<IdT, PtrT, TableT, true>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st)
-                                      : launch_fill_weighted<IdT, PtrT, TableT, false>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st);
-        if (ws != DGS_OK) return ws;
-      }
+      const dgs_status ws = replace ? launch_fill_weighted<IdT, PtrT, TableT, true>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st)
+                                    : launch_fill_weighted<IdT, PtrT, TableT, false>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, *probs, rng_seed, st);
+      if (ws != DGS_OK) return ws;
     } else if (cur.k <= 8) launch_fill<IdT, PtrT, TableT, 8>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else if (cur.k <= 16) launch_fill<IdT, PtrT, TableT, 16>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
@@ -941,7 +938,10 @@ DGS_API size_t dgs_node_table_bytes(int64_t n_nodes) {
 DGS_API size_t dgs_sample_blocks_weighted_workspace_bytes(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops,
                                                           int32_t id_bytes) {
   dgs::Plan p;
-  if (dgs::make_plan(n_seeds, fanouts, n_hops, id_bytes, 1, true, &p) != DGS_OK) return 0;
+  // sized for the split hash table, the largest of the layouts (used when there is no node table)
+  if (dgs::make_plan(n_seeds, fanouts, n_hops, id_bytes, -1, false, &p) != DGS_OK) return 0;
+  p.kind = dgs::TableKind::kSplit;
+  p.table_bytes = size_t(p.capacity) * (size_t(id_bytes) + 4);
   p.weighted = true;
   return dgs::layout(p, fanouts, nullptr, nullptr, nullptr);
 }
@@ -959,7 +959,6 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
   dgs_status s = make_plan(n_seeds, fanouts, n_hops, id_bytes, indptr.total - 1, node_table != nullptr, &p);
   if (s != DGS_OK) return s;
   if (probs != nullptr) {
-    DGS_REQUIRE(node_table != nullptr, DGS_ERR_UNSUPPORTED, "sample_blocks_weighted: a node table is required");
     DGS_REQUIRE(probs->elem_bytes == 4 && probs->total == indices.total, DGS_ERR_INVALID,
                 "sample_blocks_weighted: %lld weights of %d bytes for %lld edges (float32, one per edge)",
                 (long long)probs->total, probs->elem_bytes, (long long)indices.total);

@@ -446,8 +446,8 @@ dgs_status dgs_sample_blocks(const void* seeds, int32_t id_bytes, int64_t n_seed
  * dgs_sample_neighbors_weighted (rng_stream = first_stream + h) and dgs_unique_relabel
  * per hop: the loop of ChunkTensorSampler.sample_blocks with chunk_probs
  * (oppo_bench/single_node/utils/chunktensor_sampler.py:93-118).  All other arguments are
- * those of dgs_sample_blocks, except that `node_table` is required (DGS_ERR_UNSUPPORTED
- * without one) and the workspace is sized by the _weighted_ query.
+ * those of dgs_sample_blocks (`node_table` optional, as there); the workspace is sized by
+ * the _weighted_ query.
  */
 size_t dgs_sample_blocks_weighted_workspace_bytes(int64_t n_seeds, const int64_t* fanouts,
                                                   int32_t n_hops, int32_t id_bytes);

@@ -288,8 +288,8 @@ def test_weighted_rows_that_the_key_halves_leave_open(pkg, oracle):
 
 
 def test_weighted_fused_on_more_streams_than_node_tables(pkg, oracle, graph):
-    # a graph keeps at most four node tables, one per stream; the weighted fused driver needs one,
-    # so a fifth and sixth stream take over the table that was used longest ago
+    # a graph keeps at most four node tables, one per stream; a fifth and sixth stream take over a
+    # table whose stream is idle, or run on a hash table in their workspace: same batches either way
     indptr, indices, probs = graph
     big = 1 << 40
     cts = [pkg.create_chunktensor(torch.from_numpy(a), 1, big) for a in (indptr, indices, probs)]
@@ -309,3 +309,36 @@ def test_weighted_fused_on_more_streams_than_node_tables(pkg, oracle, graph):
         for g, w in zip(blocks, want_blocks):
             assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("id_dtype", [np.int64, np.int32])
+def test_weighted_fused_c_abi_on_every_table_kind(pkg, oracle, graph, id_dtype):
+    # the weighted multi-hop driver through the C ABI: hash table in the workspace (packed slots,
+    # then id + value arrays), then the persistent node table; every hop picks by weight
+    capi = pkg.capi
+    indptr, indices, probs = graph
+    ix = indices.astype(id_dtype)
+    ip_t, ix_t, pr_t = _dev(indptr), _dev(ix), _dev(probs)
+    rng = np.random.default_rng(21)
+    seeds = rng.integers(0, 20000, size=700).astype(id_dtype)
+    n_nodes = indptr.size - 1
+    node_table = torch.full((capi.lib.dgs_node_table_bytes(n_nodes) // 8,), -1, dtype=torch.int64, device="cuda")
+    epoch = 0  # grows by one per call for as long as the table lives
+    for fanouts, replace in (([6, 4], False), ([9, 3], True)):
+        want_f, _, want_blocks = oracle.sample_blocks(seeds, indptr, ix, fanouts, replace, 77, 3, probs=probs)
+        hop_fanouts = list(reversed(fanouts))
+        for mode in ("packed", "split", "direct", "direct"):
+            capi.check(capi.lib.dgs_debug_set(capi.DEBUG_FORCE_SPLIT_TABLE, int(mode == "split")))
+            kw = {}
+            if mode == "direct":
+                epoch += 1
+                kw = dict(node_table=node_table, epoch=epoch)
+            try:
+                hops, _, flags = capi.sample_blocks(_dev(seeds), capi.tensor_view(ip_t), capi.tensor_view(ix_t),
+                                                    hop_fanouts, replace, 77, 3, probs_view=capi.tensor_view(pr_t), **kw)
+            finally:
+                capi.check(capi.lib.dgs_debug_set(capi.DEBUG_FORCE_SPLIT_TABLE, 0))
+            assert list(flags) == [0] * len(fanouts)
+            assert np.array_equal(_np(hops[-1][0]), want_f), mode
+            for (f, s, d), w in zip(hops, reversed(want_blocks)):
+                assert np.array_equal(_np(s), w[0]) and np.array_equal(_np(d), w[1]), mode
