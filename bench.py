@@ -513,7 +513,7 @@ def main():
     # stream, has seen every buffer size on every stream, and that the GPU has left its idle
     # clocks, before anything is timed (the W warm-up batches alone are fewer than two per stream
     # and over in a millisecond).
-    setup_batches = 64
+    setup_batches = 256
     run_batches(sampler, (batches * (1 + setup_batches // len(batches)))[:setup_batches], ct_feats, inflight, sizes)
     torch.cuda.synchronize()
     # the headline: `inflight` batches on the GPU at any time, seeds already in HBM, each batch
