@@ -527,6 +527,10 @@ def main():
     ms_handed_over = 1e3 * timed_steps(sampler, batches, inflight, True)[0] / args.steps if inflight > 1 else None
     # seeds as upstream's DataLoader passes them: pageable host tensors, uploaded by the operator
     ms_host_seeds = 1e3 * timed_steps(sampler, batches_cpu, inflight)[0] / args.steps
+    # both: host seeds in, every batch handed to the calling stream -- what upstream's training loop
+    # would see (its DataLoader passes host seeds, its model runs on the current stream)
+    ms_handed_over_host_seeds = (1e3 * timed_steps(sampler, batches_cpu, inflight, True)[0] / args.steps
+                                 if inflight > 1 else None)
     # what an unmodified upstream harness runs: per hop one sampling operator and one relabel
     # operator (each returns tensors of exact length, so each waits for its lengths), then _CAPI_index
     per_hop = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, ct_probs, replace=cfg["replace"],
@@ -607,11 +611,13 @@ def main():
         "ms_per_batch_alone": ms_latency,
         "ms_per_step_handed_over": ms_handed_over,
         "ms_per_step_host_seeds": ms_host_seeds,
+        "ms_per_step_handed_over_host_seeds": ms_handed_over_host_seeds,
         "ms_per_step_per_hop_ops": ms_per_hop_ops,
         "timings": {"ms_per_step_repeats": "the timed region run three more times (spread)",
                     "ms_per_batch_alone": "one batch at a time, one stream, call to result",
                     "ms_per_step_handed_over": "as the headline, each batch handed to the calling stream",
                     "ms_per_step_host_seeds": "as the headline, seeds passed as pageable host tensors",
+                    "ms_per_step_handed_over_host_seeds": "host seeds in, each batch handed to the calling stream",
                     "ms_per_step_per_hop_ops": "upstream's own loop: _CAPI_sample_neighbors_with_chunk_tensor + "
                                                "_CAPI_tensor_relabel per hop, then _CAPI_index, one batch at a time"},
         "sample_edges_per_s": stage_edges / args.steps / (ms_sample * 1e-3),

@@ -603,7 +603,8 @@ class PendingBlocks : public torch::CustomClassHolder {
                                                  const c10::intrusive_ptr<ChunkTensor>& features,
                                                  const c10::intrusive_ptr<ChunkTensor>& probs =
                                                      c10::intrusive_ptr<ChunkTensor>(),
-                                                 const std::pair<uint64_t, uint32_t>* own_rng = nullptr) {
+                                                 const std::pair<uint64_t, uint32_t>* own_rng = nullptr,
+                                                 void* gather_after = nullptr) {
     const int32_t w = id_width(seeds_in, "seeds");
     if (features) features->CheckErrors();
     if (probs) TORCH_CHECK(probs->dtype() == torch::kFloat32, "probs store must be float32, got ", probs->dtype());
@@ -681,6 +682,9 @@ class PendingBlocks : public torch::CustomClassHolder {
       p->stream_ = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap();
       p->x_rows_ = buffer_rows > 0 ? buffer_rows : -1;
       p->x_ = torch::empty({buffer_rows, features->elem_stride()}, xopt);
+      // the caller may hold the gather back until an event of another stream (the previous
+      // batch's gather, say), while the sampler kernels above run as soon as they can
+      if (gather_after != nullptr) check(dgs_ticket_stream_wait(st, gather_after));
       if (buffer_rows > 0)
         p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
                                                 buffer_rows, sizes_dev.data_ptr<int64_t>() + hops,
@@ -762,20 +766,22 @@ c10::intrusive_ptr<PendingBlocks> SampleBlocksWeightedBegin(torch::Tensor seeds,
 // rng_stream, rng_stream + 1, ... of seed rng_seed and the process-wide generator is left alone,
 // so a caller that keeps its own counter gets the same picks whatever other threads do.
 // The general form of the *_begin operators: `probs` and `features` are optional, `rng` is empty
-// (the process-wide generator) or [seed, first stream].
+// (the process-wide generator) or [seed, first stream]; `gather_after` is 0 or the handle of an
+// event (torch.cuda.Event.cuda_event) that the feature gather, and only it, waits for.
 c10::intrusive_ptr<PendingBlocks> SampleBlocksSubmit(torch::Tensor seeds, c10::intrusive_ptr<ChunkTensor> indptr,
                                                      c10::intrusive_ptr<ChunkTensor> indices,
                                                      c10::optional<c10::intrusive_ptr<ChunkTensor>> probs,
                                                      std::vector<int64_t> fanouts, bool replace,
                                                      c10::optional<c10::intrusive_ptr<ChunkTensor>> features,
-                                                     std::vector<int64_t> rng) {
+                                                     std::vector<int64_t> rng, int64_t gather_after) {
   TORCH_CHECK(rng.empty() || rng.size() == 2, "sample_blocks_submit: rng is [] or [seed, stream]");
   std::pair<uint64_t, uint32_t> own{0, 0};
   if (!rng.empty()) own = {static_cast<uint64_t>(rng[0]), static_cast<uint32_t>(rng[1])};
   return PendingBlocks::Begin(seeds, indptr, indices, fanouts, replace,
                               features.has_value() ? *features : c10::intrusive_ptr<ChunkTensor>(),
                               probs.has_value() ? *probs : c10::intrusive_ptr<ChunkTensor>(),
-                              rng.empty() ? nullptr : &own);
+                              rng.empty() ? nullptr : &own,
+                              reinterpret_cast<void*>(static_cast<intptr_t>(gather_after)));
 }
 
 // Largest worst-case feature buffer (bytes) the fused operators allocate ahead of the sizes.

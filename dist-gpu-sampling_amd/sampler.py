@@ -158,7 +158,7 @@ class ChunkTensorSampler:
             seeds = frontier
         return frontier, seed_nodes, blocks
 
-    def submit(self, g, seed_nodes, chunk_features=None, batch=None):
+    def submit(self, g, seed_nodes, chunk_features=None, batch=None, gather_after=None):
         """Enqueues a batch on the current stream and returns at once (fused path only).  Batches
         submitted on different streams overlap on the GPU: the short kernels of one batch's first
         hops fill the gaps between the large kernels of another.  Results come from
@@ -169,7 +169,7 @@ class ChunkTensorSampler:
         rng = [] if self.seed is None else [self.seed, self._first_stream(batch)]
         handle = torch.ops.dgs_ops._CAPI_sample_blocks_submit(
             seed_nodes, self.chunk_indptr, self.chunk_indices, self.chunk_probs, hop_fanouts, self.replace,
-            chunk_features, rng)
+            chunk_features, rng, 0 if gather_after is None else gather_after.cuda_event)
         return PendingBatch(handle, seed_nodes, chunk_features is not None, torch.cuda.current_stream())
 
     def sample_blocks_and_index(self, g, seed_nodes, chunk_features):
@@ -259,8 +259,10 @@ class BatchPipeline:
     four streams a process makes do.
     """
 
-    def __init__(self, sampler, chunk_features=None, inflight=3, streams=None, hand_over=True):
+    def __init__(self, sampler, chunk_features=None, inflight=3, streams=None, hand_over=True,
+                 gathers_in_turn=True):
         self.hand_over = hand_over
+        self.gathers_in_turn = gathers_in_turn
         if inflight < 1:
             raise ValueError("inflight must be at least 1")
         self.sampler = sampler
@@ -268,12 +270,13 @@ class BatchPipeline:
         self.streams = list(streams) if streams is not None else pipeline_streams(inflight)
         if not self.streams:
             raise ValueError("no streams to run on")
+        self._event_sets = []
 
-    def _hand_out(self, pending, consumer):
+    def _hand_out(self, pending, done, consumer):
         out = pending.result()
         if not self.hand_over:
             return out
-        consumer.wait_stream(pending.stream)
+        consumer.wait_event(done)  # recorded behind the batch's last kernel when it was submitted
         tensors = [out[0]]
         for b in out[2]:
             tensors += [b.src_local, b.dst_local]
@@ -288,19 +291,37 @@ class BatchPipeline:
 
     def __call__(self, seed_batches):
         consumer = torch.cuda.current_stream()
+        n = len(self.streams)
+        # Events are made once per pipeline and reused (making one costs more than the stream wait
+        # it serves).  A wait refers to the record that precedes it, so reuse by later batches is
+        # safe; an iteration takes a set of its own, so two iterations of one pipeline do not mix.
+        events = self._event_sets.pop() if self._event_sets else (
+            [torch.cuda.Event() for _ in range(n)], [torch.cuda.Event() for _ in range(n)])
+        seeds_ready, batch_done = events
         queue = deque()
-        for i, seeds in enumerate(seed_batches):
-            st = self.streams[i % len(self.streams)]
-            # Seeds on the device may have been made just now on the caller's stream (a generator
-            # that builds them lazily, or uploads them without blocking): the batch's stream waits
-            # for that stream as it stands.  This also orders the batch behind everything else the
-            # caller has enqueued there, so seeds that should overlap with the caller's work are
-            # better passed as host tensors (the operator uploads them on the batch's own stream).
-            if i < len(self.streams) or (torch.is_tensor(seeds) and seeds.is_cuda):
-                st.wait_stream(consumer)
-            with torch.cuda.stream(st):
-                queue.append(self.sampler.submit(None, seeds, self.chunk_features))
-            if len(queue) >= len(self.streams):
-                yield self._hand_out(queue.popleft(), consumer)
-        while queue:
-            yield self._hand_out(queue.popleft(), consumer)
+        try:
+            for i, seeds in enumerate(seed_batches):
+                st = self.streams[i % n]
+                # Seeds on the device may have been made just now on the caller's stream (a generator
+                # that builds them lazily, or uploads them without blocking): the batch's stream waits
+                # for that stream as it stands.  This also orders the batch behind everything else the
+                # caller has enqueued there, so seeds that should overlap with the caller's work are
+                # better passed as host tensors (the operator uploads them on the batch's own stream).
+                # (nothing to wait for when the caller's stream has drained: a query costs a tenth
+                # of what the event pair costs)
+                if (i < n or (torch.is_tensor(seeds) and seeds.is_cuda)) and not consumer.query():
+                    seeds_ready[i % n].record(consumer)
+                    st.wait_event(seeds_ready[i % n])
+                turn = self.gathers_in_turn and self.chunk_features is not None and n > 1
+                with torch.cuda.stream(st):
+                    pending = self.sampler.submit(None, seeds, self.chunk_features,
+                                                  gather_after=batch_done[(i - 1) % n] if turn and i > 0 else None)
+                    if self.hand_over or turn:
+                        batch_done[i % n].record(st)
+                queue.append((pending, batch_done[i % n]))
+                if len(queue) >= n:
+                    yield self._hand_out(*queue.popleft(), consumer)
+            while queue:
+                yield self._hand_out(*queue.popleft(), consumer)
+        finally:
+            self._event_sets.append(events)
