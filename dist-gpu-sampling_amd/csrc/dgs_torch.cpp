@@ -29,6 +29,10 @@
 #include <torch/script.h>
 
 #include <atomic>
+#include <condition_variable>
+#include <deque>
+#include <string>
+#include <thread>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -626,6 +630,7 @@ class PendingBlocks : public torch::CustomClassHolder {
 
     auto p = c10::make_intrusive<PendingBlocks>();
     p->hops_ = hops;
+    p->stream_ = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap();
     // the kernels mirror the lengths into this call's own pinned words
     p->pinned_ = torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
     if (seeds_in.device().is_cpu() && !seeds_in.is_pinned() && n > 0) {
@@ -679,7 +684,6 @@ class PendingBlocks : public torch::CustomClassHolder {
       if (buffer_rows * row_bytes > g_gather_buffer_cap.load()) buffer_rows = g_gather_buffer_cap.load() / row_bytes;
       p->features_ = features;
       p->width_ = w;
-      p->stream_ = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap();
       p->x_rows_ = buffer_rows > 0 ? buffer_rows : -1;
       p->x_ = torch::empty({buffer_rows, features->elem_stride()}, xopt);
       // the caller may hold the gather back until an event of another stream (the previous
@@ -691,6 +695,17 @@ class PendingBlocks : public torch::CustomClassHolder {
                                                 p->x_.data_ptr(), DGS_TIER_ANY, features->bad_index_word(), st);
     }
     return p;
+  }
+
+  // The stream the batch was begun on, and a way to mark the batch's buffers as used on another
+  // stream (so that the allocator does not hand them out again while that stream still reads them).
+  c10::Stream stream() const { return stream_; }
+  void RecordStream(const c10::Stream& consumer) {
+    for (const torch::Tensor* t : {&seeds_, &all_, &x_})
+      if (t->defined() && t->is_cuda()) t->record_stream(consumer);
+    for (const auto& list : {&src_, &dst_})
+      for (const torch::Tensor& t : *list)
+        if (t.defined() && t.is_cuda()) t.record_stream(consumer);
   }
 
  private:
@@ -707,6 +722,182 @@ class PendingBlocks : public torch::CustomClassHolder {
   int64_t x_rows_ = -1;
   int32_t width_ = 0;
   c10::Stream stream_ = c10::Stream(c10::Stream::DEFAULT, c10::Device(c10::DeviceType::CPU, -1));
+};
+
+// Batches in flight without a Python step per enqueue: a worker thread begins batches
+// (PendingBlocks::Begin: some hundred microseconds of host work each, most of it kernel launches)
+// on the loop's streams in turn while the caller's thread takes delivery of finished ones.
+// Push hands seeds to the worker, Pop returns the oldest batch not yet returned, in order.
+// At most `streams.size()` batches are begun and not yet popped.
+class BatchLoop : public torch::CustomClassHolder {
+ public:
+  BatchLoop(c10::intrusive_ptr<ChunkTensor> indptr, c10::intrusive_ptr<ChunkTensor> indices,
+            c10::optional<c10::intrusive_ptr<ChunkTensor>> probs, std::vector<int64_t> fanouts, bool replace,
+            c10::optional<c10::intrusive_ptr<ChunkTensor>> features, std::vector<int64_t> streams, bool hand_over,
+            bool gathers_in_turn, std::vector<int64_t> rng)
+      : indptr_(std::move(indptr)), indices_(std::move(indices)),
+        probs_(probs.has_value() ? *probs : c10::intrusive_ptr<ChunkTensor>()), fanouts_(std::move(fanouts)),
+        replace_(replace), features_(features.has_value() ? *features : c10::intrusive_ptr<ChunkTensor>()),
+        hand_over_(hand_over), turn_(gathers_in_turn), rng_(std::move(rng)) {
+    TORCH_CHECK(!streams.empty() && streams.size() % 3 == 0,
+                "BatchLoop: streams are (stream_id, device_index, device_type) triples");
+    TORCH_CHECK(rng_.empty() || rng_.size() == 2, "BatchLoop: rng is [] or [seed, first stream]");
+    for (size_t i = 0; i < streams.size(); i += 3)
+      streams_.push_back(c10::Stream::unpack3(streams[i], static_cast<c10::DeviceIndex>(streams[i + 1]),
+                                               static_cast<c10::DeviceType>(streams[i + 2])));
+    done_.assign(streams_.size() + 1, nullptr);
+    worker_ = std::thread([this] { Work(); });
+  }
+  ~BatchLoop() override { Close(); }
+
+  // Seeds on the device are ordered behind what the calling thread's current stream holds at this
+  // moment (they may have been made there just now); host seeds need nothing, unless the caller
+  // asks for the same order (behind_caller: the first batches of an iteration, say, behind the
+  // set-up that precedes it).
+  void Push(torch::Tensor seeds, bool behind_caller) {
+    Item item;
+    item.seeds = std::move(seeds);
+    if (item.seeds.is_cuda() || behind_caller) {
+      void* st = current_stream();
+      int32_t idle = 0;
+      check(dgs_stream_query(st, &idle));
+      if (!idle) check(dgs_ticket_record(st, &item.seeds_ready));
+    }
+    {
+      const std::lock_guard<std::mutex> lock(mutex_);
+      TORCH_CHECK(!stop_, "BatchLoop: closed");
+      input_.push_back(std::move(item));
+      ++pushed_;
+    }
+    wake_worker_.notify_one();
+  }
+
+  BlocksResult Pop() {
+    Item item;
+    {
+      std::unique_lock<std::mutex> lock(mutex_);
+      TORCH_CHECK(popped_ < pushed_, "BatchLoop: nothing to pop");
+      wake_caller_.wait(lock, [this] { return !output_.empty(); });
+      item = std::move(output_.front());
+      output_.pop_front();
+      ++popped_;
+    }
+    wake_worker_.notify_one();  // a slot is free
+    TORCH_CHECK(item.error.empty(), item.error);
+    BlocksResult result = item.batch->Finish();
+    if (hand_over_) {
+      // the calling thread's stream waits for everything the batch has enqueued (Finish may just have
+      // added a gather), and the batch's buffers are marked as used there
+      void* ticket = nullptr;
+      check(dgs_ticket_record(stream_handle(item.batch->stream()), &ticket));
+      const dgs_status ws = dgs_ticket_stream_wait(current_stream(), ticket);
+      dgs_ticket_release(ticket);
+      check(ws);
+      item.batch->RecordStream(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap());
+    }
+    return result;
+  }
+
+  int64_t Pending() {
+    const std::lock_guard<std::mutex> lock(mutex_);
+    return pushed_ - popped_;
+  }
+
+  void Close() {
+    {
+      const std::lock_guard<std::mutex> lock(mutex_);
+      if (stop_) return;
+      stop_ = true;
+    }
+    wake_worker_.notify_all();
+    if (worker_.joinable()) worker_.join();
+    for (Item& item : input_)
+      if (item.seeds_ready) dgs_ticket_release(item.seeds_ready);
+    input_.clear();
+    output_.clear();  // batches nobody asked for: their destructors wait for their kernels' lengths
+    for (void*& t : done_) {
+      if (t) dgs_ticket_release(t);
+      t = nullptr;
+    }
+  }
+
+ private:
+  struct Item {
+    torch::Tensor seeds;
+    void* seeds_ready = nullptr;  // ticket on the pushing thread's stream, or null
+    c10::intrusive_ptr<PendingBlocks> batch;
+    std::string error;
+  };
+
+  static void* stream_handle(const c10::Stream& s) {
+    return c10::hip::HIPStreamMasqueradingAsCUDA(s).stream();
+  }
+
+  void Work() {
+    int64_t index = 0;
+    const int64_t n = static_cast<int64_t>(streams_.size());
+    for (;;) {
+      Item item;
+      {
+        std::unique_lock<std::mutex> lock(mutex_);
+        wake_worker_.wait(lock, [&] { return stop_ || (!input_.empty() && begun_ - popped_ < n); });
+        if (stop_) return;
+        item = std::move(input_.front());
+        input_.pop_front();
+        ++begun_;
+      }
+      try {
+        const c10::Stream st = streams_[index % n];
+        const c10::StreamGuard on_stream(st);  // allocations and launches of this batch go to its stream
+        void* raw = current_stream();
+        if (item.seeds_ready) {
+          const dgs_status ws = dgs_ticket_stream_wait(raw, item.seeds_ready);
+          dgs_ticket_release(item.seeds_ready);
+          item.seeds_ready = nullptr;
+          check(ws);
+        }
+        const bool turn = turn_ && features_ && n > 1;
+        void* gather_after = turn && index > 0 ? done_[(index - 1) % (n + 1)] : nullptr;
+        std::pair<uint64_t, uint32_t> own{0, 0};
+        if (!rng_.empty())
+          own = {static_cast<uint64_t>(rng_[0]),
+                 static_cast<uint32_t>(rng_[1] + index * static_cast<int64_t>(fanouts_.size()))};
+        item.batch = PendingBlocks::Begin(item.seeds, indptr_, indices_, fanouts_, replace_, features_, probs_,
+                                          rng_.empty() ? nullptr : &own, gather_after);
+        if (turn) {
+          // the slot's old ticket belongs to a batch that was popped long ago (at most n are in flight)
+          void*& slot = done_[index % (n + 1)];
+          if (slot) dgs_ticket_release(slot);
+          slot = nullptr;
+          check(dgs_ticket_record(raw, &slot));
+        }
+      } catch (const std::exception& err) {
+        item.error = err.what();
+      }
+      item.seeds = torch::Tensor();
+      ++index;
+      {
+        const std::lock_guard<std::mutex> lock(mutex_);
+        output_.push_back(std::move(item));
+      }
+      wake_caller_.notify_one();
+    }
+  }
+
+  c10::intrusive_ptr<ChunkTensor> indptr_, indices_, probs_;
+  std::vector<int64_t> fanouts_;
+  bool replace_;
+  c10::intrusive_ptr<ChunkTensor> features_;
+  std::vector<c10::Stream> streams_;
+  bool hand_over_, turn_;
+  std::vector<int64_t> rng_;
+  std::vector<void*> done_;  // ring of tickets behind the last batches' last launches (worker thread only)
+  std::mutex mutex_;
+  std::condition_variable wake_worker_, wake_caller_;
+  std::deque<Item> input_, output_;
+  int64_t pushed_ = 0, begun_ = 0, popped_ = 0;
+  bool stop_ = false;
+  std::thread worker_;
 };
 
 namespace {
@@ -832,6 +1023,16 @@ TORCH_LIBRARY(dgs_classes, m) {
       .def("_CAPI_synchronize_and_check", &ChunkTensor::SynchronizeAndCheck);
   // not in upstream: a sample_blocks call in flight
   m.class_<PendingBlocks>("PendingBlocks").def("_CAPI_finish", &PendingBlocks::Finish);
+  // not in upstream: batches in flight, begun by a worker thread of the extension
+  m.class_<dgs::BatchLoop>("BatchLoop")
+      .def(torch::init<c10::intrusive_ptr<ChunkTensor>, c10::intrusive_ptr<ChunkTensor>,
+                       c10::optional<c10::intrusive_ptr<ChunkTensor>>, std::vector<int64_t>, bool,
+                       c10::optional<c10::intrusive_ptr<ChunkTensor>>, std::vector<int64_t>, bool, bool,
+                       std::vector<int64_t>>())
+      .def("_CAPI_push", &dgs::BatchLoop::Push)
+      .def("_CAPI_pop", &dgs::BatchLoop::Pop)
+      .def("_CAPI_pending", &dgs::BatchLoop::Pending)
+      .def("_CAPI_close", &dgs::BatchLoop::Close);
 }
 
 TORCH_LIBRARY(dgs_ops, m) {

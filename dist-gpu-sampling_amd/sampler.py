@@ -189,6 +189,7 @@ class ChunkTensorSampler:
 
 
 _pipeline_streams = []
+_event_sets = {}  # streams of a pipeline -> spare (seeds ready, batch done) event lists
 
 
 def streams_overlap(a, b, scratch=None):
@@ -260,9 +261,12 @@ class BatchPipeline:
     """
 
     def __init__(self, sampler, chunk_features=None, inflight=3, streams=None, hand_over=True,
-                 gathers_in_turn=True):
+                 gathers_in_turn=True, native_loop=True):
         self.hand_over = hand_over
         self.gathers_in_turn = gathers_in_turn
+        self.native_loop = native_loop
+        self._loop = None
+        self._loop_busy = False
         if inflight < 1:
             raise ValueError("inflight must be at least 1")
         self.sampler = sampler
@@ -270,13 +274,15 @@ class BatchPipeline:
         self.streams = list(streams) if streams is not None else pipeline_streams(inflight)
         if not self.streams:
             raise ValueError("no streams to run on")
-        self._event_sets = []
 
     def _hand_out(self, pending, done, consumer):
         out = pending.result()
         if not self.hand_over:
             return out
-        consumer.wait_event(done)  # recorded behind the batch's last kernel when it was submitted
+        # behind everything the batch has enqueued on its stream, including a gather that result()
+        # may just have launched for a frontier that did not fit its capped buffer
+        done.record(pending.stream)
+        consumer.wait_event(done)
         tensors = [out[0]]
         for b in out[2]:
             tensors += [b.src_local, b.dst_local]
@@ -289,13 +295,67 @@ class BatchPipeline:
                 t.record_stream(consumer)
         return out
 
+    def _native(self):
+        """The extension's own loop for this pipeline (made once): a worker thread of the extension
+        begins the batches, so that Python pays one call to hand seeds in and one to take a batch out."""
+        if self._loop is None:
+            smp = self.sampler
+            triples = []
+            for st in self.streams:
+                triples += [st.stream_id, st.device_index, st.device_type]
+            self._loop = torch.classes.dgs_classes.BatchLoop(
+                smp.chunk_indptr, smp.chunk_indices, smp.chunk_probs, list(reversed(smp.fanouts)), smp.replace,
+                self.chunk_features, triples, self.hand_over, self.gathers_in_turn, [])
+        return self._loop
+
+    def _iterate_native(self, seed_batches):
+        loop = self._native()
+        n = len(self.streams)
+        with_x = self.chunk_features is not None
+        waiting = deque()
+        pushed = 0
+
+        def take():
+            frontiers, srcs, dsts, x, seeds_dev = loop._CAPI_pop()
+            blocks = ChunkTensorSampler._blocks(seeds_dev, frontiers, srcs, dsts)
+            seed_nodes = waiting.popleft()
+            return (frontiers[-1], seed_nodes, blocks, x) if with_x else (frontiers[-1], seed_nodes, blocks)
+
+        self._loop_busy = True
+        try:
+            for seeds in seed_batches:
+                # the first batch on each stream goes behind what the caller's stream holds now,
+                # later ones only if their seeds are on the device (see the Python loop below)
+                loop._CAPI_push(seeds, pushed < n)
+                pushed += 1
+                waiting.append(seeds)
+                if len(waiting) >= n:
+                    yield take()
+            while waiting:
+                yield take()
+        finally:
+            while loop._CAPI_pending() > 0:  # an iteration that was left early: nothing stays behind in the loop
+                try:
+                    loop._CAPI_pop()
+                except RuntimeError:
+                    pass
+            self._loop_busy = False
+
     def __call__(self, seed_batches):
+        # (a sampler with its own generator counts its batches in Python, and a second iteration
+        # that starts while one is under way cannot share the first one's queue: both keep the
+        # Python loop)
+        if self.native_loop and self.sampler.fused and self.sampler.seed is None and not self._loop_busy:
+            yield from self._iterate_native(seed_batches)
+            return
         consumer = torch.cuda.current_stream()
         n = len(self.streams)
-        # Events are made once per pipeline and reused (making one costs more than the stream wait
-        # it serves).  A wait refers to the record that precedes it, so reuse by later batches is
-        # safe; an iteration takes a set of its own, so two iterations of one pipeline do not mix.
-        events = self._event_sets.pop() if self._event_sets else (
+        # Events are made once per process and reused (making one costs more than the stream wait
+        # it serves, and a fresh set per iteration showed in short iterations).  A wait refers to
+        # the record that precedes it, so reuse by later batches is safe; an iteration takes a
+        # set of its own, so iterations that overlap do not mix.
+        spare = _event_sets.setdefault(n, [])
+        events = spare.pop() if spare else (
             [torch.cuda.Event() for _ in range(n)], [torch.cuda.Event() for _ in range(n)])
         seeds_ready, batch_done = events
         queue = deque()
@@ -324,4 +384,4 @@ class BatchPipeline:
             while queue:
                 yield self._hand_out(*queue.popleft(), consumer)
         finally:
-            self._event_sets.append(events)
+            spare.append(events)

@@ -593,10 +593,12 @@ def test_host_threads_sampling_from_one_graph_on_one_stream(pkg, oracle):
             assert np.array_equal(_np(gb.src_local), wb[0]) and np.array_equal(_np(gb.dst_local), wb[1])
 
 
-def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph):
+@pytest.mark.parametrize("native_loop", [True, False])
+def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph, native_loop):
     # BatchPipeline: batches in flight on its own streams, results in submission order, usable on
     # the caller's stream at once (reduced there right away, buffers dropped while later batches
-    # are still running), host and device seeds, uniform and weighted samplers
+    # are still running), host and device seeds, uniform and weighted samplers; with the
+    # extension's worker thread beginning the batches, and with the Python loop
     indptr, indices = graph
     big = 1 << 40
     rng = np.random.default_rng(8)
@@ -610,9 +612,17 @@ def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph):
     batches = [rng.integers(0, 20000, size=900).astype(np.int64) for _ in range(11)]
     for weights, inflight in ((None, 2), (None, 3), (pr_ct, 2), (None, 1)):
         sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, weights)
-        pipe = pkg.BatchPipeline(sampler, x_ct, inflight)
-        pkg.set_rng_state(99, 7)
+        pipe = pkg.BatchPipeline(sampler, x_ct, inflight, native_loop=native_loop)
         feeds = [torch.from_numpy(b) if i % 2 else _dev(b) for i, b in enumerate(batches)]
+        # an iteration that is left early leaves nothing behind, and one that starts inside another
+        # gets its own batches
+        for i, out in enumerate(pipe(feeds)):
+            if i == 0:
+                inner = [o[0].clone() for o in pipe(feeds[:3])]
+                assert len(inner) == 3
+            if i == 1:
+                break
+        pkg.set_rng_state(99, 7)
         sums, kept = [], []
         for i, (f, seeds, blocks, x) in enumerate(pipe(feeds)):
             sums.append(x.double().sum(dim=0))           # on the caller's stream, no extra wait
@@ -631,7 +641,8 @@ def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph):
     with pytest.raises(ValueError):
         pkg.BatchPipeline(sampler, x_ct, 0)
     with pytest.raises(RuntimeError):
-        list(pkg.BatchPipeline(pkg.ChunkTensorSampler([100], ip_ct, ix_ct), x_ct)([_dev(batches[0])]))
+        list(pkg.BatchPipeline(pkg.ChunkTensorSampler([100], ip_ct, ix_ct), x_ct,
+                               native_loop=native_loop)([_dev(batches[0])]))
 
 
 @pytest.mark.parametrize("cap", [1, 7, 300])
