@@ -230,10 +230,19 @@ def run_batches(sampler, seed_batches, features, inflight, consume=lambda r: Non
     are dropped at once so the allocator can hand them to the next batch).  The caller brackets
     the call with synchronisations.  Nothing here touches a batch on another stream than its own,
     so by default the pipeline does not hand batches over to the calling stream."""
+    if features is None:  # sampling + relabel only
+        return [consume(sampler.sample_blocks(None, b)) for b in seed_batches]
     if inflight <= 1 or not sampler.fused:
         return [consume(sampler.sample_blocks_and_index(None, b, features)) for b in seed_batches]
-    pipeline = sys.modules[type(sampler).__module__].BatchPipeline(sampler, features, inflight, hand_over=hand_over)
-    return [consume(r) for r in pipeline(seed_batches)]
+    # (a pipeline is made once and iterated many times, as a training loop would per epoch)
+    key = (id(sampler), id(features), inflight, hand_over)
+    if key not in _pipelines:
+        _pipelines[key] = (sys.modules[type(sampler).__module__].BatchPipeline(sampler, features, inflight,
+                                                                              hand_over=hand_over), sampler, features)
+    return [consume(r) for r in _pipelines[key][0](seed_batches)]
+
+
+_pipelines = {}
 
 
 def table_access_rates(dgs, slots, n_ops, reps=50):
@@ -500,12 +509,12 @@ def main():
         return {"frontier": r[0].numel(),
                 "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]}
 
-    def timed_steps(smp, seed_batches, n_inflight, hand_over=False):
+    def timed_steps(smp, seed_batches, n_inflight, hand_over=False, features=ct_feats):
         """W untimed warm-up batches, then exactly K batches between two synchronisations."""
-        run_batches(smp, seed_batches[:args.warmup], ct_feats, n_inflight, sizes, hand_over)
+        run_batches(smp, seed_batches[:args.warmup], features, n_inflight, sizes, hand_over)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        res = run_batches(smp, seed_batches[args.warmup:], ct_feats, n_inflight, sizes, hand_over)
+        res = run_batches(smp, seed_batches[args.warmup:], features, n_inflight, sizes, hand_over)
         torch.cuda.synchronize()
         return time.perf_counter() - t0, res
 
@@ -536,6 +545,8 @@ def main():
     per_hop = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, ct_probs, replace=cfg["replace"],
                                      fused=False)
     ms_per_hop_ops = 1e3 * timed_steps(per_hop, batches, 1)[0] / args.steps
+    # the same loop without its last line: the sampling and relabel operators alone
+    ms_per_hop_ops_no_gather = 1e3 * timed_steps(per_hop, batches, 1, features=None)[0] / args.steps
 
     # Stage split and the dominant kernel's duration, on the same batches: events on torch's
     # current stream (the one the C ABI launches on) around the sampler call and around the
@@ -613,13 +624,15 @@ def main():
         "ms_per_step_host_seeds": ms_host_seeds,
         "ms_per_step_handed_over_host_seeds": ms_handed_over_host_seeds,
         "ms_per_step_per_hop_ops": ms_per_hop_ops,
+        "ms_per_step_per_hop_ops_no_gather": ms_per_hop_ops_no_gather,
         "timings": {"ms_per_step_repeats": "the timed region run three more times (spread)",
                     "ms_per_batch_alone": "one batch at a time, one stream, call to result",
                     "ms_per_step_handed_over": "as the headline, each batch handed to the calling stream",
                     "ms_per_step_host_seeds": "as the headline, seeds passed as pageable host tensors",
                     "ms_per_step_handed_over_host_seeds": "host seeds in, each batch handed to the calling stream",
                     "ms_per_step_per_hop_ops": "upstream's own loop: _CAPI_sample_neighbors_with_chunk_tensor + "
-                                               "_CAPI_tensor_relabel per hop, then _CAPI_index, one batch at a time"},
+                                               "_CAPI_tensor_relabel per hop, then _CAPI_index, one batch at a time",
+                    "ms_per_step_per_hop_ops_no_gather": "that loop without _CAPI_index: the six operator calls alone"},
         "sample_edges_per_s": stage_edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
         "ms_sample_relabel": ms_sample,

@@ -91,6 +91,8 @@ SIGNATURES = {
     "dgs_ticket_record": (ctypes.c_int, [c_vp, ctypes.POINTER(c_vp)]),
     "dgs_ticket_stream_wait": (ctypes.c_int, [c_vp, c_vp]),
     "dgs_ticket_wait": (ctypes.c_int, [c_vp]),
+    "dgs_ticket_wait_words": (ctypes.c_int, [c_vp, c_vp, c_i32]),
+    "dgs_stream_wait_words": (ctypes.c_int, [c_vp, c_vp, c_i32]),
     "dgs_ticket_release": (ctypes.c_int, [c_vp]),
     "dgs_stream_query": (ctypes.c_int, [c_vp, ctypes.POINTER(c_i32)]),
 }
@@ -209,9 +211,19 @@ def sample_neighbors(seeds, indptr_view, indices_view, num_picks, replace, rng_s
     nnz = torch.empty(2, dtype=torch.int64, device=seeds.device)
     w = seeds.element_size()
     if two_step:
-        check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
-                                   None, ws.data_ptr(), nb, stream_ptr()))
-        cnt, flags = read_i64(nnz, 2)
+        if two_step == "mirrored":
+            # the lengths through pinned words that the count kernel writes and the host polls
+            pinned = torch.full((2,), -1, dtype=torch.int64).pin_memory()
+            check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
+                                       pinned.data_ptr(), ws.data_ptr(), nb, stream_ptr()))
+            ticket = ctypes.c_void_p()
+            check(lib.dgs_ticket_record(stream_ptr(), ctypes.byref(ticket)))
+            check(lib.dgs_ticket_wait_words(ticket, pinned.data_ptr(), 2))
+            cnt, flags = pinned.tolist()
+        else:
+            check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace),
+                                       nnz.data_ptr(), None, ws.data_ptr(), nb, stream_ptr()))
+            cnt, flags = read_i64(nnz, 2)
         rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
         cols = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
         check(lib.dgs_sample_fill(seeds.data_ptr(), w, n, indices_view, num_picks, int(replace), rng_seed,
@@ -277,9 +289,10 @@ def renumber_csc(indptr, indices, order, rank, new_indptr):
     return out
 
 
-def unique_relabel(mapping, requiring, packed_table=True):
+def unique_relabel(mapping, requiring, packed_table=True, polled=False):
     """Returns (unique, [relabelled ...]).  With `packed_table` 8-byte ids are tried in the one-word
-    slots first and the call is repeated with the two-array table if an id does not fit."""
+    slots first and the call is repeated with the two-array table if an id does not fit.
+    With `polled` the counts come through pinned words that the host polls instead of a copy."""
     dev = mapping[0].device
     dt = mapping[0].dtype
     n = sum(t.numel() for t in mapping)
@@ -290,9 +303,17 @@ def unique_relabel(mapping, requiring, packed_table=True):
     nb = lib.dgs_unique_relabel_workspace_bytes(n, w)
     ws = _ws(nb, dev)
     for packed in ((1, 0) if packed_table else (0,)):
-        check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, packed, unique.data_ptr(),
-                                     num.data_ptr(), None, None, segments(outs), ws.data_ptr(), nb, stream_ptr()))
-        u, overflow = read_i64(num, 2)
+        if polled:
+            pinned = torch.full((2,), -1, dtype=torch.int64).pin_memory()
+            check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, packed, unique.data_ptr(),
+                                         num.data_ptr(), pinned.data_ptr(), None, segments(outs), ws.data_ptr(), nb,
+                                         stream_ptr()))
+            check(lib.dgs_stream_wait_words(stream_ptr(), pinned.data_ptr(), 2))
+            u, overflow = pinned.tolist()
+        else:
+            check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, packed, unique.data_ptr(),
+                                         num.data_ptr(), None, None, segments(outs), ws.data_ptr(), nb, stream_ptr()))
+            u, overflow = read_i64(num, 2)
         if not overflow:
             break
     return unique[:u], outs

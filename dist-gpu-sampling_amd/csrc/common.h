@@ -129,6 +129,14 @@ __device__ __forceinline__ void single_block_scan(const TIn* __restrict__ in, TO
   if (threadIdx.x == 0) *sum = carry;
 }
 
+// A length word mirrored into pinned host memory: stored at system scope, so that it leaves the
+// GPU's caches at once and a host thread that polls the word (dgs_ticket_wait_words) sees it
+// while the kernel is still running.  Every word stands for itself: no order among them is
+// promised, and a reader takes each one when it has turned non-negative.
+__device__ __forceinline__ void mirror_to_host(int64_t* word, int64_t v) {
+  __hip_atomic_store(word, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 template <typename T>
 __device__ __forceinline__ void single_block_scan_1024(const T* __restrict__ in, T* __restrict__ out,
                                                        int64_t count, T* sum) {

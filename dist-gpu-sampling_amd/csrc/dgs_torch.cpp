@@ -345,23 +345,24 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
   if (one_shot) {
     rows = torch::empty({n * num_picks}, seeds.options());
     cols = torch::empty({n * num_picks}, seeds.options());
-    // count (which mirrors the length into pinned memory), a ticket, then the fill: the host waits
-    // for the ticket only, and the fill is still running when the operator returns
+    // count (which mirrors the length into pinned memory), then the fill: the host waits for the
+    // mirrored words only, and the fill is still running when the operator returns
     thread_local torch::Tensor pinned =
         torch::empty({2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(),
-                           pinned.data_ptr<int64_t>(), ws.data_ptr(), ws_bytes, st));
-    void* ticket = nullptr;
-    check(dgs_ticket_record(st, &ticket));
+    int64_t* words = pinned.data_ptr<int64_t>();
+    words[0] = words[1] = -1;  // the kernel's words are never negative: the wait below polls them
+    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(), words,
+                           ws.data_ptr(), ws_bytes, st));
     const dgs_status fill_status =
         probs != nullptr
             ? dgs_sample_fill_weighted(seeds.data_ptr(), w, n, indices, *probs, num_picks, replace, rng.first,
                                        rng.second, rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st)
             : dgs_sample_fill(seeds.data_ptr(), w, n, indices, num_picks, replace, rng.first, rng.second,
                               rows.data_ptr(), cols.data_ptr(), ws.data_ptr(), ws_bytes, st);
-    check(dgs_ticket_wait(ticket));
+    check(dgs_stream_wait_words(st, words, 2));
     check(fill_status);
-    len.assign(pinned.data_ptr<int64_t>(), pinned.data_ptr<int64_t>() + 2);
+    TORCH_CHECK(words[0] >= 0 && words[1] >= 0, "sample_neighbors: the count kernel left no lengths");
+    len.assign(words, words + 2);
   } else {
     check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(), nullptr,
                            ws.data_ptr(), ws_bytes, st));
@@ -535,10 +536,11 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> TensorRelabel(std::vector<
   // that attempt and the call is repeated with the two-array table
   int64_t u = 0;
   for (const int32_t packed : {1, 0}) {
-    void* ticket = nullptr;
+    counts_host[0] = counts_host[1] = -1;  // the kernels' words are never negative: the wait polls them
     check(dgs_unique_relabel(map_seg, req_seg, w, packed, unique.data_ptr(), counts.data_ptr<int64_t>(), counts_host,
-                             &ticket, out_seg, ws.data_ptr(), ws_bytes, current_stream()));
-    check(dgs_ticket_wait(ticket));
+                             nullptr, out_seg, ws.data_ptr(), ws_bytes, current_stream()));
+    check(dgs_stream_wait_words(current_stream(), counts_host, 2));
+    TORCH_CHECK(counts_host[0] >= 0 && counts_host[1] >= 0, "tensor_relabel: the kernels left no counts");
     u = counts_host[0];
     if (counts_host[1] == 0) break;
     TORCH_CHECK(packed != 0, "tensor_relabel: the table rejected an id");
@@ -569,12 +571,13 @@ class PendingBlocks : public torch::CustomClassHolder {
     if (ticket_ != nullptr) {
       void* t = ticket_;
       ticket_ = nullptr;
-      ws_status = dgs_ticket_wait(t);
+      ws_status = dgs_ticket_wait_words(t, pinned_.data_ptr<int64_t>(), 3 * hops_ + 1);
     }
     check(gather_status_);
     check(ws_status);
     const int64_t* sizes_host = pinned_.data_ptr<int64_t>();
     const int n_sizes = 3 * hops_ + 1;
+    for (int i = 0; i < n_sizes; ++i) TORCH_CHECK(sizes_host[i] >= 0, "sample_blocks: the kernels left no lengths");
     const std::vector<int64_t> sz(sizes_host, sizes_host + n_sizes);
     std::vector<torch::Tensor> frontier(hops_);
     for (int h = 0; h < hops_; ++h) {
@@ -633,6 +636,7 @@ class PendingBlocks : public torch::CustomClassHolder {
     p->stream_ = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap();
     // the kernels mirror the lengths into this call's own pinned words
     p->pinned_ = torch::empty({32}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    for (int i = 0; i < 32; ++i) p->pinned_.data_ptr<int64_t>()[i] = -1;  // Finish polls them: lengths are never negative
     if (seeds_in.device().is_cpu() && !seeds_in.is_pinned() && n > 0) {
       // pageable host seeds (what upstream's DataLoader passes): staged through pinned memory of
       // this batch, so that the upload is a plain asynchronous copy the host does not wait for

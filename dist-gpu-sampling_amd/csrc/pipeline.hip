@@ -638,10 +638,10 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, int64_t
       *h.nnz = edges;
       *h.flags = bad;
       if (h.host_sizes) {
-        if (h.index == 0) h.host_sizes[0] = s;
-        h.host_sizes[h.index + 1] = rank0 + part;
-        h.host_sizes[h.n_hops + 1 + h.index] = edges;
-        h.host_sizes[2 * h.n_hops + 1 + h.index] = bad;
+        if (h.index == 0) mirror_to_host(h.host_sizes, s);
+        mirror_to_host(h.host_sizes + h.index + 1, rank0 + part);
+        mirror_to_host(h.host_sizes + h.n_hops + 1 + h.index, edges);
+        mirror_to_host(h.host_sizes + 2 * h.n_hops + 1 + h.index, bad);
       }
     }
     if (len <= 0) return;

@@ -107,8 +107,8 @@ __global__ __launch_bounds__(1024) void sample_scan_kernel(const int64_t* __rest
     nnz_dev[0] = sum;
     nnz_dev[1] = any_flag;
     if (nnz_host) {  // pinned host memory: the caller reads the length without a copy
-      nnz_host[0] = sum;
-      nnz_host[1] = any_flag;
+      mirror_to_host(nnz_host, sum);
+      mirror_to_host(nnz_host + 1, any_flag);
     }
   }
 }

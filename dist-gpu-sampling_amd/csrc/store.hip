@@ -3,6 +3,7 @@
 // (upstream src/chunk_tensor.cc:112-139) have no counterpart here.
 #include <atomic>
 #include <cstdarg>
+#include <chrono>
 #include <mutex>
 #include <vector>
 #include <cstring>
@@ -271,6 +272,63 @@ DGS_API dgs_status dgs_ticket_wait(void* ticket) {
   }
   if (e != hipSuccess) {
     dgs::set_error("ticket_wait: %s", hipGetErrorString(e));
+    return DGS_ERR_HIP;
+  }
+  return DGS_OK;
+}
+
+namespace dgs {
+// Polls `n_words` host words until all are non-negative.  `still_running` is asked now and then
+// whether the work that writes them can still be under way (it may cost far more than a poll:
+// a stream query takes tens of microseconds, so the first one comes after 200 us of polling and
+// the next ones 100 us apart); when it says no, or fails, the wait ends.
+template <typename StillRunning>
+static hipError_t poll_words(const int64_t* words, int32_t n_words, StillRunning still_running) {
+  using clock = std::chrono::steady_clock;
+  int32_t seen = 0;  // words [0, seen) have turned non-negative
+  clock::time_point next_ask;
+  bool timing = false;
+  for (uint32_t spins = 1;; ++spins) {
+    while (seen < n_words && __atomic_load_n(words + seen, __ATOMIC_ACQUIRE) >= 0) ++seen;
+    if (seen == n_words) return hipSuccess;
+    if ((spins & 63u) == 0) {
+      const clock::time_point now = clock::now();
+      if (!timing) {
+        timing = true;
+        next_ask = now + std::chrono::microseconds(200);
+      } else if (now >= next_ask) {
+        const hipError_t e = still_running();
+        if (e != hipErrorNotReady) return e;  // finished (the words are what they will be) or failed
+        next_ask = clock::now() + std::chrono::microseconds(100);
+      }
+    }
+    __builtin_ia32_pause();
+  }
+}
+}  // namespace dgs
+
+DGS_API dgs_status dgs_ticket_wait_words(void* ticket, const int64_t* words, int32_t n_words) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_wait_words: null ticket");
+  DGS_REQUIRE(words != nullptr && n_words >= 1, DGS_ERR_INVALID, "ticket_wait_words: no words");
+  hipEvent_t ev = static_cast<hipEvent_t>(ticket);
+  const hipError_t e = dgs::poll_words(words, n_words, [ev] { return hipEventQuery(ev); });
+  {
+    std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
+    dgs::g_event_pool.push_back(ev);
+  }
+  if (e != hipSuccess) {
+    dgs::set_error("ticket_wait_words: %s", hipGetErrorString(e));
+    return DGS_ERR_HIP;
+  }
+  return DGS_OK;
+}
+
+DGS_API dgs_status dgs_stream_wait_words(void* stream, const int64_t* words, int32_t n_words) {
+  DGS_REQUIRE(words != nullptr && n_words >= 1, DGS_ERR_INVALID, "stream_wait_words: no words");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const hipError_t e = dgs::poll_words(words, n_words, [st] { return hipStreamQuery(st); });
+  if (e != hipSuccess) {
+    dgs::set_error("stream_wait_words: %s", hipGetErrorString(e));
     return DGS_ERR_HIP;
   }
   return DGS_OK;

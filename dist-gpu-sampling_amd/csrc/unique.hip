@@ -104,8 +104,8 @@ __global__ __launch_bounds__(1024) void unique_scan_kernel(const int* __restrict
     counts_dev[0] = sum;
     counts_dev[1] = bad;
     if (counts_host) {
-      counts_host[0] = sum;
-      counts_host[1] = bad;
+      mirror_to_host(counts_host, sum);
+      mirror_to_host(counts_host + 1, bad);
     }
   }
 }
@@ -271,8 +271,8 @@ __global__ __launch_bounds__(kSmallThreads) void small_relabel_kernel(dgs_segmen
     counts_dev[0] = base;
     counts_dev[1] = overflow;
     if (counts_host) {
-      counts_host[0] = base;
-      counts_host[1] = overflow;
+      mirror_to_host(counts_host, base);
+      mirror_to_host(counts_host + 1, overflow);
     }
   }
   // relabel: rank of every requiring id, -1 when it is not in the table; eight ids a thread at a time
@@ -445,8 +445,8 @@ DGS_API dgs_status dgs_unique_relabel(dgs_segments mapping, dgs_segments requiri
                     (requiring.len[k] == 0 || (requiring.ptr[k] && out.ptr[k])),
                 DGS_ERR_INVALID, "relabel: bad requiring/output segment %d", k);
   DGS_REQUIRE(counts_dev != nullptr, DGS_ERR_INVALID, "relabel: null counts_dev");
-  DGS_REQUIRE((counts_host == nullptr) == (counts_ticket == nullptr), DGS_ERR_INVALID,
-              "relabel: counts_host and counts_ticket go together");
+  DGS_REQUIRE(counts_ticket == nullptr || counts_host != nullptr, DGS_ERR_INVALID,
+              "relabel: a counts_ticket needs counts_host");
   const int64_t n = seg_total(mapping);
   const int64_t m = seg_total(requiring);
   DGS_REQUIRE(n <= kMaxMappingIds, DGS_ERR_UNSUPPORTED, "relabel: %lld mapping ids exceed 2^30", (long long)n);

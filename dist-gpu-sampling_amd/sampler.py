@@ -104,6 +104,7 @@ class ChunkTensorSampler:
         self.seed = None if seed is None else int(seed)
         self._batches = 0
         self._count_lock = threading.Lock()
+        self._loops = {}  # BatchPipeline's native loops (each with a worker thread), kept for reuse
 
     def _first_stream(self, batch):
         """Stream of the first hop of a batch drawn from the sampler's own state."""
@@ -265,8 +266,6 @@ class BatchPipeline:
         self.hand_over = hand_over
         self.gathers_in_turn = gathers_in_turn
         self.native_loop = native_loop
-        self._loop = None
-        self._loop_busy = False
         if inflight < 1:
             raise ValueError("inflight must be at least 1")
         self.sampler = sampler
@@ -296,20 +295,30 @@ class BatchPipeline:
         return out
 
     def _native(self):
-        """The extension's own loop for this pipeline (made once): a worker thread of the extension
-        begins the batches, so that Python pays one call to hand seeds in and one to take a batch out."""
-        if self._loop is None:
-            smp = self.sampler
+        """The extension's own loop for this pipeline: a worker thread of the extension begins the
+        batches, so that Python pays one call to hand seeds in and one to take a batch out.
+        Loops are kept with the sampler (starting a thread costs as much as half a batch) and
+        shared by its pipelines over the same features, streams and settings; returns None
+        while another iteration is using the one this pipeline would take."""
+        smp = self.sampler
+        key = (id(self.chunk_features), tuple(st.stream_id for st in self.streams), self.hand_over,
+               self.gathers_in_turn, tuple(smp.fanouts), smp.replace, id(smp.chunk_probs))
+        entry = smp._loops.get(key)
+        if entry is None:
             triples = []
             for st in self.streams:
                 triples += [st.stream_id, st.device_index, st.device_type]
-            self._loop = torch.classes.dgs_classes.BatchLoop(
+            loop = torch.classes.dgs_classes.BatchLoop(
                 smp.chunk_indptr, smp.chunk_indices, smp.chunk_probs, list(reversed(smp.fanouts)), smp.replace,
                 self.chunk_features, triples, self.hand_over, self.gathers_in_turn, [])
-        return self._loop
+            # (the features are kept with the entry so that their id stays theirs)
+            entry = smp._loops[key] = {"loop": loop, "busy": False, "features": self.chunk_features}
+        if entry["busy"]:
+            return None
+        return entry
 
-    def _iterate_native(self, seed_batches):
-        loop = self._native()
+    def _iterate_native(self, entry, seed_batches):
+        loop = entry["loop"]
         n = len(self.streams)
         with_x = self.chunk_features is not None
         waiting = deque()
@@ -321,7 +330,7 @@ class BatchPipeline:
             seed_nodes = waiting.popleft()
             return (frontiers[-1], seed_nodes, blocks, x) if with_x else (frontiers[-1], seed_nodes, blocks)
 
-        self._loop_busy = True
+        entry["busy"] = True
         try:
             for seeds in seed_batches:
                 # the first batch on each stream goes behind what the caller's stream holds now,
@@ -339,15 +348,17 @@ class BatchPipeline:
                     loop._CAPI_pop()
                 except RuntimeError:
                     pass
-            self._loop_busy = False
+            entry["busy"] = False
 
     def __call__(self, seed_batches):
         # (a sampler with its own generator counts its batches in Python, and a second iteration
         # that starts while one is under way cannot share the first one's queue: both keep the
         # Python loop)
-        if self.native_loop and self.sampler.fused and self.sampler.seed is None and not self._loop_busy:
-            yield from self._iterate_native(seed_batches)
-            return
+        if self.native_loop and self.sampler.fused and self.sampler.seed is None:
+            entry = self._native()
+            if entry is not None:
+                yield from self._iterate_native(entry, seed_batches)
+                return
         consumer = torch.cuda.current_stream()
         n = len(self.streams)
         # Events are made once per process and reused (making one costs more than the stream wait

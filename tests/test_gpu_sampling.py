@@ -39,7 +39,7 @@ def test_sample_parity_c_abi(pkg, oracle, graph, k, replace):
     seeds = rng.integers(0, 20000, size=3001).astype(np.int64)
     want_r, want_c = oracle.sample_neighbors(seeds, indptr, indices, k, replace, 0xABCDEF0123, 9)
     ip, ix = _dev(indptr), _dev(indices)
-    for two_step in (False, True):
+    for two_step in (False, True, "mirrored"):  # "mirrored": the length through polled pinned words
         r, c, flags = capi.sample_neighbors(_dev(seeds), capi.tensor_view(ip), capi.tensor_view(ix), k, replace,
                                             0xABCDEF0123, 9, two_step=two_step)
         assert flags == 0
@@ -335,8 +335,9 @@ def test_unique_relabel_parity(pkg, oracle, dtype, n, hi):
     rows = rng.choice(seeds, size=n).astype(dtype)
     want_u, (want_r, want_c) = oracle.unique_relabel([seeds, cols], [rows, cols])
     assert np.array_equal(want_u, np_unique_first(np.concatenate([seeds, cols])))
-    u, (r, c) = pkg.capi.unique_relabel([_dev(seeds), _dev(cols)], [_dev(rows), _dev(cols)])
-    assert np.array_equal(_np(u), want_u) and np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
+    for polled in (False, True):  # the counts by a copy, and through pinned words the host polls
+        u, (r, c) = pkg.capi.unique_relabel([_dev(seeds), _dev(cols)], [_dev(rows), _dev(cols)], polled=polled)
+        assert np.array_equal(_np(u), want_u) and np.array_equal(_np(r), want_r) and np.array_equal(_np(c), want_c)
     # operator layer, including an id that is absent from the mapping
     extra = np.array([hi + 5], dtype=dtype)
     u2, outs = pkg.ops._CAPI_tensor_relabel([_dev(seeds), _dev(cols)], [_dev(rows), _dev(cols), _dev(extra)])
