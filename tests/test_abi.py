@@ -80,6 +80,27 @@ def test_operator_surface_is_registered():
         torch.ops.dgs_ops._CAPI_set_nccl(2, [0] * 16, 1)
 
 
+def test_torch_dispatch_is_lightened_for_custom_class_arguments():
+    # importing the package opts torch.ScriptObject out of the __torch_function__ lookup (a miss
+    # costs two C++ exceptions per ChunkTensor argument per call) and binds the operators that
+    # take ChunkTensors to their C++ entry; DGS_PLAIN_TORCH_DISPATCH=1 leaves torch alone
+    import subprocess
+    import sys
+    import torch
+    load_pkg()
+    assert vars(torch.ScriptObject)["__torch_function__"] is torch._C._disabled_torch_function_impl
+    assert type(torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor).__name__ == "builtin_function_or_method"
+    assert type(torch.ops.dgs_ops._CAPI_sample_neighbors).__name__ == "OpOverloadPacket"
+    code = ("import importlib, os, sys, torch; sys.path.insert(0, %r); importlib.import_module('dist-gpu-sampling_amd');"
+            "print('__torch_function__' in vars(torch.ScriptObject),"
+            " type(torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor).__name__)"
+            % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    out = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, DGS_PLAIN_TORCH_DISPATCH="1"),
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.split() == ["False", "OpOverloadPacket"]
+
+
 def test_no_gpu_means_a_loud_error_not_a_fallback():
     import torch
     if torch.cuda.is_available():

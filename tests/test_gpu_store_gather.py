@@ -272,3 +272,29 @@ def test_gather_dyn_leaves_a_buffer_alone_that_is_too_small(pkg, dim):
         assert torch.equal(out[:written].cpu(), full[idx[:written].cpu()]), count
         assert (out[written:] == -3.0).all().item(), count
     st.close()
+
+
+def test_waiting_for_words_that_nobody_writes_ends_with_the_ticket(pkg):
+    # dgs_ticket_wait_words / dgs_stream_wait_words poll pinned words that the kernels turn
+    # non-negative; a ticket whose point is reached, or a stream that has drained, ends the wait
+    # all the same (here: nothing was launched that would write the words), and words that were
+    # written before the call end it at once
+    import ctypes
+    import time
+    capi = pkg.capi
+    words = torch.full((3,), -1, dtype=torch.int64).pin_memory()
+    torch.cuda.synchronize()
+    ticket = ctypes.c_void_p()
+    capi.check(capi.lib.dgs_ticket_record(capi.stream_ptr(), ctypes.byref(ticket)))
+    t0 = time.perf_counter()
+    capi.check(capi.lib.dgs_ticket_wait_words(ticket, words.data_ptr(), 3))
+    assert time.perf_counter() - t0 < 0.5 and words.tolist() == [-1, -1, -1]
+    t0 = time.perf_counter()
+    capi.check(capi.lib.dgs_stream_wait_words(capi.stream_ptr(), words.data_ptr(), 3))
+    assert time.perf_counter() - t0 < 0.5
+    words[:] = torch.tensor([0, 7, 1 << 40])
+    capi.check(capi.lib.dgs_ticket_record(capi.stream_ptr(), ctypes.byref(ticket)))
+    capi.check(capi.lib.dgs_ticket_wait_words(ticket, words.data_ptr(), 3))
+    capi.check(capi.lib.dgs_stream_wait_words(capi.stream_ptr(), words.data_ptr(), 3))
+    with pytest.raises(capi.DgsError):
+        capi.check(capi.lib.dgs_stream_wait_words(capi.stream_ptr(), None, 3))
