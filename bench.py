@@ -451,7 +451,7 @@ def main():
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + sorted(LARGE))
     ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
     ap.add_argument("--inflight", type=int, default=None,
-                    help="batches in flight on as many streams (1 = one blocking call per batch); default 3 for "
+                    help="batches in flight on as many streams (1 = one blocking call per batch); default 4 for "
                          "c0/c1/c1w and 2 for the large workloads, whose batches are long enough for two to fill the GPU")
     ap.add_argument("--gather-buffer-cap-gib", type=float, default=None,
                     help="largest feature buffer the fused operator allocates ahead of a batch's sizes "
@@ -470,7 +470,7 @@ def main():
     dgs = importlib.import_module("dist-gpu-sampling_amd")
     torch.cuda.set_device(0)
     if args.inflight is None:
-        args.inflight = 2 if args.workload in LARGE else 3
+        args.inflight = 2 if args.workload in LARGE else 4
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
     if args.workload in LARGE:
@@ -533,12 +533,15 @@ def main():
     ms_latency = 1e3 * timed_steps(sampler, batches, 1)[0] / args.steps
     # batches in flight again, each handed over to the calling stream (made to wait for the batch,
     # buffers recorded there): what a consumer on another stream than the batch's own sees
-    ms_handed_over = 1e3 * timed_steps(sampler, batches, inflight, True)[0] / args.steps if inflight > 1 else None
+    # (the calling stream is one more stream: with it, at most four share the GPU's hardware queues)
+    handed_inflight = min(inflight, 3)
+    ms_handed_over = (1e3 * timed_steps(sampler, batches, handed_inflight, True)[0] / args.steps
+                      if inflight > 1 else None)
     # seeds as upstream's DataLoader passes them: pageable host tensors, uploaded by the operator
     ms_host_seeds = 1e3 * timed_steps(sampler, batches_cpu, inflight)[0] / args.steps
     # both: host seeds in, every batch handed to the calling stream -- what upstream's training loop
     # would see (its DataLoader passes host seeds, its model runs on the current stream)
-    ms_handed_over_host_seeds = (1e3 * timed_steps(sampler, batches_cpu, inflight, True)[0] / args.steps
+    ms_handed_over_host_seeds = (1e3 * timed_steps(sampler, batches_cpu, handed_inflight, True)[0] / args.steps
                                  if inflight > 1 else None)
     # what an unmodified upstream harness runs: per hop one sampling operator and one relabel
     # operator (each returns tensors of exact length, so each waits for its lengths), then _CAPI_index
@@ -627,7 +630,8 @@ def main():
         "ms_per_step_per_hop_ops_no_gather": ms_per_hop_ops_no_gather,
         "timings": {"ms_per_step_repeats": "the timed region run three more times (spread)",
                     "ms_per_batch_alone": "one batch at a time, one stream, call to result",
-                    "ms_per_step_handed_over": "as the headline, each batch handed to the calling stream",
+                    "ms_per_step_handed_over": "as the headline, each batch handed to the calling stream "
+                                               "(at most three batches in flight: the calling stream is a stream too)",
                     "ms_per_step_host_seeds": "as the headline, seeds passed as pageable host tensors",
                     "ms_per_step_handed_over_host_seeds": "host seeds in, each batch handed to the calling stream",
                     "ms_per_step_per_hop_ops": "upstream's own loop: _CAPI_sample_neighbors_with_chunk_tensor + "

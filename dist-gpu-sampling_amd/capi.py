@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libdgs_hip.so")
 DGS_OK, DGS_ERR_INVALID, DGS_ERR_HIP, DGS_ERR_WORKSPACE, DGS_ERR_UNSUPPORTED, DGS_ERR_RANGE = range(6)
 TIER_ANY, TIER_DEVICE, TIER_HOST = 0, 1, 2
 DEBUG_FORCE_SPLIT_TABLE, DEBUG_WEIGHTED_GROUP, DEBUG_GATHER_LDS_BYTES, DEBUG_SAMPLER_GRID_CAP = 0, 1, 2, 3
+DEBUG_SAMPLER_BUCKETED = 4
 PROBE_LOAD, PROBE_STORE, PROBE_ATOMIC_MIN, PROBE_ATOMIC_MIN_NO_RETURN = 0, 1, 2, 3
 MAX_SEGMENTS = 8
 

@@ -118,7 +118,7 @@ struct Hop {
   int32_t k;
   int32_t index;            // hop number
   uint32_t rng_stream;
-  int32_t pad_;
+  int32_t bucketed;         // non-zero: first occurrences come from the bucketed pass (see Buckets)
 };
 
 // (written without a conditional so that the read is not moved behind a test)
@@ -133,6 +133,39 @@ __device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h
 __device__ __forceinline__ int64_t first_rank(const Hop& h, int64_t s) { return h.index == 0 ? 0 : s; }
 constexpr int kRelabelItems = 4;  // padded picks per thread in relabel_tile
 __host__ __device__ __forceinline__ int relabel_groups(int k) { return (k + kRelabelItems - 1) / kRelabelItems; }
+
+// ---- a large last hop without memory-side atomics -------------------------------------------
+// The atomicMin per pick is what a large hop costs most (every device-scope atomic executes at
+// the memory side: 26.7 G/s, 31 us for the 832 k picks of a 1024 x [5,10,15] batch, and as much
+// again while other batches share the GPU).  The last hop needs no table entry afterwards, so its
+// first occurrences can be found without the table: the picks, together with the ids the
+// frontier already holds, are grouped by the low bits of the id (count, column scan, scatter:
+// streamed reads and writes), and one block per group takes the smallest position of every id in
+// an LDS array indexed by the id's high bits.  A pick's slot word then says everything the later
+// stages need: first occurrence (id | kFirstBit), a repeat of an id the frontier held before
+// this hop (its rank | kRankBit: final, no further lookup), or a repeat of a pick of this hop
+// (that pick's position, whose rank the compaction records).  Same result as the table gives.
+constexpr int kBucketTile = 4096;                    // units (frontier ids, then pick positions) per count/scatter block
+constexpr int kBucketTileItems = kBucketTile / kBlock;
+constexpr int kMinBuckets = 512;
+constexpr int kMaxBuckets = 2048;
+constexpr int kBucketRange = 8192;                   // ids per bucket at most: 32 KB of LDS
+constexpr int64_t kBucketedMaxNodes = int64_t(kMaxBuckets) * kBucketRange;
+constexpr int64_t kBucketedMinPicks = int64_t(1) << 18;  // worst-case picks of the hop below which the table is cheaper
+constexpr int64_t kBucketedMaxUnits = int64_t(1) << 23;  // bounds the extra workspace (8 bytes a unit)
+constexpr uint32_t kRankBit = 0x40000000u;
+
+struct Buckets {
+  uint2* items;      // [units_max] (id, order value) grouped by bucket; order value = rank of a frontier id, position of a pick
+  int* hist;         // [tiles_max][buckets] units of a tile per bucket, then their exclusive prefix down the column
+  int* total;        // [buckets]
+  int* start;        // [buckets + 1]
+  int64_t units_max; // items[] holds this many
+  int32_t tiles_max; // tiles of units: front_tiles over the frontier array, the rest over the hop's padded positions
+  int32_t front_tiles;
+  int32_t log_buckets;
+  uint32_t n_nodes;
+};
 
 // rank of the id at position p, given p's slot word
 template <typename TableT>
@@ -247,16 +280,25 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   // for all of the thread's picks before any is used, and both before the block adds up its
   // prefix (whose barrier nothing here has to wait behind).
   bool live[kRelabelItems];
+  bool known[kRelabelItems];  // bucketed hop: the word of a repeat may be the rank itself
   uint32_t at[kRelabelItems];
 #pragma unroll
   for (int j = 0; j < kRelabelItems; ++j) {
     live[j] = mine[j] && i[j] < s && !is_bad_row(rc[j]) && uint32_t(l[j]) < rc[j];
     at[j] = uint32_t(p[j]);
-    if (live[j] && !(word[j] & kFirstBit)) at[j] = table.value(word[j]);
+    known[j] = false;
+    if (live[j] && !(word[j] & kFirstBit)) {
+      if (h.bucketed) {
+        known[j] = (word[j] & kRankBit) != 0;
+        at[j] = word[j] & (kRankBit - 1);
+      } else {
+        at[j] = table.value(word[j]);
+      }
+    }
   }
   uint32_t rank[kRelabelItems];
 #pragma unroll
-  for (int j = 0; j < kRelabelItems; ++j) rank[j] = live[j] ? h.rank_at[at[j]] : 0u;
+  for (int j = 0; j < kRelabelItems; ++j) rank[j] = !live[j] ? 0u : known[j] ? at[j] : h.rank_at[at[j]];
   const int64_t prefix = block_sum<kBlock, int64_t>(part, lds);
 #pragma unroll
   for (int j = 0; j < kRelabelItems; ++j) {
@@ -291,7 +333,9 @@ __device__ __forceinline__ bool emit_pick(const Hop& h, const TableT& table, con
   if (have) {
     const IdT col = indices.at(edge);
     ok = table.holds(col);
-    if (ok) {
+    if (ok && h.bucketed) {
+      word = uint32_t(col) | kFirstBit;  // a first occurrence until the bucketed pass says otherwise; the table is left alone
+    } else if (ok) {
       bool first;
       uint32_t displaced;
       word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
@@ -524,6 +568,254 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
   }
 }
 
+// ---- the bucketed pass (see Buckets) --------------------------------------------------------
+
+// The units of a bucketed hop are the frontier's ids (order value = rank) and the hop's padded
+// positions (order value = position, which is above every rank).  They are cut into tiles of
+// kBucketTile whose addresses do not depend on the hop's length, so that a block can ask for its
+// units at once: front_tiles tiles over the frontier array as large as it can get, then the
+// tiles of the padded positions.  Tiles that hold nothing (beyond the real frontier, beyond the
+// real positions) are skipped when rows of hist are numbered: row = tile for a frontier tile
+// that holds ids, (frontier tiles that hold ids) + (tile - front_tiles) for a position tile.
+struct TileOfUnits {
+  bool front;      // a tile of frontier ids
+  int64_t first;   // its first rank, or its first position relative to the hop's pos_base
+};
+__device__ __forceinline__ TileOfUnits bucket_tile(const Buckets& b, int64_t tile) {
+  TileOfUnits t;
+  t.front = tile < b.front_tiles;
+  t.first = (t.front ? tile : tile - b.front_tiles) * kBucketTile;
+  return t;
+}
+// rows of hist in use, and the row of a tile (-1: the tile holds nothing)
+__device__ __forceinline__ int64_t bucket_front_rows(int64_t s) { return (s + kBucketTile - 1) / kBucketTile; }
+__device__ __forceinline__ int64_t bucket_rows(const Hop& h, int64_t s) {
+  return bucket_front_rows(s) + (s * h.k + kBucketTile - 1) / kBucketTile;
+}
+__device__ __forceinline__ int64_t bucket_row(const Hop& h, const TileOfUnits& t, int64_t s) {
+  if (t.front) return t.first < s ? t.first / kBucketTile : -1;
+  return t.first < s * h.k ? bucket_front_rows(s) + t.first / kBucketTile : -1;
+}
+// A thread's units of a tile, requested without knowing the hop's length (every address lies inside
+// its array whatever the length turns out to be); `valid` then says which of them count.
+template <typename IdT>
+struct UnitsOfThread {
+  uint32_t id[kBucketTileItems];
+  uint32_t order[kBucketTileItems];
+  bool inside[kBucketTileItems];  // the address was inside the array, so id[] was loaded
+  __device__ __forceinline__ void load(const Hop& h, const TileOfUnits& t) {
+#pragma unroll
+    for (int j = 0; j < kBucketTileItems; ++j) {
+      const int64_t at = t.first + j * kBlock + threadIdx.x;
+      if (t.front) {
+        inside[j] = at < h.s_max;
+        id[j] = inside[j] ? uint32_t(static_cast<const IdT*>(h.frontier)[at]) : 0u;
+        order[j] = uint32_t(at);
+      } else {
+        inside[j] = at < h.len_max;
+        const uint32_t word = inside[j] ? h.slot[h.pos_base + at] : kInvalidSlot;  // id | kFirstBit as the fill left it
+        inside[j] = inside[j] && word != kInvalidSlot;
+        id[j] = word & ~kFirstBit;
+        order[j] = uint32_t(h.pos_base + at);
+      }
+    }
+  }
+  __device__ __forceinline__ bool valid(const Hop& h, const TileOfUnits& t, int64_t s, int j) const {
+    const int64_t at = t.first + j * kBlock + threadIdx.x;
+    return inside[j] && at < (t.front ? s : s * h.k);
+  }
+};
+
+// hist[row][bucket] = units of the tile whose id falls into the bucket (id mod buckets)
+template <typename IdT>
+__global__ __launch_bounds__(kBlock) void bucket_count_kernel(Hop h, Buckets b) {
+  __shared__ int cnt[kMaxBuckets];
+  const int buckets = 1 << b.log_buckets;
+  for (int64_t tile = blockIdx.x; tile < b.tiles_max; tile += gridDim.x) {
+    const TileOfUnits t = bucket_tile(b, tile);
+    UnitsOfThread<IdT> mine;
+    mine.load(h, t);
+    const int64_t s = seeds_of(h);
+    const int64_t row = bucket_row(h, t, s);
+    if (row < 0 || row >= b.tiles_max) continue;  // whole blocks skip a tile together
+    for (int j = threadIdx.x; j < buckets; j += kBlock) cnt[j] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kBucketTileItems; ++j)
+      if (mine.valid(h, t, s, j)) atomicAdd(&cnt[mine.id[j] & uint32_t(buckets - 1)], 1);
+    __syncthreads();
+    for (int j = threadIdx.x; j < buckets; j += kBlock) b.hist[row * buckets + j] = cnt[j];
+    __syncthreads();
+  }
+}
+
+// Down every column of hist: exclusive prefix in place, total[bucket] = the column's sum.  A
+// block takes 32 buckets; its 32 x 32 threads split the rows into 32 runs.
+__global__ __launch_bounds__(1024) void bucket_scan_kernel(Hop h, Buckets b) {
+  __shared__ int part[32][33];
+  const int buckets = 1 << b.log_buckets;
+  const int lane = threadIdx.x & 31, run = threadIdx.x >> 5;
+  const int bucket = blockIdx.x * 32 + lane;  // the grid has buckets / 32 blocks
+  int64_t rows = bucket_rows(h, seeds_of(h));
+  if (rows > b.tiles_max) rows = b.tiles_max;
+  const int64_t per = (rows + 31) / 32;
+  const int64_t t0 = run * per < rows ? run * per : rows;
+  const int64_t t1 = t0 + per < rows ? t0 + per : rows;
+  int sum = 0;
+  for (int64_t t = t0; t < t1; ++t) sum += b.hist[t * buckets + bucket];
+  part[run][lane] = sum;
+  __syncthreads();
+  int before = 0;
+  for (int r = 0; r < run; ++r) before += part[r][lane];
+  for (int64_t t = t0; t < t1; ++t) {
+    const int v = b.hist[t * buckets + bucket];
+    b.hist[t * buckets + bucket] = before;
+    before += v;
+  }
+  if (run == 31) b.total[bucket] = before;  // the runs before the last one, plus its own
+}
+
+// Every unit goes to its bucket's stretch of items[]: start of the bucket (prefix over total[],
+// which every block works out for itself) + the units of earlier rows + a turn among its own
+// tile's.  A tile's units are first put in bucket order in LDS and written out from there, so
+// that what goes to one bucket leaves as one contiguous piece instead of unit by unit.
+template <typename IdT>
+__global__ __launch_bounds__(kBlock) void bucket_scatter_kernel(Hop h, Buckets b) {
+  __shared__ int start[kMaxBuckets];   // first item of every bucket
+  __shared__ int base[kMaxBuckets];    // where the tile's first staged unit of a bucket goes, minus its place in the stage
+  __shared__ int cur[kMaxBuckets];     // next free place in the stage for every bucket
+  __shared__ uint2 stage[kBucketTile];
+  __shared__ int lds[kBlock / kWave];
+  const int buckets = 1 << b.log_buckets;
+  const int mine = buckets / kBlock;  // 2..8 consecutive buckets per thread
+  // the first tile's units and the bucket totals, requested together
+  TileOfUnits t = bucket_tile(b, blockIdx.x);
+  UnitsOfThread<IdT> units;
+  if (int64_t(blockIdx.x) < b.tiles_max) units.load(h, t);
+  int own[kMaxBuckets / kBlock];
+  int sum = 0;
+#pragma unroll
+  for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
+    own[j] = j < mine ? b.total[threadIdx.x * mine + j] : 0;
+    sum += own[j];
+  }
+  const int64_t s = seeds_of(h);
+  int64_t rows = bucket_rows(h, s);
+  if (rows > b.tiles_max) rows = b.tiles_max;
+  int all;
+  int at = block_exclusive_scan<kBlock, int>(sum, &all, lds);
+#pragma unroll
+  for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
+    if (j < mine) {
+      start[threadIdx.x * mine + j] = at;
+      if (blockIdx.x == 0) b.start[threadIdx.x * mine + j] = at;
+      at += own[j];
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) b.start[buckets] = all;
+  __syncthreads();
+  for (int64_t tile = blockIdx.x; tile < b.tiles_max; tile += gridDim.x) {
+    if (tile != int64_t(blockIdx.x)) {
+      t = bucket_tile(b, tile);
+      units.load(h, t);
+    }
+    const int64_t row = bucket_row(h, t, s);
+    if (row < 0 || row >= rows) continue;  // whole blocks skip a tile together
+    // this tile's units per bucket: the difference of the column prefixes of this row and the next
+    int before[kMaxBuckets / kBlock];
+    sum = 0;
+#pragma unroll
+    for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
+      own[j] = before[j] = 0;
+      if (j < mine) {
+        const int bucket = threadIdx.x * mine + j;
+        before[j] = b.hist[row * buckets + bucket];
+        const int upto = row + 1 < rows ? b.hist[(row + 1) * buckets + bucket] : b.total[bucket];
+        own[j] = upto - before[j];
+        if (own[j] < 0 || own[j] > kBucketTile) own[j] = 0;  // cannot happen; keeps what follows inside the stage
+        sum += own[j];
+      }
+    }
+    at = block_exclusive_scan<kBlock, int>(sum, &all, lds);
+#pragma unroll
+    for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
+      if (j < mine) {
+        const int bucket = threadIdx.x * mine + j;
+        cur[bucket] = at;
+        base[bucket] = start[bucket] + before[j] - at;
+        at += own[j];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kBucketTileItems; ++j) {
+      if (units.valid(h, t, s, j)) {
+        const int to = atomicAdd(&cur[units.id[j] & uint32_t(buckets - 1)], 1);
+        if (to >= 0 && to < kBucketTile) stage[to] = make_uint2(units.id[j], units.order[j]);
+      }
+    }
+    __syncthreads();
+    const int staged = all < kBucketTile ? all : kBucketTile;
+    for (int e = threadIdx.x; e < staged; e += kBlock) {
+      const uint2 it = stage[e];
+      const int64_t to = int64_t(base[it.x & uint32_t(buckets - 1)]) + e;
+      if (to >= 0 && to < b.units_max) b.items[to] = it;
+    }
+    __syncthreads();
+  }
+}
+
+// One block per bucket: the smallest order value of every id (LDS, indexed by id / buckets), then
+// the slot word of every pick that is not its id's first occurrence.
+__global__ __launch_bounds__(kBlock) void bucket_first_kernel(Hop h, Buckets b) {
+  __shared__ uint32_t best[kBucketRange];
+  const int buckets = 1 << b.log_buckets;
+  const uint32_t range = (b.n_nodes + uint32_t(buckets) - 1) >> b.log_buckets;  // <= kBucketRange by the plan
+  const uint32_t pos_begin = uint32_t(h.pos_base), pos_end = uint32_t(h.pos_base + h.len_max);
+  for (int bucket = blockIdx.x; bucket < buckets; bucket += gridDim.x) {
+    int64_t begin = b.start[bucket], end = b.start[bucket + 1];
+    if (begin < 0) begin = 0;
+    if (end > b.units_max) end = b.units_max;
+    // a thread's first kKept items stay in registers for the second pass (a bucket of the usual
+    // size is then read once), and are requested before the LDS array is cleared
+    constexpr int kKept = 8;
+    uint2 kept[kKept];
+#pragma unroll
+    for (int r = 0; r < kKept; ++r) {
+      const int64_t j = begin + threadIdx.x + int64_t(r) * kBlock;
+      kept[r] = j < end ? b.items[j] : make_uint2(0u, 0u);
+    }
+    for (uint32_t j = threadIdx.x; j < range && j < uint32_t(kBucketRange); j += kBlock) best[j] = 0xffffffffu;
+    __syncthreads();
+    for (int64_t j = begin + threadIdx.x, r = 0; j < end; j += kBlock, ++r) {
+      uint2 it = make_uint2(0u, 0u);
+      if (r < kKept) {
+#pragma unroll
+        for (int q = 0; q < kKept; ++q) if (q == r) it = kept[q];
+      } else {
+        it = b.items[j];
+      }
+      const uint32_t at = it.x >> b.log_buckets;
+      if (at < range && at < uint32_t(kBucketRange)) atomicMin(&best[at], it.y);
+    }
+    __syncthreads();
+    for (int64_t j = begin + threadIdx.x, r = 0; j < end; j += kBlock, ++r) {
+      uint2 it = make_uint2(0u, 0u);
+      if (r < kKept) {
+#pragma unroll
+        for (int q = 0; q < kKept; ++q) if (q == r) it = kept[q];
+      } else {
+        it = b.items[j];
+      }
+      const uint32_t at = it.x >> b.log_buckets;
+      if (it.y < pos_begin || it.y >= pos_end || at >= range || at >= uint32_t(kBucketRange)) continue;  // a frontier id
+      const uint32_t least = best[at];  // first occurrences keep the word the fill gave them
+      if (least != it.y) h.slot[it.y] = least < pos_begin ? (least | kRankBit) : least;
+    }
+    __syncthreads();
+  }
+}
+
 // One virtual block of the flag launch: 1024 padded positions.
 template <typename IdT, typename TableT, bool EARLY>
 __device__ __forceinline__ void flag_tile(const Hop& h, int64_t tile, const TableT& table) {
@@ -697,7 +989,14 @@ struct Plan {
   uint32_t capacity = 0;     // hash table slots (one table for all hops)
   size_t table_bytes = 0;    // 0 for the direct table
   bool weighted = false;     // picks by edge weight: per-hop queues for long rows
+  bool bucketed = false;     // the last hop finds its first occurrences by the bucketed pass
+  bool bucket_space = false; // the workspace has room for that pass
+  int32_t log_buckets = 0;
+  uint32_t n_nodes = 0;
 };
+
+// units (frontier ids + padded positions) the bucketed pass of the last hop handles at most
+inline int64_t bucket_units_max(const Plan& p) { return p.s_max[p.n_hops]; }
 
 dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, int32_t id_bytes,
                      int64_t n_nodes, bool have_node_table, Plan* p) {
@@ -716,10 +1015,23 @@ dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, in
     DGS_REQUIRE(p->s_max[h + 1] <= kMaxPositions, DGS_ERR_UNSUPPORTED,
                 "sample_blocks: worst-case frontier of hop %d exceeds 2^30 ids", h);
   }
+  // room for the bucketed pass whenever its size is bounded (whether it runs is decided below)
+  p->bucket_space = n_hops >= 2 && bucket_units_max(*p) <= kBucketedMaxUnits;
   if (have_node_table) {
     DGS_REQUIRE(n_nodes >= 0 && n_nodes < 0x7fffffffLL, DGS_ERR_UNSUPPORTED,
                 "sample_blocks: a node table needs fewer than 2^31 nodes (have %lld)", (long long)n_nodes);
     p->kind = TableKind::kDirect;
+    // the bucketed pass: slot words are ids (the direct table's), ids fit the LDS arrays, and the
+    // hop is large enough for its four extra launches to cost less than the atomics they replace
+    // (test hook: 1 never, 2 whatever the size)
+    const int64_t mode = debug_option(DGS_DEBUG_SAMPLER_BUCKETED);
+    const bool large = p->nnz_max[n_hops - 1] >= kBucketedMinPicks;
+    p->bucketed = p->bucket_space && n_nodes >= 1 && n_nodes <= kBucketedMaxNodes && fanouts[n_hops - 1] >= 1 &&
+                  mode != 1 && (large || mode == 2);
+    int log_b = 0;
+    while ((1 << log_b) < kMinBuckets || (int64_t(kBucketRange) << log_b) < n_nodes) ++log_b;
+    p->log_buckets = log_b;
+    p->n_nodes = uint32_t(n_nodes);
   } else {
     // ids fit the packed slot when every node id is below 2^32 - 1
     p->kind = id_bytes == 4 || (n_nodes >= 0 && n_nodes < 0xffffffffLL) ? TableKind::kPacked : TableKind::kSplit;
@@ -732,7 +1044,8 @@ dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, in
 }
 
 // Lays the workspace out; with base == nullptr only the size is computed.
-size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void** table) {
+size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void** table,
+              Buckets* buckets = nullptr) {
   Carver c(base);
   char* t = c.take<char>(p.table_bytes);
   if (table) *table = t;
@@ -765,8 +1078,22 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
     v.len_max = int64_t(len);
     v.k = int32_t(fanouts[h]);
     v.index = h;
+    v.bucketed = p.bucketed && h == p.n_hops - 1;
     if (hops) hops[h] = v;
     pos_base += int64_t(len);
+  }
+  if (p.bucket_space) {
+    Buckets b{};
+    b.units_max = bucket_units_max(p);
+    b.front_tiles = int32_t((p.s_max[p.n_hops - 1] + kBucketTile - 1) / kBucketTile);
+    b.tiles_max = b.front_tiles + int32_t((p.nnz_max[p.n_hops - 1] + kBucketTile - 1) / kBucketTile);
+    b.items = c.take<uint2>(size_t(b.units_max));
+    b.hist = c.take<int>(size_t(b.tiles_max) * kMaxBuckets);
+    b.total = c.take<int>(kMaxBuckets);
+    b.start = c.take<int>(kMaxBuckets + 1);
+    b.log_buckets = p.log_buckets;
+    b.n_nodes = p.n_nodes;
+    if (buckets) *buckets = b;
   }
   return c.used + 256;
 }
@@ -812,7 +1139,7 @@ dgs_status launch_fill_weighted(const Hop& cur, const Hop& prev, int64_t relabel
 }
 
 template <typename IdT, typename PtrT, typename TableT>
-dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_view& indptr,
+dgs_status run_blocks(const Plan& p, Hop* hops, const Buckets& buckets, const TableT& table, const dgs_view& indptr,
                       const dgs_view& indices, const dgs_view* probs, bool replace, uint64_t rng_seed,
                       void** sizes_ticket, hipStream_t st) {
   if (p.weighted) {  // the long-row queues of all hops start empty (their counters are one array, hop 0's first)
@@ -842,6 +1169,19 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
     else if (cur.k <= 32) launch_fill<IdT, PtrT, TableT, 32>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     else launch_fill<IdT, PtrT, TableT, 64>(cur, prev, surplus, clear_begin, clear_n16, table, indptr, indices, replace, rng_seed, st);
     DGS_LAUNCH_CHECK();
+
+    if (cur.bucketed) {  // the picks' slot words hold ids so far: group them and find the first occurrences
+      const int n_buckets = 1 << buckets.log_buckets;
+      const uint32_t tile_grid = capped_grid(buckets.tiles_max);
+      hipLaunchKernelGGL(bucket_count_kernel<IdT>, dim3(tile_grid), dim3(kBlock), 0, st, cur, buckets);
+      DGS_LAUNCH_CHECK();
+      hipLaunchKernelGGL(bucket_scan_kernel, dim3(uint32_t(n_buckets / 32)), dim3(1024), 0, st, cur, buckets);
+      DGS_LAUNCH_CHECK();
+      hipLaunchKernelGGL(bucket_scatter_kernel<IdT>, dim3(tile_grid), dim3(kBlock), 0, st, cur, buckets);
+      DGS_LAUNCH_CHECK();
+      hipLaunchKernelGGL(bucket_first_kernel, dim3(capped_grid(n_buckets)), dim3(kBlock), 0, st, cur, buckets);
+      DGS_LAUNCH_CHECK();
+    }
 
     const int64_t len_max = (h == 0 ? cur.s_max : 0) + cur.s_max * cur.k;
     const int64_t pos_tiles = (len_max + kPosTile - 1) / kPosTile;
@@ -890,20 +1230,20 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const TableT& table, const dgs_v
 }
 
 template <typename IdT, typename PtrT>
-dgs_status run_blocks_table(const Plan& p, Hop* hops, void* hash_table, void* node_table, uint32_t epoch,
-                            const dgs_view& indptr, const dgs_view& indices, const dgs_view* probs, bool replace,
-                            uint64_t rng_seed, void** sizes_ticket, hipStream_t st) {
+dgs_status run_blocks_table(const Plan& p, Hop* hops, const Buckets& buckets, void* hash_table, void* node_table,
+                            uint32_t epoch, const dgs_view& indptr, const dgs_view& indices, const dgs_view* probs,
+                            bool replace, uint64_t rng_seed, void** sizes_ticket, hipStream_t st) {
   if (p.kind == TableKind::kDirect)
-    return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, DirectTable<IdT>(node_table, epoch, uint32_t(indptr.total - 1)),
+    return run_blocks<IdT, PtrT, DirectTable<IdT>>(p, hops, buckets, DirectTable<IdT>(node_table, epoch, uint32_t(indptr.total - 1)),
                                                    indptr, indices, probs, replace, rng_seed, sizes_ticket, st);
   const int64_t n16 = int64_t(p.table_bytes / 16);
   hipLaunchKernelGGL(clear_kernel, dim3(capped_grid((n16 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                      static_cast<uint4*>(hash_table), n16);
   DGS_LAUNCH_CHECK();
   if (p.kind == TableKind::kPacked)
-    return run_blocks<IdT, PtrT, Table<IdT, true>>(p, hops, Table<IdT, true>(hash_table, p.capacity), indptr,
+    return run_blocks<IdT, PtrT, Table<IdT, true>>(p, hops, buckets, Table<IdT, true>(hash_table, p.capacity), indptr,
                                                    indices, probs, replace, rng_seed, sizes_ticket, st);
-  return run_blocks<IdT, PtrT, Table<IdT, false>>(p, hops, Table<IdT, false>(hash_table, p.capacity), indptr,
+  return run_blocks<IdT, PtrT, Table<IdT, false>>(p, hops, buckets, Table<IdT, false>(hash_table, p.capacity), indptr,
                                                   indices, probs, replace, rng_seed, sizes_ticket, st);
 }
 
@@ -993,7 +1333,8 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
               "sample_blocks: workspace must be 256-byte aligned");
   Hop hops[DGS_MAX_HOPS];
   void* hash_table = nullptr;
-  layout(p, fanouts, workspace, hops, &hash_table);
+  Buckets buckets{};
+  layout(p, fanouts, workspace, hops, &hash_table, &buckets);
   for (int h = 0; h < n_hops; ++h) {
     Hop& t = hops[h];
     DGS_REQUIRE(p.nnz_max[h] == 0 || (outs[h].src_local && outs[h].dst_local), DGS_ERR_INVALID,
@@ -1017,11 +1358,11 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
   const bool rep = replace != 0;
   if (id_bytes == 8)
     return indptr.elem_bytes == 8
-               ? run_blocks_table<int64_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st)
-               : run_blocks_table<int64_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st);
+               ? run_blocks_table<int64_t, int64_t>(p, hops, buckets, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st)
+               : run_blocks_table<int64_t, int32_t>(p, hops, buckets, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st);
   return indptr.elem_bytes == 8
-             ? run_blocks_table<int32_t, int64_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st)
-             : run_blocks_table<int32_t, int32_t>(p, hops, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st);
+             ? run_blocks_table<int32_t, int64_t>(p, hops, buckets, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st)
+             : run_blocks_table<int32_t, int32_t>(p, hops, buckets, hash_table, node_table, node_table_epoch, indptr, indices, probs, rep, rng_seed, sizes_ticket, st);
 }
 }  // namespace
 

@@ -25,7 +25,7 @@ void set_error(const char* fmt, ...) {
 // HBM bytes held by live stores (upstream src/cuda_context.h:11-38, made atomic).
 static std::atomic<int64_t> g_allocated{0};
 
-constexpr int kDebugOptions = 4;
+constexpr int kDebugOptions = 5;
 static std::atomic<int64_t> g_debug[kDebugOptions];
 int64_t debug_option(int32_t option) {
   return option >= 0 && option < kDebugOptions ? g_debug[option].load(std::memory_order_relaxed) : 0;

@@ -55,12 +55,17 @@ int dgs_abi_version(void);
  *                                reserves, 0..65536: bounds how many of its blocks share a CU
  *   DGS_DEBUG_SAMPLER_GRID_CAP   > 0: most blocks a launch of dgs_sample_blocks may have
  *                                (larger launches loop over their blocks)
+ *   DGS_DEBUG_SAMPLER_BUCKETED   how the last hop of dgs_sample_blocks[_weighted] with a node
+ *                                table finds its first occurrences: 0 by size (the bucketed LDS
+ *                                pass for a large hop, the table's atomics otherwise), 1 always
+ *                                the table, 2 the bucketed pass whatever the size
  */
 enum {
   DGS_DEBUG_FORCE_SPLIT_TABLE = 0,
   DGS_DEBUG_WEIGHTED_GROUP = 1,
   DGS_DEBUG_GATHER_LDS_BYTES = 2,
-  DGS_DEBUG_SAMPLER_GRID_CAP = 3
+  DGS_DEBUG_SAMPLER_GRID_CAP = 3,
+  DGS_DEBUG_SAMPLER_BUCKETED = 4
 };
 dgs_status dgs_debug_set(int32_t option, int64_t value);
 

@@ -22,3 +22,13 @@ def powerlaw_graph(rng, n, mean_deg, max_deg, zero_frac=0.02, id_dtype=np.int64,
 def np_unique_first(x):
     u, first = np.unique(x, return_index=True)
     return u[np.argsort(first, kind="stable")]
+
+
+LAST_HOP_MODES = ["last hop by size", "last hop bucketed"]
+
+
+def set_last_hop_mode(pkg, mode):
+    """How the fused sampler's last hop finds its first occurrences in this test: by size (small
+    test inputs then take the node table's atomics) or always through the bucketed LDS pass."""
+    capi = pkg.capi
+    capi.check(capi.lib.dgs_debug_set(capi.DEBUG_SAMPLER_BUCKETED, 2 if mode == LAST_HOP_MODES[1] else 0))

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import load_pkg, powerlaw_graph
+from helpers import load_pkg, powerlaw_graph, LAST_HOP_MODES, set_last_hop_mode
 
 pytestmark = pytest.mark.gpu
 
@@ -13,6 +13,13 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def pkg():
     return load_pkg()
+
+
+@pytest.fixture(params=LAST_HOP_MODES)
+def last_hop(request, pkg):
+    set_last_hop_mode(pkg, request.param)
+    yield request.param
+    set_last_hop_mode(pkg, LAST_HOP_MODES[0])
 
 
 def _dev(a):
@@ -29,7 +36,7 @@ def _same_blocks(got, want):
 
 
 @pytest.mark.parametrize("sweep", [2024, 7])
-def test_random_cases_match_the_oracle(pkg, oracle, sweep):
+def test_random_cases_match_the_oracle(pkg, oracle, sweep, last_hop):
     rng = np.random.default_rng(sweep)
     big = 1 << 40
     for case in range(40):

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import load_pkg, np_unique_first, powerlaw_graph
+from helpers import load_pkg, np_unique_first, powerlaw_graph, LAST_HOP_MODES, set_last_hop_mode
 
 pytestmark = pytest.mark.gpu
 
@@ -13,6 +13,13 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def pkg():
     return load_pkg()
+
+
+@pytest.fixture(params=LAST_HOP_MODES)
+def last_hop(request, pkg):
+    set_last_hop_mode(pkg, request.param)
+    yield request.param
+    set_last_hop_mode(pkg, LAST_HOP_MODES[0])
 
 
 def _dev(a):
@@ -110,7 +117,7 @@ def test_sample_any_fanout_without_replacement(pkg, oracle, id_dtype):
     assert r.numel() == sum(min(int(deg[s]), 3000) for s in seeds)
 
 
-def test_seed_ids_outside_the_graph_are_refused(pkg, oracle, graph):
+def test_seed_ids_outside_the_graph_are_refused(pkg, oracle, graph, last_hop):
     # a seed id is checked before it addresses indptr: its row emits nothing, the call is flagged,
     # the operators raise
     capi = pkg.capi
@@ -144,7 +151,7 @@ def test_seed_ids_outside_the_graph_are_refused(pkg, oracle, graph):
     assert flags[0] == 2 and flags[1] == 0
 
 
-def test_neighbour_ids_outside_the_graph_are_refused(pkg):
+def test_neighbour_ids_outside_the_graph_are_refused(pkg, last_hop):
     # a graph whose edge array holds an id that is no node: with the direct node table the id would
     # address the table, so it is checked first and the call raises
     n = 1000
@@ -167,7 +174,7 @@ def test_neighbour_ids_outside_the_graph_are_refused(pkg):
         pkg.ChunkTensorSampler([8], ip_ct, ix_ct).sample_blocks(None, torch.tensor([30]))
 
 
-def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph):
+def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph, last_hop):
     # when the worst-case feature buffer exceeds the cap the gather goes into the largest buffer the
     # cap allows, and a frontier that does not fit even that is gathered once its size is known,
     # into exactly that many rows
@@ -208,7 +215,7 @@ def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph):
     assert results[1][2] < results[0][2]
 
 
-def test_samplers_with_their_own_generator(pkg, oracle, graph):
+def test_samplers_with_their_own_generator(pkg, oracle, graph, last_hop):
     # a sampler made with seed= draws batch b from its own streams whatever other threads do
     import threading
     indptr, indices = graph
@@ -401,7 +408,7 @@ def _check_blocks(blocks_gpu, o_blocks):
 @pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int64, np.int64), (np.int32, np.int64), (np.int32, np.int32)])
 @pytest.mark.parametrize("fanouts,replace", [([15, 10, 5], False), ([5], False), ([3, 0, 4], False), ([64, 2], False),
                                              ([7, 9], True), ([20, 15, 10], False)])
-def test_fused_sample_blocks_parity(pkg, oracle, id_dtype, ptr_dtype, fanouts, replace):
+def test_fused_sample_blocks_parity(pkg, oracle, id_dtype, ptr_dtype, fanouts, replace, last_hop):
     rng = np.random.default_rng(len(fanouts) * 31 + fanouts[0])
     indptr, indices = powerlaw_graph(rng, 30000, 12, 2000, id_dtype=id_dtype, ptr_dtype=ptr_dtype)
     t_ip, t_ix = torch.from_numpy(indptr), torch.from_numpy(indices)
@@ -427,7 +434,7 @@ def test_fused_sample_blocks_parity(pkg, oracle, id_dtype, ptr_dtype, fanouts, r
         assert torch.equal(x.cpu(), feats[torch.from_numpy(o_frontier).long()])
 
 
-def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph):
+def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph, last_hop):
     capi = pkg.capi
     indptr, indices = graph
     ip, ix = _dev(indptr), _dev(indices)
@@ -462,7 +469,7 @@ def test_fused_sample_blocks_c_abi_and_split_table(pkg, oracle, graph):
     assert capi.lib.dgs_sample_blocks_plan(10, fan, 1, out, out) == capi.DGS_ERR_UNSUPPORTED
 
 
-def test_fused_long_tile_lists(pkg, oracle):
+def test_fused_long_tile_lists(pkg, oracle, last_hop):
     # > 2048 position tiles and > 2048 row tiles in the last hop: the separate scan launches
     rng = np.random.default_rng(5)
     indptr, indices = powerlaw_graph(rng, 1_000_000, 6, 200, zero_frac=0.1)
@@ -480,7 +487,7 @@ def test_fused_long_tile_lists(pkg, oracle):
     assert 60_000 * 41 > 2048 * 256 and blocks[0].num_dst > 200_000
 
 
-def test_host_seeds_are_accepted(pkg, oracle, graph):
+def test_host_seeds_are_accepted(pkg, oracle, graph, last_hop):
     # upstream's sampler receives host-side seed_nodes and uploads them itself
     indptr, indices = graph
     ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
@@ -595,7 +602,7 @@ def test_host_threads_sampling_from_one_graph_on_one_stream(pkg, oracle):
 
 
 @pytest.mark.parametrize("native_loop", [True, False])
-def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph, native_loop):
+def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph, native_loop, last_hop):
     # BatchPipeline: batches in flight on its own streams, results in submission order, usable on
     # the caller's stream at once (reduced there right away, buffers dropped while later batches
     # are still running), host and device seeds, uniform and weighted samplers; with the
@@ -647,7 +654,7 @@ def test_batch_pipeline_hands_out_usable_batches(pkg, oracle, graph, native_loop
 
 
 @pytest.mark.parametrize("cap", [1, 7, 300])
-def test_fused_sampler_under_a_small_grid_cap(pkg, oracle, graph, cap, request):
+def test_fused_sampler_under_a_small_grid_cap(pkg, oracle, graph, cap, request, last_hop):
     # every launch of the fused sampler loops over its blocks when there are more than the cap:
     # the results do not depend on the cap
     capi = pkg.capi

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import load_pkg, powerlaw_graph
+from helpers import load_pkg, powerlaw_graph, LAST_HOP_MODES, set_last_hop_mode
 
 pytestmark = pytest.mark.gpu
 
@@ -13,6 +13,13 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def pkg():
     return load_pkg()
+
+
+@pytest.fixture(params=LAST_HOP_MODES)
+def last_hop(request, pkg):
+    set_last_hop_mode(pkg, request.param)
+    yield request.param
+    set_last_hop_mode(pkg, LAST_HOP_MODES[0])
 
 
 def _dev(a):
@@ -173,7 +180,7 @@ def test_weighted_inclusion_frequencies(pkg):
 
 
 @pytest.mark.parametrize("replace", [False, True])
-def test_weighted_sampler_loop(pkg, oracle, graph, replace):
+def test_weighted_sampler_loop(pkg, oracle, graph, replace, last_hop):
     # ChunkTensorSampler with chunk_probs: the upstream loop with weighted picks in every hop, through
     # the fused driver (default), the per-hop operators, and with batches in flight on two streams
     indptr, indices, probs = graph
@@ -221,7 +228,7 @@ def test_weighted_sampler_loop(pkg, oracle, graph, replace):
     torch.cuda.synchronize()
 
 
-def test_weighted_fused_long_rows_and_wide_fanout(pkg, oracle):
+def test_weighted_fused_long_rows_and_wide_fanout(pkg, oracle, last_hop):
     # rows longer than a wave's share (block-per-row launch inside the fused driver), fanout 64,
     # rows without positive weights, int32 ids with int64 offsets
     rng = np.random.default_rng(6)
@@ -249,7 +256,7 @@ def test_weighted_fused_long_rows_and_wide_fanout(pkg, oracle):
             assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
 
 
-def test_weighted_rows_that_the_key_halves_leave_open(pkg, oracle):
+def test_weighted_rows_that_the_key_halves_leave_open(pkg, oracle, last_hop):
     # the race first compares the upper 32 bits of the keys and repeats a row on full keys when
     # those tie where it matters: infinite weights (all keys 0), fewer usable weights than picks
     # (the unusable ones tie), on rows served by a lane group, by a wave and by a whole block;
@@ -287,7 +294,7 @@ def test_weighted_rows_that_the_key_halves_leave_open(pkg, oracle):
             assert np.array_equal(_np(g.src_local), w[0]) and np.array_equal(_np(g.dst_local), w[1])
 
 
-def test_weighted_fused_on_more_streams_than_node_tables(pkg, oracle, graph):
+def test_weighted_fused_on_more_streams_than_node_tables(pkg, oracle, graph, last_hop):
     # a graph keeps at most four node tables, one per stream; a fifth and sixth stream take over a
     # table whose stream is idle, or run on a hash table in their workspace: same batches either way
     indptr, indices, probs = graph
@@ -312,7 +319,7 @@ def test_weighted_fused_on_more_streams_than_node_tables(pkg, oracle, graph):
 
 
 @pytest.mark.parametrize("id_dtype", [np.int64, np.int32])
-def test_weighted_fused_c_abi_on_every_table_kind(pkg, oracle, graph, id_dtype):
+def test_weighted_fused_c_abi_on_every_table_kind(pkg, oracle, graph, id_dtype, last_hop):
     # the weighted multi-hop driver through the C ABI: hash table in the workspace (packed slots,
     # then id + value arrays), then the persistent node table; every hop picks by weight
     capi = pkg.capi
