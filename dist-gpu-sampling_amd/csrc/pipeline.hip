@@ -1303,6 +1303,9 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
                 "sample_blocks_weighted: %lld weights of %d bytes for %lld edges (float32, one per edge)",
                 (long long)probs->total, probs->elem_bytes, (long long)indices.total);
     p.weighted = true;
+    // weighted picks: the fill is bound by the races, not by its atomics, and the bucketed pass only
+    // lengthens the batch (measured: + 25 us alone, the same step with four batches in flight)
+    if (debug_option(DGS_DEBUG_SAMPLER_BUCKETED) != 2) p.bucketed = false;
   }
   const size_t need = probs != nullptr ? dgs_sample_blocks_weighted_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes)
                                        : dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes);

@@ -57,8 +57,9 @@ int dgs_abi_version(void);
  *                                (larger launches loop over their blocks)
  *   DGS_DEBUG_SAMPLER_BUCKETED   how the last hop of dgs_sample_blocks[_weighted] with a node
  *                                table finds its first occurrences: 0 by size (the bucketed LDS
- *                                pass for a large hop, the table's atomics otherwise), 1 always
- *                                the table, 2 the bucketed pass whatever the size
+ *                                pass for a large hop of uniform picks, the table's atomics
+ *                                otherwise), 1 always the table, 2 the bucketed pass whatever
+ *                                the size and the kind of picks
  */
 enum {
   DGS_DEBUG_FORCE_SPLIT_TABLE = 0,
