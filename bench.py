@@ -452,7 +452,7 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
     ap.add_argument("--inflight", type=int, default=None,
                     help="batches in flight on as many streams (1 = one blocking call per batch); default 4 for "
-                         "c0/c1/c1w and 2 for the large workloads, whose batches are long enough for two to fill the GPU")
+                         "c0/c1/c1w and 3 for the large workloads (measured best of 2..4 on each)")
     ap.add_argument("--gather-buffer-cap-gib", type=float, default=None,
                     help="largest feature buffer the fused operator allocates ahead of a batch's sizes "
                          "(the library's default when not given)")
@@ -470,7 +470,7 @@ def main():
     dgs = importlib.import_module("dist-gpu-sampling_amd")
     torch.cuda.set_device(0)
     if args.inflight is None:
-        args.inflight = 2 if args.workload in LARGE else 4
+        args.inflight = 3 if args.workload in LARGE else 4
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
     if args.workload in LARGE:
