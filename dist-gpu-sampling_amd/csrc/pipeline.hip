@@ -18,8 +18,13 @@
 //     tells whether it is (so far) the smallest of its id and which position it displaced;
 //     the displaced one is marked lost.  "First occurrence" is then decided from two
 //     streamed arrays, without a second random read of the table.  Random 8-byte
-//     accesses are what bounds these kernels (about 42 G transactions/s on MI355X), so
-//     a hop costs two of them per pick: the indices read and the table atomic.
+//     accesses are what bounds these kernels (on MI355X: loads 71 G/s, atomics 26.7 G/s, every
+//     device-scope atomic being executed at the memory side), and a hop costs two of them
+//     per pick: the indices read and the table atomic.
+//
+// A large last hop of uniform picks does without the table altogether (see Buckets below): its
+// fill records the picked ids, four launches group them by id and take the smallest position of
+// every id in LDS, and flag / compact / relabel read the same slot words as on the table path.
 //
 // Critical path per hop (3 launches): fill -> flag -> compact.
 //   fill     G lanes per seed row (G = 8..64): indptr pair, picks by the dgs-philox-1
