@@ -650,13 +650,34 @@ class PendingBlocks : public torch::CustomClassHolder {
     p->src_.resize(hops);
     p->dst_.resize(hops);
     std::vector<dgs_block_out> outs(hops);
-    p->all_ = torch::empty({seeds_max[hops]}, opt);  // every hop's frontier is a prefix of it
+    // The id outputs of the batch (the frontier array, of which every hop's frontier is a prefix,
+    // and the edge lists) and its device-side lengths are pieces of ONE allocation: a dozen
+    // tensors cost a dozen trips to the allocator here, and as many stream records and events
+    // again when the batch is handed to another stream and dropped there.
+    int64_t carved = 0;
+    const auto piece = [&carved](int64_t bytes) {
+      const int64_t at = carved;
+      carved += (bytes + 255) / 256 * 256;
+      return at;
+    };
+    const int64_t all_at = piece(seeds_max[hops] * w);
+    std::vector<int64_t> src_at(hops), dst_at(hops);
     for (int h = 0; h < hops; ++h) {
-      p->src_[h] = torch::empty({edges_max[h]}, opt);
-      p->dst_[h] = torch::empty({edges_max[h]}, opt);
+      src_at[h] = piece(edges_max[h] * w);
+      dst_at[h] = piece(edges_max[h] * w);
+    }
+    const int64_t sizes_at = piece(n_sizes * 8);
+    p->ids_ = device_bytes(static_cast<size_t>(carved), dev);
+    const auto ids_of = [&](int64_t at, int64_t count) {
+      return p->ids_.narrow(0, at, count * w).view(p->seeds_.scalar_type());
+    };
+    p->all_ = ids_of(all_at, seeds_max[hops]);
+    for (int h = 0; h < hops; ++h) {
+      p->src_[h] = ids_of(src_at[h], edges_max[h]);
+      p->dst_[h] = ids_of(dst_at[h], edges_max[h]);
       outs[h] = dgs_block_out{p->src_[h].data_ptr(), p->dst_[h].data_ptr()};
     }
-    torch::Tensor sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
+    torch::Tensor sizes_dev = p->ids_.narrow(0, sizes_at, n_sizes * 8).view(torch::kInt64);
     const size_t ws_bytes = probs ? dgs_sample_blocks_weighted_workspace_bytes(n, fanouts.data(), hops, w)
                                   : dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
     torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
@@ -705,11 +726,9 @@ class PendingBlocks : public torch::CustomClassHolder {
   // stream (so that the allocator does not hand them out again while that stream still reads them).
   c10::Stream stream() const { return stream_; }
   void RecordStream(const c10::Stream& consumer) {
-    for (const torch::Tensor* t : {&seeds_, &all_, &x_})
+    // (the frontier and the edge lists are views of ids_)
+    for (const torch::Tensor* t : {&seeds_, &ids_, &x_})
       if (t->defined() && t->is_cuda()) t->record_stream(consumer);
-    for (const auto& list : {&src_, &dst_})
-      for (const torch::Tensor& t : *list)
-        if (t.defined() && t.is_cuda()) t.record_stream(consumer);
   }
 
  private:
@@ -717,7 +736,7 @@ class PendingBlocks : public torch::CustomClassHolder {
   bool finished_ = false;
   void* ticket_ = nullptr;
   dgs_status gather_status_ = DGS_OK;
-  torch::Tensor pinned_, seeds_, all_, x_;
+  torch::Tensor pinned_, seeds_, ids_, all_, x_;  // ids_: the allocation all_, src_ and dst_ are views of
   torch::Tensor staged_seeds_;  // pinned copy of host seeds, alive until the batch is finished
   std::vector<torch::Tensor> src_, dst_;
   // the feature gather: rows of the buffer it was enqueued into (-1: none), and what a second,
