@@ -719,3 +719,40 @@ def test_pipeline_streams_do_not_share_a_hardware_queue(pkg):
                 assert pkg.streams_overlap(chosen[i], chosen[j])
     assert not pkg.streams_overlap(chosen[0], chosen[0])  # one stream runs in order
     del others
+
+
+def test_batch_loop_of_the_extension_directly(pkg, oracle, graph):
+    # torch.classes.dgs_classes.BatchLoop without the Python pipeline around it: batches come back in
+    # the order they were pushed, whatever mix of host and device seeds; nothing is pending after
+    # the last pop; a closed loop refuses more
+    indptr, indices = graph
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    feats = torch.randn((20000, 16))
+    x_ct = pkg.create_chunktensor(feats, 1, big)
+    streams = pkg.pipeline_streams(2)
+    triples = []
+    for st in streams:
+        triples += [st.stream_id, st.device_index, st.device_type]
+    loop = torch.classes.dgs_classes.BatchLoop(ip_ct, ix_ct, None, [4, 6], False, x_ct, triples, True, True, [])
+    rng = np.random.default_rng(3)
+    batches = [rng.integers(0, 20000, size=300).astype(np.int64) for _ in range(5)]
+    pkg.set_rng_state(5, 100)
+    for i, b in enumerate(batches):
+        loop._CAPI_push(torch.from_numpy(b) if i % 2 else _dev(b), i < 2)
+    assert loop._CAPI_pending() == 5
+    for i, b in enumerate(batches):
+        frontiers, srcs, dsts, x, seeds_dev = loop._CAPI_pop()
+        want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, [6, 4], False, 5, 100 + 2 * i)
+        assert np.array_equal(_np(frontiers[-1]), want_f) and np.array_equal(_np(seeds_dev), b)
+        for h, wb in enumerate(reversed(want_blocks)):
+            assert np.array_equal(_np(srcs[h]), wb[0]) and np.array_equal(_np(dsts[h]), wb[1])
+        assert torch.equal(x.cpu(), feats[torch.from_numpy(want_f)])
+    assert loop._CAPI_pending() == 0
+    with pytest.raises(RuntimeError, match="nothing to pop"):
+        loop._CAPI_pop()
+    loop._CAPI_close()
+    loop._CAPI_close()  # closing twice is fine
+    with pytest.raises(RuntimeError, match="closed"):
+        loop._CAPI_push(_dev(batches[0]), False)
