@@ -764,7 +764,7 @@ class BatchLoop : public torch::CustomClassHolder {
         hand_over_(hand_over), turn_(gathers_in_turn), rng_(std::move(rng)) {
     TORCH_CHECK(!streams.empty() && streams.size() % 3 == 0,
                 "BatchLoop: streams are (stream_id, device_index, device_type) triples");
-    TORCH_CHECK(rng_.empty() || rng_.size() == 2, "BatchLoop: rng is [] or [seed, first stream]");
+    TORCH_CHECK(rng_.size() <= 1, "BatchLoop: rng is [] (the process-wide generator) or [seed] (the caller's own)");
     for (size_t i = 0; i < streams.size(); i += 3)
       streams_.push_back(c10::Stream::unpack3(streams[i], static_cast<c10::DeviceIndex>(streams[i + 1]),
                                                static_cast<c10::DeviceType>(streams[i + 2])));
@@ -777,9 +777,15 @@ class BatchLoop : public torch::CustomClassHolder {
   // moment (they may have been made there just now); host seeds need nothing, unless the caller
   // asks for the same order (behind_caller: the first batches of an iteration, say, behind the
   // set-up that precedes it).
-  void Push(torch::Tensor seeds, bool behind_caller) {
+  // `first_stream`: with a generator of the caller's own (rng = [seed]), the stream of the batch's
+  // first hop, which the caller counts (a sampler numbers its batches in submission order);
+  // ignored otherwise.
+  void Push(torch::Tensor seeds, bool behind_caller, int64_t first_stream) {
     Item item;
     item.seeds = std::move(seeds);
+    item.first_stream = first_stream;
+    TORCH_CHECK(rng_.empty() || (first_stream >= 0 && first_stream <= 0xffffffffLL),
+                "BatchLoop: a generator of the caller's own needs the batch's first stream, 0..2^32-1");
     if (item.seeds.is_cuda() || behind_caller) {
       void* st = current_stream();
       int32_t idle = 0;
@@ -848,6 +854,7 @@ class BatchLoop : public torch::CustomClassHolder {
   struct Item {
     torch::Tensor seeds;
     void* seeds_ready = nullptr;  // ticket on the pushing thread's stream, or null
+    int64_t first_stream = -1;
     c10::intrusive_ptr<PendingBlocks> batch;
     std::string error;
   };
@@ -882,9 +889,7 @@ class BatchLoop : public torch::CustomClassHolder {
         const bool turn = turn_ && features_ && n > 1;
         void* gather_after = turn && index > 0 ? done_[(index - 1) % (n + 1)] : nullptr;
         std::pair<uint64_t, uint32_t> own{0, 0};
-        if (!rng_.empty())
-          own = {static_cast<uint64_t>(rng_[0]),
-                 static_cast<uint32_t>(rng_[1] + index * static_cast<int64_t>(fanouts_.size()))};
+        if (!rng_.empty()) own = {static_cast<uint64_t>(rng_[0]), static_cast<uint32_t>(item.first_stream)};
         item.batch = PendingBlocks::Begin(item.seeds, indptr_, indices_, fanouts_, replace_, features_, probs_,
                                           rng_.empty() ? nullptr : &own, gather_after);
         if (turn) {

@@ -302,7 +302,7 @@ class BatchPipeline:
         while another iteration is using the one this pipeline would take."""
         smp = self.sampler
         key = (id(self.chunk_features), tuple(st.stream_id for st in self.streams), self.hand_over,
-               self.gathers_in_turn, tuple(smp.fanouts), smp.replace, id(smp.chunk_probs))
+               self.gathers_in_turn, tuple(smp.fanouts), smp.replace, id(smp.chunk_probs), smp.seed)
         entry = smp._loops.get(key)
         if entry is None:
             triples = []
@@ -310,7 +310,8 @@ class BatchPipeline:
                 triples += [st.stream_id, st.device_index, st.device_type]
             loop = torch.classes.dgs_classes.BatchLoop(
                 smp.chunk_indptr, smp.chunk_indices, smp.chunk_probs, list(reversed(smp.fanouts)), smp.replace,
-                self.chunk_features, triples, self.hand_over, self.gathers_in_turn, [])
+                self.chunk_features, triples, self.hand_over, self.gathers_in_turn,
+                [] if smp.seed is None else [smp.seed])
             # (the features are kept with the entry so that their id stays theirs)
             entry = smp._loops[key] = {"loop": loop, "busy": False, "features": self.chunk_features}
         if entry["busy"]:
@@ -323,6 +324,7 @@ class BatchPipeline:
         with_x = self.chunk_features is not None
         waiting = deque()
         pushed = 0
+        seeded = self.sampler.seed
 
         def take():
             frontiers, srcs, dsts, x, seeds_dev = loop._CAPI_pop()
@@ -335,7 +337,8 @@ class BatchPipeline:
             for seeds in seed_batches:
                 # the first batch on each stream goes behind what the caller's stream holds now,
                 # later ones only if their seeds are on the device (see the Python loop below)
-                loop._CAPI_push(seeds, pushed < n)
+                # (a sampler with its own generator numbers its batches here, in submission order)
+                loop._CAPI_push(seeds, pushed < n, -1 if seeded is None else self.sampler._first_stream(None))
                 pushed += 1
                 waiting.append(seeds)
                 if len(waiting) >= n:
@@ -351,10 +354,9 @@ class BatchPipeline:
             entry["busy"] = False
 
     def __call__(self, seed_batches):
-        # (a sampler with its own generator counts its batches in Python, and a second iteration
-        # that starts while one is under way cannot share the first one's queue: both keep the
-        # Python loop)
-        if self.native_loop and self.sampler.fused and self.sampler.seed is None:
+        # (a second iteration that starts while one is under way cannot share the first one's
+        # queue: it keeps the Python loop)
+        if self.native_loop and self.sampler.fused:
             entry = self._native()
             if entry is not None:
                 yield from self._iterate_native(entry, seed_batches)

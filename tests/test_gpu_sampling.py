@@ -740,7 +740,7 @@ def test_batch_loop_of_the_extension_directly(pkg, oracle, graph):
     batches = [rng.integers(0, 20000, size=300).astype(np.int64) for _ in range(5)]
     pkg.set_rng_state(5, 100)
     for i, b in enumerate(batches):
-        loop._CAPI_push(torch.from_numpy(b) if i % 2 else _dev(b), i < 2)
+        loop._CAPI_push(torch.from_numpy(b) if i % 2 else _dev(b), i < 2, -1)
     assert loop._CAPI_pending() == 5
     for i, b in enumerate(batches):
         frontiers, srcs, dsts, x, seeds_dev = loop._CAPI_pop()
@@ -755,4 +755,31 @@ def test_batch_loop_of_the_extension_directly(pkg, oracle, graph):
     loop._CAPI_close()
     loop._CAPI_close()  # closing twice is fine
     with pytest.raises(RuntimeError, match="closed"):
-        loop._CAPI_push(_dev(batches[0]), False)
+        loop._CAPI_push(_dev(batches[0]), False, -1)
+
+
+@pytest.mark.parametrize("native_loop", [True, False])
+def test_batch_pipeline_with_a_sampler_that_has_its_own_generator(pkg, oracle, graph, native_loop):
+    # batch b of such a sampler draws from streams b * hops ... of its seed, in submission order,
+    # whichever loop begins the batches, and leaves the process-wide generator alone
+    indptr, indices = graph
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    fanouts = [5, 3]
+    rng = np.random.default_rng(21)
+    batches = [rng.integers(0, 20000, size=500).astype(np.int64) for _ in range(7)]
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, seed=4242)
+    pkg.set_rng_state(9, 9)
+    pipe = pkg.BatchPipeline(sampler, None, 3, native_loop=native_loop)
+    got = [(f.clone(), [(b.src_local.clone(), b.dst_local.clone()) for b in blocks])
+           for f, _, blocks in pipe([_dev(b) for b in batches[:4]])]
+    got += [(f.clone(), [(b.src_local.clone(), b.dst_local.clone()) for b in blocks])
+            for f, _, blocks in pipe([torch.from_numpy(b) for b in batches[4:]])]  # the count goes on
+    torch.cuda.synchronize()
+    for i, b in enumerate(batches):
+        want_f, _, want_blocks = oracle.sample_blocks(b, indptr, indices, fanouts, False, 4242, 2 * i)
+        assert np.array_equal(_np(got[i][0]), want_f), i
+        for (src, dst), wb in zip(got[i][1], want_blocks):
+            assert np.array_equal(_np(src), wb[0]) and np.array_equal(_np(dst), wb[1])
+    assert pkg.ops._CAPI_get_rng_state() == [9, 9]
