@@ -783,3 +783,35 @@ def test_batch_pipeline_with_a_sampler_that_has_its_own_generator(pkg, oracle, g
         for (src, dst), wb in zip(got[i][1], want_blocks):
             assert np.array_equal(_np(src), wb[0]) and np.array_equal(_np(dst), wb[1])
     assert pkg.ops._CAPI_get_rng_state() == [9, 9]
+
+
+@pytest.mark.parametrize("n_nodes", [1 << 24, (1 << 24) + 1])
+def test_bucketed_last_hop_at_its_largest_graph(pkg, oracle, n_nodes):
+    # 2^24 nodes is the most the bucketed pass takes (2048 buckets x 8192 ids in LDS); one node
+    # more and the hop stays on the table.  Ids from the very top of the range are picked and
+    # seeded, so the last LDS entries of the last buckets are in use.
+    rng = np.random.default_rng(n_nodes & 0xff)
+    deg = np.zeros(n_nodes, dtype=np.int64)
+    busy = np.concatenate([rng.integers(0, n_nodes, size=40000), np.arange(n_nodes - 3000, n_nodes)])
+    deg[busy] = rng.integers(1, 30, size=busy.size)
+    indptr = np.zeros(n_nodes + 1, dtype=np.int64)
+    np.cumsum(deg, out=indptr[1:])
+    pool = np.concatenate([busy, np.arange(n_nodes - 64, n_nodes), np.arange(64)])
+    indices = pool[rng.integers(0, pool.size, size=int(indptr[-1]))].astype(np.int64)
+    seeds = np.concatenate([busy[rng.integers(0, busy.size, size=1500)], np.arange(n_nodes - 20, n_nodes)]).astype(np.int64)
+    fanouts = [6, 5]
+    want_f, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, False, 31, 4)
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct)
+    set_last_hop_mode(pkg, LAST_HOP_MODES[1])
+    try:
+        pkg.set_rng_state(31, 4)
+        frontier, _, blocks = sampler.sample_blocks(None, _dev(seeds))
+    finally:
+        set_last_hop_mode(pkg, LAST_HOP_MODES[0])
+    assert np.array_equal(_np(frontier), want_f)
+    _check_blocks(blocks, want_blocks)
+    assert want_f.max() >= n_nodes - 20
+    del ip_ct, ix_ct, sampler
+    torch.cuda.empty_cache()
