@@ -143,29 +143,30 @@ __host__ __device__ __forceinline__ int relabel_groups(int k) { return (k + kRel
 // The atomicMin per pick is what a large hop costs most (every device-scope atomic executes at
 // the memory side: 26.7 G/s, 31 us for the 832 k picks of a 1024 x [5,10,15] batch, and as much
 // again while other batches share the GPU).  The last hop needs no table entry afterwards, so its
-// first occurrences can be found without the table: the picks, together with the ids the
-// frontier already holds, are grouped by the low bits of the id (count, column scan, scatter:
-// streamed reads and writes), and one block per group takes the smallest position of every id in
+// first occurrences can be found without the table.  The hop's units -- the ids the frontier
+// already holds (order value = rank) and the padded positions (order value = position, above
+// every rank) -- are cut into tiles of 4096; a block puts its tile's units in bucket order
+// (bucket = low bits of the id) and notes where every bucket's piece begins; then one block per
+// bucket walks that bucket's pieces in all tiles and takes the smallest order value of every id in
 // an LDS array indexed by the id's high bits.  A pick's slot word then says everything the later
-// stages need: first occurrence (id | kFirstBit), a repeat of an id the frontier held before
-// this hop (its rank | kRankBit: final, no further lookup), or a repeat of a pick of this hop
-// (that pick's position, whose rank the compaction records).  Same result as the table gives.
-constexpr int kBucketTile = 4096;                    // units (frontier ids, then pick positions) per count/scatter block
+// stages need: first occurrence (id | kFirstBit, as the fill left it), a repeat of an id the
+// frontier held before this hop (its rank | kRankBit: final, no further lookup), or a repeat of
+// a pick of this hop (that pick's position, whose rank the compaction records).  Same result as
+// the table gives.
+constexpr int kBucketTile = 4096;                    // units per tile
 constexpr int kBucketTileItems = kBucketTile / kBlock;
 constexpr int kMinBuckets = 512;
 constexpr int kMaxBuckets = 2048;
 constexpr int kBucketRange = 8192;                   // ids per bucket at most: 32 KB of LDS
+constexpr int kMaxBucketTiles = 2048;                // tiles a bucket's block can walk (its LDS index of them)
 constexpr int64_t kBucketedMaxNodes = int64_t(kMaxBuckets) * kBucketRange;
 constexpr int64_t kBucketedMinPicks = int64_t(1) << 18;  // worst-case picks of the hop below which the table is cheaper
-constexpr int64_t kBucketedMaxUnits = int64_t(1) << 23;  // bounds the extra workspace (8 bytes a unit)
+constexpr int64_t kBucketedMaxUnits = int64_t(kMaxBucketTiles - 2) * kBucketTile;  // so that the tiles fit that index; bounds the extra workspace too
 constexpr uint32_t kRankBit = 0x40000000u;
 
 struct Buckets {
-  uint2* items;      // [units_max] (id, order value) grouped by bucket; order value = rank of a frontier id, position of a pick
-  int* hist;         // [tiles_max][buckets] units of a tile per bucket, then their exclusive prefix down the column
-  int* total;        // [buckets]
-  int* start;        // [buckets + 1]
-  int64_t units_max; // items[] holds this many
+  uint2* items;      // [tiles_max][kBucketTile] (id, order value), every tile's units in bucket order
+  uint16_t* piece;   // [tiles_max][buckets + 1] where every bucket's piece begins inside its tile; [buckets] = the tile's units
   int32_t tiles_max; // tiles of units: front_tiles over the frontier array, the rest over the hop's padded positions
   int32_t front_tiles;
   int32_t log_buckets;
@@ -575,13 +576,9 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
 
 // ---- the bucketed pass (see Buckets) --------------------------------------------------------
 
-// The units of a bucketed hop are the frontier's ids (order value = rank) and the hop's padded
-// positions (order value = position, which is above every rank).  They are cut into tiles of
-// kBucketTile whose addresses do not depend on the hop's length, so that a block can ask for its
-// units at once: front_tiles tiles over the frontier array as large as it can get, then the
-// tiles of the padded positions.  Tiles that hold nothing (beyond the real frontier, beyond the
-// real positions) are skipped when rows of hist are numbered: row = tile for a frontier tile
-// that holds ids, (frontier tiles that hold ids) + (tile - front_tiles) for a position tile.
+// Tiles are laid out so that no address depends on the hop's length: front_tiles tiles over the
+// frontier array as large as it can get, then the tiles of the padded positions.  A block can
+// therefore ask for its units at once and decide afterwards which of them count.
 struct TileOfUnits {
   bool front;      // a tile of frontier ids
   int64_t first;   // its first rank, or its first position relative to the hop's pos_base
@@ -592,14 +589,9 @@ __device__ __forceinline__ TileOfUnits bucket_tile(const Buckets& b, int64_t til
   t.first = (t.front ? tile : tile - b.front_tiles) * kBucketTile;
   return t;
 }
-// rows of hist in use, and the row of a tile (-1: the tile holds nothing)
-__device__ __forceinline__ int64_t bucket_front_rows(int64_t s) { return (s + kBucketTile - 1) / kBucketTile; }
-__device__ __forceinline__ int64_t bucket_rows(const Hop& h, int64_t s) {
-  return bucket_front_rows(s) + (s * h.k + kBucketTile - 1) / kBucketTile;
-}
-__device__ __forceinline__ int64_t bucket_row(const Hop& h, const TileOfUnits& t, int64_t s) {
-  if (t.front) return t.first < s ? t.first / kBucketTile : -1;
-  return t.first < s * h.k ? bucket_front_rows(s) + t.first / kBucketTile : -1;
+// whether the tile holds anything at the hop's real length
+__device__ __forceinline__ bool bucket_tile_live(const Hop& h, const TileOfUnits& t, int64_t s) {
+  return t.first < (t.front ? s : s * h.k);
 }
 // A thread's units of a tile, requested without knowing the hop's length (every address lies inside
 // its array whatever the length turns out to be); `valid` then says which of them count.
@@ -631,186 +623,135 @@ struct UnitsOfThread {
   }
 };
 
-// hist[row][bucket] = units of the tile whose id falls into the bucket (id mod buckets)
+// One block per tile: the tile's units in bucket order (counted, placed and staged in LDS, then
+// written as one contiguous run), and where every bucket's piece begins.
 template <typename IdT>
-__global__ __launch_bounds__(kBlock) void bucket_count_kernel(Hop h, Buckets b) {
-  __shared__ int cnt[kMaxBuckets];
-  const int buckets = 1 << b.log_buckets;
-  for (int64_t tile = blockIdx.x; tile < b.tiles_max; tile += gridDim.x) {
-    const TileOfUnits t = bucket_tile(b, tile);
-    UnitsOfThread<IdT> mine;
-    mine.load(h, t);
-    const int64_t s = seeds_of(h);
-    const int64_t row = bucket_row(h, t, s);
-    if (row < 0 || row >= b.tiles_max) continue;  // whole blocks skip a tile together
-    for (int j = threadIdx.x; j < buckets; j += kBlock) cnt[j] = 0;
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < kBucketTileItems; ++j)
-      if (mine.valid(h, t, s, j)) atomicAdd(&cnt[mine.id[j] & uint32_t(buckets - 1)], 1);
-    __syncthreads();
-    for (int j = threadIdx.x; j < buckets; j += kBlock) b.hist[row * buckets + j] = cnt[j];
-    __syncthreads();
-  }
-}
-
-// Down every column of hist: exclusive prefix in place, total[bucket] = the column's sum.  A
-// block takes 32 buckets; its 32 x 32 threads split the rows into 32 runs.
-__global__ __launch_bounds__(1024) void bucket_scan_kernel(Hop h, Buckets b) {
-  __shared__ int part[32][33];
-  const int buckets = 1 << b.log_buckets;
-  const int lane = threadIdx.x & 31, run = threadIdx.x >> 5;
-  const int bucket = blockIdx.x * 32 + lane;  // the grid has buckets / 32 blocks
-  int64_t rows = bucket_rows(h, seeds_of(h));
-  if (rows > b.tiles_max) rows = b.tiles_max;
-  const int64_t per = (rows + 31) / 32;
-  const int64_t t0 = run * per < rows ? run * per : rows;
-  const int64_t t1 = t0 + per < rows ? t0 + per : rows;
-  int sum = 0;
-  for (int64_t t = t0; t < t1; ++t) sum += b.hist[t * buckets + bucket];
-  part[run][lane] = sum;
-  __syncthreads();
-  int before = 0;
-  for (int r = 0; r < run; ++r) before += part[r][lane];
-  for (int64_t t = t0; t < t1; ++t) {
-    const int v = b.hist[t * buckets + bucket];
-    b.hist[t * buckets + bucket] = before;
-    before += v;
-  }
-  if (run == 31) b.total[bucket] = before;  // the runs before the last one, plus its own
-}
-
-// Every unit goes to its bucket's stretch of items[]: start of the bucket (prefix over total[],
-// which every block works out for itself) + the units of earlier rows + a turn among its own
-// tile's.  A tile's units are first put in bucket order in LDS and written out from there, so
-// that what goes to one bucket leaves as one contiguous piece instead of unit by unit.
-template <typename IdT>
-__global__ __launch_bounds__(kBlock) void bucket_scatter_kernel(Hop h, Buckets b) {
-  __shared__ int start[kMaxBuckets];   // first item of every bucket
-  __shared__ int base[kMaxBuckets];    // where the tile's first staged unit of a bucket goes, minus its place in the stage
-  __shared__ int cur[kMaxBuckets];     // next free place in the stage for every bucket
+__global__ __launch_bounds__(kBlock) void bucket_sort_kernel(Hop h, Buckets b) {
+  __shared__ int cnt[kMaxBuckets];     // units per bucket, then the next free place of every bucket in the stage
   __shared__ uint2 stage[kBucketTile];
   __shared__ int lds[kBlock / kWave];
   const int buckets = 1 << b.log_buckets;
   const int mine = buckets / kBlock;  // 2..8 consecutive buckets per thread
-  // the first tile's units and the bucket totals, requested together
-  TileOfUnits t = bucket_tile(b, blockIdx.x);
-  UnitsOfThread<IdT> units;
-  if (int64_t(blockIdx.x) < b.tiles_max) units.load(h, t);
-  int own[kMaxBuckets / kBlock];
-  int sum = 0;
-#pragma unroll
-  for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
-    own[j] = j < mine ? b.total[threadIdx.x * mine + j] : 0;
-    sum += own[j];
-  }
-  const int64_t s = seeds_of(h);
-  int64_t rows = bucket_rows(h, s);
-  if (rows > b.tiles_max) rows = b.tiles_max;
-  int all;
-  int at = block_exclusive_scan<kBlock, int>(sum, &all, lds);
-#pragma unroll
-  for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
-    if (j < mine) {
-      start[threadIdx.x * mine + j] = at;
-      if (blockIdx.x == 0) b.start[threadIdx.x * mine + j] = at;
-      at += own[j];
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x == 0) b.start[buckets] = all;
-  __syncthreads();
   for (int64_t tile = blockIdx.x; tile < b.tiles_max; tile += gridDim.x) {
-    if (tile != int64_t(blockIdx.x)) {
-      t = bucket_tile(b, tile);
-      units.load(h, t);
-    }
-    const int64_t row = bucket_row(h, t, s);
-    if (row < 0 || row >= rows) continue;  // whole blocks skip a tile together
-    // this tile's units per bucket: the difference of the column prefixes of this row and the next
-    int before[kMaxBuckets / kBlock];
-    sum = 0;
+    const TileOfUnits t = bucket_tile(b, tile);
+    UnitsOfThread<IdT> units;
+    units.load(h, t);
+    const int64_t s = seeds_of(h);
+    if (!bucket_tile_live(h, t, s)) continue;  // whole blocks skip a tile together
+    for (int j = threadIdx.x; j < buckets; j += kBlock) cnt[j] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kBucketTileItems; ++j)
+      if (units.valid(h, t, s, j)) atomicAdd(&cnt[units.id[j] & uint32_t(buckets - 1)], 1);
+    __syncthreads();
+    int own[kMaxBuckets / kBlock];
+    int sum = 0;
 #pragma unroll
     for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
-      own[j] = before[j] = 0;
-      if (j < mine) {
-        const int bucket = threadIdx.x * mine + j;
-        before[j] = b.hist[row * buckets + bucket];
-        const int upto = row + 1 < rows ? b.hist[(row + 1) * buckets + bucket] : b.total[bucket];
-        own[j] = upto - before[j];
-        if (own[j] < 0 || own[j] > kBucketTile) own[j] = 0;  // cannot happen; keeps what follows inside the stage
-        sum += own[j];
-      }
+      own[j] = j < mine ? cnt[threadIdx.x * mine + j] : 0;
+      sum += own[j];
     }
-    at = block_exclusive_scan<kBlock, int>(sum, &all, lds);
+    int all;
+    int at = block_exclusive_scan<kBlock, int>(sum, &all, lds);
+    uint16_t* piece = b.piece + tile * (buckets + 1);
 #pragma unroll
     for (int j = 0; j < kMaxBuckets / kBlock; ++j) {
       if (j < mine) {
-        const int bucket = threadIdx.x * mine + j;
-        cur[bucket] = at;
-        base[bucket] = start[bucket] + before[j] - at;
+        cnt[threadIdx.x * mine + j] = at;  // (the scan's barriers lie between the reads above and this)
+        piece[threadIdx.x * mine + j] = uint16_t(at);
         at += own[j];
       }
     }
+    if (threadIdx.x == 0) piece[buckets] = uint16_t(all);  // <= 4096
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < kBucketTileItems; ++j) {
       if (units.valid(h, t, s, j)) {
-        const int to = atomicAdd(&cur[units.id[j] & uint32_t(buckets - 1)], 1);
+        const int to = atomicAdd(&cnt[units.id[j] & uint32_t(buckets - 1)], 1);
         if (to >= 0 && to < kBucketTile) stage[to] = make_uint2(units.id[j], units.order[j]);
       }
     }
     __syncthreads();
     const int staged = all < kBucketTile ? all : kBucketTile;
-    for (int e = threadIdx.x; e < staged; e += kBlock) {
-      const uint2 it = stage[e];
-      const int64_t to = int64_t(base[it.x & uint32_t(buckets - 1)]) + e;
-      if (to >= 0 && to < b.units_max) b.items[to] = it;
-    }
+    for (int e = threadIdx.x; e < staged; e += kBlock) b.items[tile * kBucketTile + e] = stage[e];
     __syncthreads();
   }
 }
 
-// One block per bucket: the smallest order value of every id (LDS, indexed by id / buckets), then
-// the slot word of every pick that is not its id's first occurrence.
+// One block per bucket.  It lists the bucket's pieces in the live tiles (LDS: where each begins in
+// items[] and how many units came before it), so that its threads can share the bucket's units
+// evenly whatever their spread over the tiles; then the smallest order value of every id (LDS,
+// indexed by id / buckets), then the slot word of every pick that is not its id's first occurrence.
 __global__ __launch_bounds__(kBlock) void bucket_first_kernel(Hop h, Buckets b) {
   __shared__ uint32_t best[kBucketRange];
+  __shared__ int piece_at[kMaxBucketTiles];      // first unit of the tile's piece, as an index into items[]
+  __shared__ int piece_before[kMaxBucketTiles];  // units of the bucket in the tiles before
+  __shared__ int lds[kBlock / kWave];
   const int buckets = 1 << b.log_buckets;
   const uint32_t range = (b.n_nodes + uint32_t(buckets) - 1) >> b.log_buckets;  // <= kBucketRange by the plan
   const uint32_t pos_begin = uint32_t(h.pos_base), pos_end = uint32_t(h.pos_base + h.len_max);
+  const int64_t s = seeds_of(h);
+  const int tiles = b.tiles_max < kMaxBucketTiles ? b.tiles_max : kMaxBucketTiles;
+  const int64_t item_count = int64_t(b.tiles_max) * kBucketTile;
   for (int bucket = blockIdx.x; bucket < buckets; bucket += gridDim.x) {
-    int64_t begin = b.start[bucket], end = b.start[bucket + 1];
-    if (begin < 0) begin = 0;
-    if (end > b.units_max) end = b.units_max;
-    // a thread's first kKept items stay in registers for the second pass (a bucket of the usual
-    // size is then read once), and are requested before the LDS array is cleared
+    for (uint32_t j = threadIdx.x; j < range && j < uint32_t(kBucketRange); j += kBlock) best[j] = 0xffffffffu;
+    // the bucket's pieces: kBlock tiles at a time, a running total carried along
+    int total = 0;
+    for (int t0 = 0; t0 < tiles; t0 += kBlock) {
+      const int tile = t0 + threadIdx.x;
+      int from = 0, count = 0;
+      if (tile < tiles && bucket_tile_live(h, bucket_tile(b, tile), s)) {
+        const uint16_t* piece = b.piece + int64_t(tile) * (buckets + 1);
+        from = piece[bucket];
+        const int upto = piece[bucket + 1];
+        if (from <= upto && upto <= kBucketTile) count = upto - from;
+      }
+      int sum;
+      const int before = block_exclusive_scan<kBlock, int>(count, &sum, lds);
+      if (tile < tiles) {
+        piece_at[tile] = tile * kBucketTile + from;
+        piece_before[tile] = total + before;
+      }
+      total += sum;
+    }
+    __syncthreads();
+    // unit j of the bucket lives in the last tile whose piece_before is <= j
+    const auto unit = [&](int j) {
+      int lo = 0, hi = tiles - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (piece_before[mid] <= j) lo = mid; else hi = mid - 1;
+      }
+      const int64_t at = int64_t(piece_at[lo]) + (j - piece_before[lo]);
+      return at >= 0 && at < item_count ? b.items[at] : make_uint2(0u, 0u);
+    };
+    // a thread's first kKept units stay in registers for the second pass
     constexpr int kKept = 8;
     uint2 kept[kKept];
 #pragma unroll
     for (int r = 0; r < kKept; ++r) {
-      const int64_t j = begin + threadIdx.x + int64_t(r) * kBlock;
-      kept[r] = j < end ? b.items[j] : make_uint2(0u, 0u);
+      const int j = threadIdx.x + r * kBlock;
+      kept[r] = j < total ? unit(j) : make_uint2(0u, 0u);
     }
-    for (uint32_t j = threadIdx.x; j < range && j < uint32_t(kBucketRange); j += kBlock) best[j] = 0xffffffffu;
-    __syncthreads();
-    for (int64_t j = begin + threadIdx.x, r = 0; j < end; j += kBlock, ++r) {
+    for (int j = threadIdx.x, r = 0; j < total; j += kBlock, ++r) {
       uint2 it = make_uint2(0u, 0u);
       if (r < kKept) {
 #pragma unroll
         for (int q = 0; q < kKept; ++q) if (q == r) it = kept[q];
       } else {
-        it = b.items[j];
+        it = unit(j);
       }
       const uint32_t at = it.x >> b.log_buckets;
       if (at < range && at < uint32_t(kBucketRange)) atomicMin(&best[at], it.y);
     }
     __syncthreads();
-    for (int64_t j = begin + threadIdx.x, r = 0; j < end; j += kBlock, ++r) {
+    for (int j = threadIdx.x, r = 0; j < total; j += kBlock, ++r) {
       uint2 it = make_uint2(0u, 0u);
       if (r < kKept) {
 #pragma unroll
         for (int q = 0; q < kKept; ++q) if (q == r) it = kept[q];
       } else {
-        it = b.items[j];
+        it = unit(j);
       }
       const uint32_t at = it.x >> b.log_buckets;
       if (it.y < pos_begin || it.y >= pos_end || at >= range || at >= uint32_t(kBucketRange)) continue;  // a frontier id
@@ -1089,13 +1030,10 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
   }
   if (p.bucket_space) {
     Buckets b{};
-    b.units_max = bucket_units_max(p);
     b.front_tiles = int32_t((p.s_max[p.n_hops - 1] + kBucketTile - 1) / kBucketTile);
     b.tiles_max = b.front_tiles + int32_t((p.nnz_max[p.n_hops - 1] + kBucketTile - 1) / kBucketTile);
-    b.items = c.take<uint2>(size_t(b.units_max));
-    b.hist = c.take<int>(size_t(b.tiles_max) * kMaxBuckets);
-    b.total = c.take<int>(kMaxBuckets);
-    b.start = c.take<int>(kMaxBuckets + 1);
+    b.items = c.take<uint2>(size_t(b.tiles_max) * kBucketTile);
+    b.piece = c.take<uint16_t>(size_t(b.tiles_max) * (kMaxBuckets + 1));
     b.log_buckets = p.log_buckets;
     b.n_nodes = p.n_nodes;
     if (buckets) *buckets = b;
@@ -1177,12 +1115,8 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const Buckets& buckets, const Ta
 
     if (cur.bucketed) {  // the picks' slot words hold ids so far: group them and find the first occurrences
       const int n_buckets = 1 << buckets.log_buckets;
-      const uint32_t tile_grid = capped_grid(buckets.tiles_max);
-      hipLaunchKernelGGL(bucket_count_kernel<IdT>, dim3(tile_grid), dim3(kBlock), 0, st, cur, buckets);
-      DGS_LAUNCH_CHECK();
-      hipLaunchKernelGGL(bucket_scan_kernel, dim3(uint32_t(n_buckets / 32)), dim3(1024), 0, st, cur, buckets);
-      DGS_LAUNCH_CHECK();
-      hipLaunchKernelGGL(bucket_scatter_kernel<IdT>, dim3(tile_grid), dim3(kBlock), 0, st, cur, buckets);
+      hipLaunchKernelGGL(bucket_sort_kernel<IdT>, dim3(capped_grid(buckets.tiles_max)), dim3(kBlock), 0, st, cur,
+                         buckets);
       DGS_LAUNCH_CHECK();
       hipLaunchKernelGGL(bucket_first_kernel, dim3(capped_grid(n_buckets)), dim3(kBlock), 0, st, cur, buckets);
       DGS_LAUNCH_CHECK();
