@@ -695,21 +695,30 @@ __global__ __launch_bounds__(kBlock) void bucket_first_kernel(Hop h, Buckets b) 
   const int64_t item_count = int64_t(b.tiles_max) * kBucketTile;
   for (int bucket = blockIdx.x; bucket < buckets; bucket += gridDim.x) {
     for (uint32_t j = threadIdx.x; j < range && j < uint32_t(kBucketRange); j += kBlock) best[j] = 0xffffffffu;
-    // the bucket's pieces: kBlock tiles at a time, a running total carried along
-    int total = 0;
-    for (int t0 = 0; t0 < tiles; t0 += kBlock) {
-      const int tile = t0 + threadIdx.x;
-      int from = 0, count = 0;
+    // the bucket's pieces: every thread asks for those of its tiles (tile = round * kBlock + thread)
+    // at once, then the rounds are scanned one after the other, a running total carried along
+    constexpr int kRounds = kMaxBucketTiles / kBlock;
+    int from[kRounds], upto[kRounds];
+#pragma unroll
+    for (int q = 0; q < kRounds; ++q) {
+      const int tile = q * kBlock + threadIdx.x;
+      from[q] = upto[q] = 0;
       if (tile < tiles && bucket_tile_live(h, bucket_tile(b, tile), s)) {
         const uint16_t* piece = b.piece + int64_t(tile) * (buckets + 1);
-        from = piece[bucket];
-        const int upto = piece[bucket + 1];
-        if (from <= upto && upto <= kBucketTile) count = upto - from;
+        from[q] = piece[bucket];
+        upto[q] = piece[bucket + 1];
       }
+    }
+    int total = 0;
+#pragma unroll
+    for (int q = 0; q < kRounds; ++q) {
+      if (q * kBlock >= tiles) break;  // the same for every thread
+      const int tile = q * kBlock + threadIdx.x;
+      const int count = from[q] <= upto[q] && upto[q] <= kBucketTile ? upto[q] - from[q] : 0;
       int sum;
       const int before = block_exclusive_scan<kBlock, int>(count, &sum, lds);
       if (tile < tiles) {
-        piece_at[tile] = tile * kBucketTile + from;
+        piece_at[tile] = tile * kBucketTile + from[q];
         piece_before[tile] = total + before;
       }
       total += sum;
