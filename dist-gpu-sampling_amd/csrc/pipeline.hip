@@ -23,7 +23,7 @@
 //     per pick: the indices read and the table atomic.
 //
 // A large last hop of uniform picks does without the table altogether (see Buckets below): its
-// fill records the picked ids, four launches group them by id and take the smallest position of
+// fill records the picked ids, two launches group them by id and take the smallest position of
 // every id in LDS, and flag / compact / relabel read the same slot words as on the table path.
 //
 // Critical path per hop (3 launches): fill -> flag -> compact.
@@ -977,7 +977,7 @@ dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, in
                 "sample_blocks: a node table needs fewer than 2^31 nodes (have %lld)", (long long)n_nodes);
     p->kind = TableKind::kDirect;
     // the bucketed pass: slot words are ids (the direct table's), ids fit the LDS arrays, and the
-    // hop is large enough for its four extra launches to cost less than the atomics they replace
+    // hop is large enough for its two extra launches to cost less than the atomics they replace
     // (test hook: 1 never, 2 whatever the size)
     const int64_t mode = debug_option(DGS_DEBUG_SAMPLER_BUCKETED);
     const bool large = p->nnz_max[n_hops - 1] >= kBucketedMinPicks;
@@ -1251,8 +1251,8 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
                 "sample_blocks_weighted: %lld weights of %d bytes for %lld edges (float32, one per edge)",
                 (long long)probs->total, probs->elem_bytes, (long long)indices.total);
     p.weighted = true;
-    // weighted picks: the fill is bound by the races, not by its atomics, and the bucketed pass only
-    // lengthens the batch (measured: + 25 us alone, the same step with four batches in flight)
+    // weighted picks: the fill is bound by the races, not by its atomics, and the bucketed pass
+    // changes the step by a per cent either way (measured with three and four batches in flight)
     if (debug_option(DGS_DEBUG_SAMPLER_BUCKETED) != 2) p.bucketed = false;
   }
   const size_t need = probs != nullptr ? dgs_sample_blocks_weighted_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes)
