@@ -667,17 +667,36 @@ class PendingBlocks : public torch::CustomClassHolder {
       dst_at[h] = piece(edges_max[h] * w);
     }
     const int64_t sizes_at = piece(n_sizes * 8);
-    p->ids_ = device_bytes(static_cast<size_t>(carved), dev);
-    const auto ids_of = [&](int64_t at, int64_t count) {
-      return p->ids_.narrow(0, at, count * w).view(p->seeds_.scalar_type());
-    };
-    p->all_ = ids_of(all_at, seeds_max[hops]);
-    for (int h = 0; h < hops; ++h) {
-      p->src_[h] = ids_of(src_at[h], edges_max[h]);
-      p->dst_[h] = ids_of(dst_at[h], edges_max[h]);
-      outs[h] = dgs_block_out{p->src_[h].data_ptr(), p->dst_[h].data_ptr()};
+    // (up to kOneBlockBytes: beyond that the pieces are hundreds of megabytes each, the calls to the
+    // allocator no longer matter and separate blocks are reused more freely: C4, whose worst case
+    // is 511 MB of ids per batch, ran 4 % slower out of one block)
+    constexpr int64_t kOneBlockBytes = int64_t(128) << 20;
+    torch::Tensor sizes_dev;
+    if (carved <= kOneBlockBytes) {
+      torch::Tensor block = device_bytes(static_cast<size_t>(carved), dev);
+      const auto ids_of = [&](int64_t at, int64_t count) {
+        return block.narrow(0, at, count * w).view(p->seeds_.scalar_type());
+      };
+      p->all_ = ids_of(all_at, seeds_max[hops]);
+      for (int h = 0; h < hops; ++h) {
+        p->src_[h] = ids_of(src_at[h], edges_max[h]);
+        p->dst_[h] = ids_of(dst_at[h], edges_max[h]);
+      }
+      sizes_dev = block.narrow(0, sizes_at, n_sizes * 8).view(torch::kInt64);
+      p->owned_.push_back(block);
+    } else {
+      p->all_ = torch::empty({seeds_max[hops]}, opt);
+      p->owned_.push_back(p->all_);
+      for (int h = 0; h < hops; ++h) {
+        p->src_[h] = torch::empty({edges_max[h]}, opt);
+        p->dst_[h] = torch::empty({edges_max[h]}, opt);
+        p->owned_.push_back(p->src_[h]);
+        p->owned_.push_back(p->dst_[h]);
+      }
+      sizes_dev = torch::empty({n_sizes}, opt.dtype(torch::kInt64));
+      p->owned_.push_back(sizes_dev);  // (kept with the batch: the kernels write it after this call returns)
     }
-    torch::Tensor sizes_dev = p->ids_.narrow(0, sizes_at, n_sizes * 8).view(torch::kInt64);
+    for (int h = 0; h < hops; ++h) outs[h] = dgs_block_out{p->src_[h].data_ptr(), p->dst_[h].data_ptr()};
     const size_t ws_bytes = probs ? dgs_sample_blocks_weighted_workspace_bytes(n, fanouts.data(), hops, w)
                                   : dgs_sample_blocks_workspace_bytes(n, fanouts.data(), hops, w);
     torch::Tensor ws = device_bytes(ws_bytes, dev);  // freed on return: the allocator reuses it in stream order
@@ -726,9 +745,10 @@ class PendingBlocks : public torch::CustomClassHolder {
   // stream (so that the allocator does not hand them out again while that stream still reads them).
   c10::Stream stream() const { return stream_; }
   void RecordStream(const c10::Stream& consumer) {
-    // (the frontier and the edge lists are views of ids_)
-    for (const torch::Tensor* t : {&seeds_, &ids_, &x_})
+    // (the frontier and the edge lists are, or are views of, the tensors in owned_)
+    for (const torch::Tensor* t : {&seeds_, &x_})
       if (t->defined() && t->is_cuda()) t->record_stream(consumer);
+    for (const torch::Tensor& t : owned_) t.record_stream(consumer);
   }
 
  private:
@@ -736,7 +756,8 @@ class PendingBlocks : public torch::CustomClassHolder {
   bool finished_ = false;
   void* ticket_ = nullptr;
   dgs_status gather_status_ = DGS_OK;
-  torch::Tensor pinned_, seeds_, ids_, all_, x_;  // ids_: the allocation all_, src_ and dst_ are views of
+  torch::Tensor pinned_, seeds_, all_, x_;
+  std::vector<torch::Tensor> owned_;  // the allocations behind all_, src_, dst_ and the device-side lengths
   torch::Tensor staged_seeds_;  // pinned copy of host seeds, alive until the batch is finished
   std::vector<torch::Tensor> src_, dst_;
   // the feature gather: rows of the buffer it was enqueued into (-1: none), and what a second,
