@@ -815,3 +815,26 @@ def test_bucketed_last_hop_at_its_largest_graph(pkg, oracle, n_nodes):
     assert want_f.max() >= n_nodes - 20
     del ip_ct, ix_ct, sampler
     torch.cuda.empty_cache()
+
+
+def test_bucketed_last_hop_near_its_largest_worst_case(pkg, oracle, graph):
+    # 1024 seeds x [7, 30, 31] (hop order): the last hop's worst case is 8.1 M units, just inside what
+    # the bucketed pass has room for (1985 of its 2048 tiles; most of them stay empty on this graph,
+    # whose 20,000 nodes the frontier soon exhausts), and the pass is chosen by size
+    indptr, indices = graph
+    rng = np.random.default_rng(17)
+    seeds = rng.permutation(20000)[:1024].astype(np.int64)
+    fanouts = [31, 30, 7]
+    want_f, _, want_blocks = oracle.sample_blocks(seeds, indptr, indices, fanouts, False, 77, 3)
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct)
+    for mode in LAST_HOP_MODES:
+        set_last_hop_mode(pkg, mode)
+        try:
+            pkg.set_rng_state(77, 3)
+            frontier, _, blocks = sampler.sample_blocks(None, _dev(seeds))
+        finally:
+            set_last_hop_mode(pkg, LAST_HOP_MODES[0])
+        assert np.array_equal(_np(frontier), want_f), mode
+        _check_blocks(blocks, want_blocks)
