@@ -75,3 +75,32 @@ def test_random_cases_match_the_oracle(pkg, oracle, sweep, last_hop):
         f, _, blocks = pkg.ChunkTensorSampler(fan_w, ip_ct, ix_ct, pr_ct, replace).sample_blocks(None, _dev(seeds))
         assert np.array_equal(_np(f), want_f), ("weighted frontier",) + what
         assert _same_blocks(blocks, want_b), ("weighted blocks",) + what
+
+
+def test_random_larger_cases_match_the_oracle(pkg, oracle, last_hop):
+    # fewer, larger cases: up to 300 k nodes, up to five hops, several thousand seeds, so that
+    # frontiers span many tiles and the last hop's units many pieces per bucket; worst-case sizes
+    # (seeds x product of (1 + fanout)) are kept below 2 * 10^7 ids
+    rng = np.random.default_rng(99)
+    big = 1 << 40
+    for case in range(8):
+        n = int(rng.integers(50_000, 300_000))
+        idt = rng.choice([np.int32, np.int64])
+        indptr, indices = powerlaw_graph(rng, n, int(rng.integers(4, 24)), int(rng.integers(50, 5000)),
+                                         zero_frac=float(rng.random() * 0.2), id_dtype=idt, ptr_dtype=np.int64)
+        while True:
+            fan = [int(rng.integers(1, 13)) for _ in range(int(rng.integers(2, 6)))]
+            n_seeds = int(rng.integers(500, 5000))
+            if n_seeds * np.prod([1 + k for k in fan]) <= 2e7:
+                break
+        replace = bool(rng.random() < 0.3)
+        seeds = rng.integers(0, n, size=n_seeds).astype(idt)
+        what = (case, n, idt.__name__, fan, replace, n_seeds)
+        ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+        ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+        seed, stream = int(rng.integers(0, 2 ** 62)), int(rng.integers(0, 1000))
+        want_f, _, want_b = oracle.sample_blocks(seeds, indptr, indices, fan, replace, seed, stream)
+        pkg.set_rng_state(seed, stream)
+        f, _, blocks = pkg.ChunkTensorSampler(fan, ip_ct, ix_ct, replace=replace).sample_blocks(None, _dev(seeds))
+        assert np.array_equal(_np(f), want_f), ("frontier",) + what
+        assert _same_blocks(blocks, want_b), ("blocks",) + what
