@@ -28,44 +28,48 @@ from . import capi  # noqa: E402
 torch.ops.load_library(TORCH_LIB)
 
 
-def _lighten_torch_dispatch():
-    """Takes two per-call costs of torch's Python front end off operators that run for 30 us.
-
-    1. For every argument that is not a tensor, torch asks `hasattr(arg, "__torch_function__")`.
-       On a custom-class object (torch.ScriptObject: every ChunkTensor) the miss goes through
-       the class's `__getattr__` and two C++ exceptions: 5.4 us per argument per call, 11 us of a
-       34 us `_CAPI_sample_neighbors_with_chunk_tensor`.  torch's own opt-out value for that
-       protocol, set on the class, makes the lookup a hit that means "no override" (0.03 us).
-    2. For operators with custom-class arguments, `OpOverloadPacket.__call__` first walks the
-       arguments in Python looking for FakeScriptObjects (export/compile tracing; 4 us a call)
-       and then calls the C++ entry `packet._op`.  The names in `torch.ops.dgs_ops` that take
-       ChunkTensors are bound to that entry directly.  They remain callables with the same
-       arguments, results and errors; what they lose is the tracing support, which these
-       operators (blocking reads of data-dependent sizes) do not have anyway.
-
-    Set DGS_PLAIN_TORCH_DISPATCH=1 to leave torch as it is."""
-    if os.environ.get("DGS_PLAIN_TORCH_DISPATCH", "0") not in ("", "0"):
-        return
-    if "__torch_function__" not in vars(torch.ScriptObject):
-        torch.ScriptObject.__torch_function__ = torch._C._disabled_torch_function_impl
-    for name in ("_CAPI_sample_neighbors_with_chunk_tensor", "_CAPI_sample_neighbors_with_probs_with_chunk_tensor",
-                 "_CAPI_sample_blocks", "_CAPI_sample_blocks_and_index", "_CAPI_sample_blocks_begin",
-                 "_CAPI_sample_blocks_and_index_begin", "_CAPI_sample_blocks_weighted_begin",
-                 "_CAPI_sample_blocks_submit"):
-        entry = getattr(getattr(torch.ops.dgs_ops, name), "_op", None)
-        if callable(entry):
-            setattr(torch.ops.dgs_ops, name, entry)
+_script_object_had_opt_out = "__torch_function__" in vars(torch.ScriptObject)
 
 
-_lighten_torch_dispatch()
+def lighten_torch_dispatch(enable=True):
+    """Opt-in, process-wide: takes a per-argument cost of torch's Python front end off operators
+    that run for 30 us.  Returns whether the shortcut is in place afterwards.
+
+    For every operator argument that is not a tensor, torch asks
+    `hasattr(arg, "__torch_function__")`.  On a custom-class object (torch.ScriptObject: every
+    ChunkTensor, and every object of any other extension's custom classes) the miss goes through
+    the class's `__getattr__` and two C++ exceptions: 5.4 us per argument per call, 11 us of a
+    34 us `_CAPI_sample_neighbors_with_chunk_tensor`.  torch's own opt-out value for that
+    protocol, set on the class, makes the lookup a hit that means "no override" (0.03 us).
+    Because torch.ScriptObject is shared by all custom classes of the process, nothing here does
+    this on import: a program calls lighten_torch_dispatch() if it wants it (bench.py does, and
+    reports the per-hop operators both ways), lighten_torch_dispatch(False) takes it back, and
+    DGS_LIGHT_TORCH_DISPATCH=1 in the environment asks for it at import.
+
+    The package's own calls also skip `OpOverloadPacket.__call__` (a walk over the arguments in
+    Python, 4 us a call) by calling the packets' C++ entries (sampler.fast_ops); that touches
+    nothing of torch: `torch.ops.dgs_ops.<name>` stay the packets torch made, with their
+    `.default` overloads and schemas."""
+    if enable:
+        if "__torch_function__" not in vars(torch.ScriptObject):
+            torch.ScriptObject.__torch_function__ = torch._C._disabled_torch_function_impl
+    elif not _script_object_had_opt_out and "__torch_function__" in vars(torch.ScriptObject):
+        del torch.ScriptObject.__torch_function__
+    return "__torch_function__" in vars(torch.ScriptObject)
+
+
+if os.environ.get("DGS_LIGHT_TORCH_DISPATCH", "0") not in ("", "0"):
+    lighten_torch_dispatch()
 
 from .sampler import (  # noqa: E402
     BatchPipeline,
     ChunkTensorSampler,
     Block,
     PendingBatch,
+    cached_bytes_per_gpu,
     create_chunktensor,
     create_dgs_communicator,
+    fast_ops,
     get_available_memory,
     pipeline_streams,
     set_gather_buffer_cap,
@@ -79,5 +83,5 @@ from . import loading_factor  # noqa: E402
 ChunkTensor = torch.classes.dgs_classes.ChunkTensor
 ops = torch.ops.dgs_ops
 
-__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "create_chunktensor",
-           "create_dgs_communicator", "get_available_memory", "set_rng_state", "set_gather_buffer_cap", "pipeline_streams", "streams_overlap", "HIP_LIB", "TORCH_LIB"]
+__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "cached_bytes_per_gpu", "create_chunktensor",
+           "create_dgs_communicator", "get_available_memory", "set_rng_state", "set_gather_buffer_cap", "pipeline_streams", "streams_overlap", "lighten_torch_dispatch", "fast_ops", "HIP_LIB", "TORCH_LIB"]

@@ -18,6 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(HERE, "libdgs_hip.so")
 TORCH_LIB = os.path.join(HERE, "libdgs.so")
+OBJ_DIR = os.path.join(HERE, "build")  # objects of the HIP sources (not tracked)
 
 HIP_SOURCES = ["store.hip", "gather.hip", "sample.hip", "weighted.hip", "placement.hip", "unique.hip", "pipeline.hip"]
 HIP_HEADERS = ["common.h", "table.h", "picks.h", "weights.h", "race.h", "sample_workspace.h"]
@@ -37,16 +38,29 @@ def _stale(target, sources):
 
 
 def build_hip(force=True):
-    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    deps = srcs + [os.path.join(CSRC, h) for h in HIP_HEADERS] + [os.path.join(INCLUDE, "dgs_hip.h")]
-    if not force and not _stale(HIP_LIB, deps):
-        return HIP_LIB
+    """One object per source (compiled side by side: the sources are independent), then one link.
+    Without `force` only the objects older than their source or a header are compiled again."""
+    from concurrent.futures import ThreadPoolExecutor
+    headers = [os.path.join(CSRC, h) for h in HIP_HEADERS] + [os.path.join(INCLUDE, "dgs_hip.h")]
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    _run([hipcc, "-O3", "--offload-arch=" + ARCH, "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
-          # packed-FP32 instruction selection is switched off for every kernel in this library
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-          "-Wall", "-Wextra", "-Wno-unused-command-line-argument",
-          "-I" + INCLUDE, "-o", HIP_LIB] + srcs)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    flags = ["-O3", "--offload-arch=" + ARCH, "-std=c++17", "-fPIC", "-fvisibility=hidden",
+             # packed-FP32 instruction selection is switched off for every kernel in this library
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wall", "-Wextra", "-Wno-unused-command-line-argument", "-I" + INCLUDE]
+    jobs = []
+    objects = []
+    for name in HIP_SOURCES:
+        src = os.path.join(CSRC, name)
+        obj = os.path.join(OBJ_DIR, name.replace(".hip", ".o"))
+        objects.append(obj)
+        if force or _stale(obj, [src] + headers):
+            jobs.append([hipcc] + flags + ["-c", src, "-o", obj])
+    if jobs:
+        with ThreadPoolExecutor(max_workers=min(len(jobs), int(os.environ.get("MAX_JOBS", "8")))) as pool:
+            list(pool.map(_run, jobs))
+    if jobs or _stale(HIP_LIB, objects):
+        _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", HIP_LIB] + objects)
     return HIP_LIB
 
 

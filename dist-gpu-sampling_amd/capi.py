@@ -60,7 +60,7 @@ SIGNATURES = {
     "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
     "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_workspace_bytes": (c_sz, [c_i64]),
-    "dgs_sample_count": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "dgs_sample_count": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i64, c_i32, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_fill": (ctypes.c_int, [c_vp, c_i32, c_i64, View, c_i64, c_i32, c_u64, c_u32, c_vp, c_vp,
                                        c_vp, c_sz, c_vp]),
     "dgs_sample_neighbors": (ctypes.c_int, [c_vp, c_i32, c_i64, View, View, c_i64, c_i32, c_u64, c_u32,
@@ -96,6 +96,7 @@ SIGNATURES = {
     "dgs_stream_wait_words": (ctypes.c_int, [c_vp, c_vp, c_i32]),
     "dgs_ticket_release": (ctypes.c_int, [c_vp]),
     "dgs_stream_query": (ctypes.c_int, [c_vp, ctypes.POINTER(c_i32)]),
+    "dgs_ticket_query": (ctypes.c_int, [c_vp, ctypes.POINTER(c_i32)]),
 }
 
 if not os.path.exists(LIB_PATH):
@@ -215,14 +216,14 @@ def sample_neighbors(seeds, indptr_view, indices_view, num_picks, replace, rng_s
         if two_step == "mirrored":
             # the lengths through pinned words that the count kernel writes and the host polls
             pinned = torch.full((2,), -1, dtype=torch.int64).pin_memory()
-            check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
+            check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, indices_view.total, num_picks, int(replace), nnz.data_ptr(),
                                        pinned.data_ptr(), ws.data_ptr(), nb, stream_ptr()))
             ticket = ctypes.c_void_p()
             check(lib.dgs_ticket_record(stream_ptr(), ctypes.byref(ticket)))
             check(lib.dgs_ticket_wait_words(ticket, pinned.data_ptr(), 2))
             cnt, flags = pinned.tolist()
         else:
-            check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace),
+            check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, indices_view.total, num_picks, int(replace),
                                        nnz.data_ptr(), None, ws.data_ptr(), nb, stream_ptr()))
             cnt, flags = read_i64(nnz, 2)
         rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
@@ -263,7 +264,7 @@ def sample_neighbors_weighted(seeds, indptr_view, indices_view, probs_view, num_
     nnz = torch.empty(2, dtype=torch.int64, device=seeds.device)
     w = seeds.element_size()
     if two_step:
-        check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, num_picks, int(replace), nnz.data_ptr(),
+        check(lib.dgs_sample_count(seeds.data_ptr(), w, n, indptr_view, indices_view.total, num_picks, int(replace), nnz.data_ptr(),
                                    None, ws.data_ptr(), nb, stream_ptr()))
         cnt, flags = read_i64(nnz, 2)
         rows = torch.empty(cnt, dtype=seeds.dtype, device=seeds.device)
@@ -290,9 +291,10 @@ def renumber_csc(indptr, indices, order, rank, new_indptr):
     return out
 
 
-def unique_relabel(mapping, requiring, packed_table=True, polled=False):
+def unique_relabel(mapping, requiring, packed_table=True, polled=False, retry=True):
     """Returns (unique, [relabelled ...]).  With `packed_table` 8-byte ids are tried in the one-word
-    slots first and the call is repeated with the two-array table if an id does not fit.
+    slots first and the call is repeated with the two-array table if an id does not fit
+    (`retry=False`: it is not, and the void results of the first attempt are returned as they are).
     With `polled` the counts come through pinned words that the host polls instead of a copy."""
     dev = mapping[0].device
     dt = mapping[0].dtype
@@ -303,7 +305,7 @@ def unique_relabel(mapping, requiring, packed_table=True, polled=False):
     w = mapping[0].element_size()
     nb = lib.dgs_unique_relabel_workspace_bytes(n, w)
     ws = _ws(nb, dev)
-    for packed in ((1, 0) if packed_table else (0,)):
+    for packed in ((1, 0) if packed_table and retry else (1,) if packed_table else (0,)):
         if polled:
             pinned = torch.full((2,), -1, dtype=torch.int64).pin_memory()
             check(lib.dgs_unique_relabel(segments(mapping), segments(requiring), w, packed, unique.data_ptr(),

@@ -130,7 +130,11 @@ class ChunkTensor : public torch::CustomClassHolder {
     // without a copy, the kernels write it through its device mapping)
     bad_index_ = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
   }
-  ~ChunkTensor() override { dgs_store_destroy(store_); }
+  ~ChunkTensor() override {
+    for (auto& entry : node_tables_)
+      if (entry.second.done != nullptr) dgs_ticket_release(entry.second.done);
+    dgs_store_destroy(store_);
+  }
 
   // Raises if a gather that has run since the last check met an index outside the rows it may
   // read (those output rows were zero-filled).  Gathers are asynchronous, so the error surfaces
@@ -230,12 +234,14 @@ class ChunkTensor : public torch::CustomClassHolder {
   // (up to kMaxNodeTables; further streams get none and the call uses a hash table instead).
   // Two calls on the same stream share their table one after the other, which is only right if
   // all launches of the first precede all launches of the second: the caller holds
-  // enqueue_lock() from before this call until its last launch is enqueued.
+  // enqueue_lock() from before this call until node_table_used() behind its last launch that
+  // reads the table.
   std::unique_lock<std::mutex> enqueue_lock() { return std::unique_lock<std::mutex>(node_table_mutex_); }
   // When every table belongs to another stream, the caller takes over the one used longest ago
-  // among those whose stream has nothing left to run (a stream that is no longer used, such as
-  // one made per epoch).  If all of them are busy the caller gets no table and its call builds a
-  // hash table in its workspace.
+  // among those whose last call has finished (a stream that is no longer used, such as one made
+  // per epoch).  "Finished" is asked of a ticket recorded behind that call (node_table_used),
+  // never of the other stream's handle, which may have been destroyed since.  If all tables are
+  // busy the caller gets none and its call builds a hash table in its workspace.
   std::pair<void*, uint32_t> node_table(void* stream) {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
@@ -245,12 +251,13 @@ class ChunkTensor : public torch::CustomClassHolder {
       if (node_tables_.size() >= kMaxNodeTables) {
         auto pick = node_tables_.end();
         for (auto jt = node_tables_.begin(); jt != node_tables_.end(); ++jt) {
-          int32_t idle = 0;
-          check(dgs_stream_query(jt->first, &idle));
-          if (idle && (pick == node_tables_.end() || jt->second.last_use < pick->second.last_use)) pick = jt;
+          int32_t finished = 1;  // a table that was handed out and never used has nothing pending
+          if (jt->second.done != nullptr) check(dgs_ticket_query(jt->second.done, &finished));
+          if (finished && (pick == node_tables_.end() || jt->second.last_use < pick->second.last_use)) pick = jt;
         }
         if (pick == node_tables_.end()) return {nullptr, 0u};
         NodeTable taken = std::move(pick->second);
+        pick->second.done = nullptr;
         node_tables_.erase(pick);
         // the memory came from another stream's pool: it must not be handed out again while
         // this stream still uses it
@@ -270,6 +277,31 @@ class ChunkTensor : public torch::CustomClassHolder {
     }
     t.last_use = ++uses_;
     return {t.entries.data_ptr(), ++t.epoch};
+  }
+  // Marks the end of a call that used `stream`'s table: everything enqueued on the stream so far.
+  // (Called with enqueue_lock() held.)
+  void node_table_used(void* stream) {
+    auto it = node_tables_.find(stream);
+    if (it == node_tables_.end()) return;
+    if (it->second.done != nullptr) dgs_ticket_release(it->second.done);
+    it->second.done = nullptr;
+    check(dgs_ticket_record(stream, &it->second.done));
+  }
+  // Gives up the node table of a stream (0: the current stream), e.g. before the stream is
+  // destroyed; returns whether there was one.  Kernels of earlier calls that still use the table
+  // keep their memory: torch's allocator hands a block out again in stream order only.
+  bool ReleaseNodeTable(int64_t stream_handle) {
+    const std::unique_lock<std::mutex> lock = enqueue_lock();
+    void* key = stream_handle != 0 ? reinterpret_cast<void*>(static_cast<intptr_t>(stream_handle)) : current_stream();
+    auto it = node_tables_.find(key);
+    if (it == node_tables_.end()) return false;
+    if (it->second.done != nullptr) dgs_ticket_release(it->second.done);
+    node_tables_.erase(it);
+    return true;
+  }
+  int64_t NodeTableCount() {
+    const std::unique_lock<std::mutex> lock = enqueue_lock();
+    return static_cast<int64_t>(node_tables_.size());
   }
 
   const dgs_view& view() const { return view_; }
@@ -291,6 +323,7 @@ class ChunkTensor : public torch::CustomClassHolder {
     torch::Tensor entries;
     uint32_t epoch = 0;
     uint64_t last_use = 0;
+    void* done = nullptr;  // ticket behind the last call that used the table (null: never used)
   };
   uint64_t uses_ = 0;
   static constexpr size_t kMaxNodeTables = 4;
@@ -351,7 +384,7 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
         torch::empty({2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
     int64_t* words = pinned.data_ptr<int64_t>();
     words[0] = words[1] = -1;  // the kernel's words are never negative: the wait below polls them
-    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(), words,
+    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, indices.total, num_picks, replace, nnz_dev.data_ptr<int64_t>(), words,
                            ws.data_ptr(), ws_bytes, st));
     const dgs_status fill_status =
         probs != nullptr
@@ -364,7 +397,7 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor& seeds_
     TORCH_CHECK(words[0] >= 0 && words[1] >= 0, "sample_neighbors: the count kernel left no lengths");
     len.assign(words, words + 2);
   } else {
-    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, num_picks, replace, nnz_dev.data_ptr<int64_t>(), nullptr,
+    check(dgs_sample_count(seeds.data_ptr(), w, n, indptr, indices.total, num_picks, replace, nnz_dev.data_ptr<int64_t>(), nullptr,
                            ws.data_ptr(), ws_bytes, st));
     len = read_back(nnz_dev, 2);
     rows = torch::empty({len[0]}, seeds.options());
@@ -716,6 +749,7 @@ class PendingBlocks : public torch::CustomClassHolder {
                               replace, rng.first, rng.second, table.first, table.second, p->all_.data_ptr(),
                               outs.data(), sizes_dev.data_ptr<int64_t>(), p->pinned_.data_ptr<int64_t>(),
                               &p->ticket_, ws.data_ptr(), ws_bytes, st));
+    if (table.first != nullptr) indptr->node_table_used(st);  // the last launch above is the table's last reader
     if (features) {
       const auto xopt = torch::TensorOptions().dtype(features->dtype()).device(dev);
       const int64_t row_bytes = features->elem_stride() * static_cast<int64_t>(c10::elementSize(features->dtype()));
@@ -813,11 +847,18 @@ class BatchLoop : public torch::CustomClassHolder {
       check(dgs_stream_query(st, &idle));
       if (!idle) check(dgs_ticket_record(st, &item.seeds_ready));
     }
+    bool closed;
     {
       const std::lock_guard<std::mutex> lock(mutex_);
-      TORCH_CHECK(!stop_, "BatchLoop: closed");
-      input_.push_back(std::move(item));
-      ++pushed_;
+      closed = stop_;
+      if (!closed) {
+        input_.push_back(std::move(item));
+        ++pushed_;
+      }
+    }
+    if (closed) {  // the ticket taken above goes back before the call fails
+      if (item.seeds_ready) dgs_ticket_release(item.seeds_ready);
+      TORCH_CHECK(false, "BatchLoop: closed");
     }
     wake_worker_.notify_one();
   }
@@ -826,8 +867,11 @@ class BatchLoop : public torch::CustomClassHolder {
     Item item;
     {
       std::unique_lock<std::mutex> lock(mutex_);
+      TORCH_CHECK(!stop_, "BatchLoop: closed");
       TORCH_CHECK(popped_ < pushed_, "BatchLoop: nothing to pop");
-      wake_caller_.wait(lock, [this] { return !output_.empty(); });
+      // (a loop that is closed while this thread waits gives its pending batches up: the wait ends)
+      wake_caller_.wait(lock, [this] { return stop_ || !output_.empty(); });
+      TORCH_CHECK(!output_.empty(), "BatchLoop: closed");
       item = std::move(output_.front());
       output_.pop_front();
       ++popped_;
@@ -861,10 +905,20 @@ class BatchLoop : public torch::CustomClassHolder {
     }
     wake_worker_.notify_all();
     if (worker_.joinable()) worker_.join();
-    for (Item& item : input_)
+    std::deque<Item> unbegun, unclaimed;
+    {
+      // batches that were pushed and never popped are given up: nothing is pending afterwards, and a
+      // thread that waits in Pop is woken (it finds the loop closed)
+      const std::lock_guard<std::mutex> lock(mutex_);
+      unbegun.swap(input_);
+      unclaimed.swap(output_);
+      popped_ = pushed_;
+    }
+    wake_caller_.notify_all();
+    for (Item& item : unbegun)
       if (item.seeds_ready) dgs_ticket_release(item.seeds_ready);
-    input_.clear();
-    output_.clear();  // batches nobody asked for: their destructors wait for their kernels' lengths
+    unbegun.clear();
+    unclaimed.clear();  // batches nobody asked for: their destructors wait for their kernels' lengths
     for (void*& t : done_) {
       if (t) dgs_ticket_release(t);
       t = nullptr;
@@ -1069,7 +1123,10 @@ TORCH_LIBRARY(dgs_classes, m) {
       .def("_CAPI_host_index", &ChunkTensor::HostIndex)
       .def("_CAPI_load_from_tensor", &ChunkTensor::LoadFromTensor)
       // not in upstream: waits for the current stream, then raises if a gather met a bad row id
-      .def("_CAPI_synchronize_and_check", &ChunkTensor::SynchronizeAndCheck);
+      .def("_CAPI_synchronize_and_check", &ChunkTensor::SynchronizeAndCheck)
+      // not in upstream: the fused sampler's per-stream node tables of a graph's indptr store
+      .def("_CAPI_release_node_table", &ChunkTensor::ReleaseNodeTable)
+      .def("_CAPI_node_table_count", &ChunkTensor::NodeTableCount);
   // not in upstream: a sample_blocks call in flight
   m.class_<PendingBlocks>("PendingBlocks").def("_CAPI_finish", &PendingBlocks::Finish);
   // not in upstream: batches in flight, begun by a worker thread of the extension

@@ -50,13 +50,13 @@ dgs_status static_scratch_of(void** out) {
 
 constexpr int kMaxGroupPicks = 64;   // fill_group_kernel handles num_picks <= 64
 constexpr int kMaxLdsPicks = 2048;   // fill_wave_kernel keeps Floyd's set in LDS
-constexpr int kFlagDegree = 1;       // some row has degree >= 2^32
+constexpr int kFlagDegree = 1;       // some row has degree >= 2^32, or offsets outside the edge array
 constexpr int kFlagSeed = 2;         // some seed id is not a row of the graph
 
 template <typename IdT, typename PtrT>
 __global__ __launch_bounds__(kTile) void sample_count_kernel(
-    const IdT* __restrict__ seeds, int64_t n_seeds, TierView<PtrT> indptr, int64_t k, bool replace,
-    int64_t* __restrict__ row_start, uint32_t* __restrict__ row_deg, int64_t* __restrict__ row_off,
+    const IdT* __restrict__ seeds, int64_t n_seeds, TierView<PtrT> indptr, int64_t n_edges, int64_t k,
+    bool replace, int64_t* __restrict__ row_start, uint32_t* __restrict__ row_deg, int64_t* __restrict__ row_off,
     int64_t* __restrict__ tile_sum, int* __restrict__ tile_flag) {
   __shared__ int64_t lds[kTile / kWave];
   __shared__ int flag;
@@ -71,7 +71,8 @@ __global__ __launch_bounds__(kTile) void sample_count_kernel(
     if (row_in_range(indptr, row)) {  // checked before the offsets are read
       b = int64_t(indptr.at(row));
       deg = int64_t(indptr.at(row + 1)) - b;
-      if (deg < 0 || deg > 0xffffffffLL) { bad |= kFlagDegree; deg = 0; }
+      // offsets that leave the edge array are refused here, before the fill reads through them
+      if (deg < 0 || deg > 0xffffffffLL || b < 0 || b + deg > n_edges) { bad |= kFlagDegree; b = 0; deg = 0; }
     } else {
       bad |= kFlagSeed;
     }
@@ -264,12 +265,12 @@ __global__ __launch_bounds__(kTile) void fill_wave_global_kernel(
 }
 
 template <typename IdT, typename PtrT>
-dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr, int64_t k, bool replace,
-                     const SampleWorkspace& w, int64_t* nnz_dev, int64_t* nnz_host, hipStream_t st) {
+dgs_status run_count(const void* seeds, int64_t n_seeds, const dgs_view& indptr, int64_t n_edges, int64_t k,
+                     bool replace, const SampleWorkspace& w, int64_t* nnz_dev, int64_t* nnz_host, hipStream_t st) {
   const int64_t tiles = (n_seeds + kTile - 1) / kTile;
   if (tiles > 0) {
     hipLaunchKernelGGL((sample_count_kernel<IdT, PtrT>), dim3(uint32_t(tiles)), dim3(kTile), 0, st,
-                       static_cast<const IdT*>(seeds), n_seeds, TierView<PtrT>(indptr), k, replace,
+                       static_cast<const IdT*>(seeds), n_seeds, TierView<PtrT>(indptr), n_edges, k, replace,
                        w.row_start, w.row_deg, w.row_off, w.tile_sum, w.tile_flag);
     DGS_LAUNCH_CHECK();
   }
@@ -329,7 +330,7 @@ DGS_API size_t dgs_sample_workspace_bytes(int64_t n_seeds) {
 }
 
 DGS_API dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indptr,
-                                    int64_t num_picks, int32_t replace, int64_t* nnz_dev, int64_t* nnz_host,
+                                    int64_t n_edges, int64_t num_picks, int32_t replace, int64_t* nnz_dev, int64_t* nnz_host,
                                     void* workspace, size_t workspace_bytes, void* stream) {
   using namespace dgs;
   dgs_status s = check_sample_args("sample_count", seeds, id_bytes, n_seeds, num_picks, workspace, workspace_bytes);
@@ -337,15 +338,16 @@ DGS_API dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t
   DGS_REQUIRE(width_ok(indptr.elem_bytes), DGS_ERR_INVALID, "sample_count: indptr width %d is not 4 or 8",
               indptr.elem_bytes);
   DGS_REQUIRE(nnz_dev != nullptr, DGS_ERR_INVALID, "sample_count: null nnz_dev");
+  DGS_REQUIRE(n_edges >= 0, DGS_ERR_INVALID, "sample_count: n_edges=%lld", (long long)n_edges);
   hipStream_t st = static_cast<hipStream_t>(stream);
   SampleWorkspace w;
   sample_workspace_layout(n_seeds, workspace, &w);
   const bool rep = replace != 0;
   if (id_bytes == 8)
-    return indptr.elem_bytes == 8 ? run_count<int64_t, int64_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st)
-                                  : run_count<int64_t, int32_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st);
-  return indptr.elem_bytes == 8 ? run_count<int32_t, int64_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st)
-                                : run_count<int32_t, int32_t>(seeds, n_seeds, indptr, num_picks, rep, w, nnz_dev, nnz_host, st);
+    return indptr.elem_bytes == 8 ? run_count<int64_t, int64_t>(seeds, n_seeds, indptr, n_edges, num_picks, rep, w, nnz_dev, nnz_host, st)
+                                  : run_count<int64_t, int32_t>(seeds, n_seeds, indptr, n_edges, num_picks, rep, w, nnz_dev, nnz_host, st);
+  return indptr.elem_bytes == 8 ? run_count<int32_t, int64_t>(seeds, n_seeds, indptr, n_edges, num_picks, rep, w, nnz_dev, nnz_host, st)
+                                : run_count<int32_t, int32_t>(seeds, n_seeds, indptr, n_edges, num_picks, rep, w, nnz_dev, nnz_host, st);
 }
 
 DGS_API dgs_status dgs_sample_fill(const void* seeds, int32_t id_bytes, int64_t n_seeds, dgs_view indices,
@@ -373,7 +375,7 @@ DGS_API dgs_status dgs_sample_neighbors(const void* seeds, int32_t id_bytes, int
                                         int32_t replace, uint64_t rng_seed, uint32_t rng_stream,
                                         void* out_rows, void* out_cols, int64_t* nnz_dev, void* workspace,
                                         size_t workspace_bytes, void* stream) {
-  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, num_picks, replace, nnz_dev, nullptr, workspace,
+  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, indices.total, num_picks, replace, nnz_dev, nullptr, workspace,
                                   workspace_bytes, stream);
   if (s != DGS_OK) return s;
   return dgs_sample_fill(seeds, id_bytes, n_seeds, indices, num_picks, replace, rng_seed, rng_stream, out_rows,

@@ -58,7 +58,7 @@ DGS_API const char* dgs_status_name(dgs_status s) {
   }
 }
 
-DGS_API int dgs_abi_version(void) { return 2; }
+DGS_API int dgs_abi_version(void) { return 3; }
 
 DGS_API dgs_status dgs_debug_set(int32_t option, int64_t value) {
   DGS_REQUIRE(option >= 0 && option < dgs::kDebugOptions, DGS_ERR_INVALID, "debug_set: unknown option %d", option);
@@ -343,13 +343,34 @@ DGS_API dgs_status dgs_ticket_release(void* ticket) {
 
 DGS_API dgs_status dgs_stream_query(void* stream, int32_t* idle) {
   DGS_REQUIRE(idle != nullptr, DGS_ERR_INVALID, "stream_query: null output");
+  *idle = 0;
   const hipError_t e = hipStreamQuery(static_cast<hipStream_t>(stream));
-  if (e == hipErrorNotReady) {
-    *idle = 0;
+  if (e == hipErrorNotReady) return DGS_OK;
+  if (e == hipSuccess) {
+    *idle = 1;
     return DGS_OK;
   }
-  if (e != hipSuccess) (void)hipGetLastError();  // a handle that names no live stream: nothing can be pending on it
-  *idle = 1;
+  if (e == hipErrorInvalidHandle || e == hipErrorInvalidResourceHandle || e == hipErrorContextIsDestroyed) {
+    // the handle names no live stream: nothing can be pending on it.  Only this error is taken
+    // off the runtime's last-error slot; any other one stays there and is reported.
+    (void)hipGetLastError();
+    *idle = 1;
+    return DGS_OK;
+  }
+  dgs::set_error("stream_query: %s", hipGetErrorString(e));
+  return DGS_ERR_HIP;
+}
+
+DGS_API dgs_status dgs_ticket_query(void* ticket, int32_t* reached) {
+  DGS_REQUIRE(ticket != nullptr && reached != nullptr, DGS_ERR_INVALID, "ticket_query: null argument");
+  *reached = 0;
+  const hipError_t e = hipEventQuery(static_cast<hipEvent_t>(ticket));
+  if (e == hipErrorNotReady) return DGS_OK;
+  if (e != hipSuccess) {
+    dgs::set_error("ticket_query: %s", hipGetErrorString(e));
+    return DGS_ERR_HIP;
+  }
+  *reached = 1;
   return DGS_OK;
 }
 

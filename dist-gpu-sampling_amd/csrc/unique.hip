@@ -20,6 +20,11 @@ constexpr int kItems = 4;
 constexpr int kTileIds = kThreads * kItems;   // ids per block in flag / compact
 constexpr uint32_t kFirstBit = 0x80000000u;   // marks a first occurrence in slot[]
 constexpr int64_t kMaxMappingIds = int64_t(1) << 30;
+// slot[] word of a mapping id the table could not take (the call's results are void then: the
+// overflow word is set).  It lies beyond the mask of every table but the largest possible one
+// (2^31 slots), where it names a real slot; lookup_kernel checks a word against the mask, and what
+// the slot holds against the number of positions, before either is used as an index.
+constexpr uint32_t kNoSlot = 0x7fffffffu;
 
 // Element i of the logical concatenation, or of a single array when count == 1.
 template <typename IdT>
@@ -60,7 +65,7 @@ __global__ __launch_bounds__(kThreads) void insert_kernel(dgs_segments mapping, 
   const IdT key = seg_load<IdT>(mapping, i);
   if (!table.holds(key)) {
     *overflow = 1;
-    slot[i] = 0;  // some slot of the table, no first bit: the call's results are void anyway
+    slot[i] = kNoSlot;  // no slot, no first bit: the call's results are void, and a lookup through this word gives -1
     return;
   }
   bool first;
@@ -156,10 +161,13 @@ struct SegmentAlias {
 // words of the first occurrences (a streamed array), the table keeps every id's smallest
 // position: an element that is itself a first occurrence of the mapping list needs no random
 // read at all, any other one reads the table entry and then that position's word.
+// Nothing read from the table or from slot[] is used as an index before it has been checked: a
+// slot word must name a slot of the table, and the position a table entry holds must be one of
+// the n mapping positions (an entry that was never filled holds 0xffffffff).
 template <typename IdT, typename TableT>
 __global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring, int64_t m, TableT table,
-                                                          const uint32_t* __restrict__ slot, SegmentAlias alias,
-                                                          dgs_segments out) {
+                                                          const uint32_t* __restrict__ slot, int64_t n,
+                                                          SegmentAlias alias, dgs_segments out) {
   const int64_t j = int64_t(blockIdx.x) * kThreads + threadIdx.x;
   if (j >= m) return;
   int seg;
@@ -175,10 +183,13 @@ __global__ __launch_bounds__(kThreads) void lookup_kernel(dgs_segments requiring
     const IdT key = static_cast<const IdT*>(requiring.ptr[seg])[off];
     s = table.holds(key) ? table.find(key) : table.mask + 1;  // an id the table cannot hold is not in it
   }
-  IdT rank;
-  if (holds_rank) rank = IdT(s);
-  else if (s > table.mask) rank = IdT(-1);
-  else rank = IdT(slot[table.value(s)] & ~kFirstBit);
+  IdT rank = IdT(-1);
+  if (holds_rank) {
+    rank = IdT(s);
+  } else if (s <= table.mask) {
+    const uint32_t first_at = table.value(s);  // smallest mapping position of the id
+    if (int64_t(first_at) < n) rank = IdT(slot[first_at] & ~kFirstBit);
+  }
   static_cast<IdT*>(const_cast<void*>(out.ptr[seg]))[off] = rank;
 }
 
@@ -397,7 +408,7 @@ dgs_status run_unique_relabel(const dgs_segments& mapping, int64_t n, const dgs_
       }
     }
     hipLaunchKernelGGL((lookup_kernel<IdT, TableT>), dim3(uint32_t((m + kThreads - 1) / kThreads)), dim3(kThreads),
-                       0, st, requiring, m, table, w.slot, alias, out);
+                       0, st, requiring, m, table, w.slot, n, alias, out);
     DGS_LAUNCH_CHECK();
   }
   return DGS_OK;

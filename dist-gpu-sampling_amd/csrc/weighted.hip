@@ -234,7 +234,7 @@ DGS_API dgs_status dgs_sample_neighbors_weighted(const void* seeds, int32_t id_b
   DGS_REQUIRE(replace != 0 || num_picks <= dgs::kMaxWeightedPicks, DGS_ERR_UNSUPPORTED,
               "sample_neighbors_weighted: num_picks %lld above %d without replacement", (long long)num_picks,
               dgs::kMaxWeightedPicks);
-  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, num_picks, replace, nnz_dev, nullptr, workspace,
+  dgs_status s = dgs_sample_count(seeds, id_bytes, n_seeds, indptr, indices.total, num_picks, replace, nnz_dev, nullptr, workspace,
                                   workspace_bytes, stream);
   if (s != DGS_OK) return s;
   return dgs_sample_fill_weighted(seeds, id_bytes, n_seeds, indices, probs, num_picks, replace, rng_seed,

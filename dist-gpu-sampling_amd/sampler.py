@@ -7,6 +7,23 @@ from collections import deque, namedtuple
 
 import torch
 
+class _FastOps:
+    """torch.ops.dgs_ops.<name> by their C++ entries (`OpOverloadPacket._op`): the same callables
+    with the same arguments, results and errors, minus the packet's Python-side walk over the
+    arguments for FakeScriptObjects (export / compile tracing, which operators that block on
+    data-dependent sizes do not support anyway; 4 us a call).  Nothing of torch is modified."""
+
+    def __getattr__(self, name):
+        packet = getattr(torch.ops.dgs_ops, name)
+        entry = getattr(packet, "_op", None)
+        entry = entry if callable(entry) else packet
+        setattr(self, name, entry)
+        return entry
+
+
+fast_ops = _FastOps()
+
+
 # One message-flow block: edges (src_local[e] -> dst_local[e]); src_ids / dst_ids map
 # local to global node ids (upstream: block.srcdata[dgl.NID] / block.dstdata[dgl.NID]).
 Block = namedtuple("Block", ["src_local", "dst_local", "num_src", "num_dst", "src_ids", "dst_ids"])
@@ -43,13 +60,18 @@ def get_available_memory(device, reserved_mem, local_group=None):
     return int(max(available, 0))
 
 
+def cached_bytes_per_gpu(total_bytes, num_gpus, available_mem, cache_rate=1.0):
+    """chunktensor_sampler.py:40-42: int(min(total_bytes * cache_rate // num_gpus, available_mem))."""
+    return int(min(total_bytes * cache_rate // num_gpus, available_mem))
+
+
 def create_chunktensor(tensor, num_gpus, available_mem, cache_rate=1.0, root_rank=0, local_group=None):
-    """chunktensor_sampler.py:32-60: capacity per GPU =
-    int(min(total_bytes * cache_rate // num_gpus, available_mem))."""
+    """chunktensor_sampler.py:32-60: a store of the tensor's shape and dtype whose capacity per GPU
+    is cached_bytes_per_gpu(...), filled from the tensor."""
     if num_gpus != 1:
         raise ValueError("this build runs at world size 1")
     total_size = tensor.numel() * tensor.element_size()
-    cached_size_per_gpu = int(min(total_size * cache_rate // num_gpus, available_mem))
+    cached_size_per_gpu = cached_bytes_per_gpu(total_size, num_gpus, available_mem, cache_rate)
     chunk_tensor = torch.classes.dgs_classes.ChunkTensor(list(tensor.shape), tensor.dtype, cached_size_per_gpu)
     chunk_tensor._CAPI_load_from_tensor(tensor)
     return chunk_tensor
@@ -105,6 +127,9 @@ class ChunkTensorSampler:
         self._batches = 0
         self._count_lock = threading.Lock()
         self._loops = {}  # BatchPipeline's native loops (each with a worker thread), kept for reuse
+        # where the operators are looked up: their C++ entries, or torch.ops.dgs_ops itself (what
+        # an unmodified upstream harness calls through) when a caller sets that
+        self.ops = fast_ops
 
     def _first_stream(self, batch):
         """Stream of the first hop of a batch drawn from the sampler's own state."""
@@ -136,7 +161,7 @@ class ChunkTensorSampler:
                 finally:
                     torch.ops.dgs_ops._CAPI_set_rng_state(*saved)
         if self.fused:
-            frontiers, srcs, dsts, seeds = torch.ops.dgs_ops._CAPI_sample_blocks(
+            frontiers, srcs, dsts, seeds = self.ops._CAPI_sample_blocks(
                 seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace)
             return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts)
         return self._sample_blocks_per_hop(seed_nodes)
@@ -148,12 +173,12 @@ class ChunkTensorSampler:
         frontier = seeds
         for fan_out in reversed(self.fanouts):
             if self.chunk_probs is not None:
-                coo_row, coo_col = torch.ops.dgs_ops._CAPI_sample_neighbors_with_probs_with_chunk_tensor(
+                coo_row, coo_col = self.ops._CAPI_sample_neighbors_with_probs_with_chunk_tensor(
                     seeds, self.chunk_indptr, self.chunk_indices, self.chunk_probs, fan_out, self.replace)
             else:
-                coo_row, coo_col = torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor(
+                coo_row, coo_col = self.ops._CAPI_sample_neighbors_with_chunk_tensor(
                     seeds, self.chunk_indptr, self.chunk_indices, fan_out, self.replace)
-            frontier, (coo_row, coo_col) = torch.ops.dgs_ops._CAPI_tensor_relabel(
+            frontier, (coo_row, coo_col) = self.ops._CAPI_tensor_relabel(
                 [seeds, coo_col], [coo_row, coo_col])
             blocks.insert(0, Block(coo_col, coo_row, frontier.numel(), seeds.numel(), frontier, seeds))
             seeds = frontier
@@ -168,7 +193,7 @@ class ChunkTensorSampler:
             raise RuntimeError("submit() needs the fused path: every fanout <= 64")
         hop_fanouts = list(reversed(self.fanouts))
         rng = [] if self.seed is None else [self.seed, self._first_stream(batch)]
-        handle = torch.ops.dgs_ops._CAPI_sample_blocks_submit(
+        handle = self.ops._CAPI_sample_blocks_submit(
             seed_nodes, self.chunk_indptr, self.chunk_indices, self.chunk_probs, hop_fanouts, self.replace,
             chunk_features, rng, 0 if gather_after is None else gather_after.cuda_event)
         return PendingBatch(handle, seed_nodes, chunk_features is not None, torch.cuda.current_stream())
@@ -183,7 +208,7 @@ class ChunkTensorSampler:
             return frontier, seed_nodes, blocks, chunk_features._CAPI_index(frontier)
         if self.chunk_probs is not None or self.seed is not None:
             return self.submit(g, seed_nodes, chunk_features).result()
-        frontiers, srcs, dsts, x, seeds = torch.ops.dgs_ops._CAPI_sample_blocks_and_index(
+        frontiers, srcs, dsts, x, seeds = self.ops._CAPI_sample_blocks_and_index(
             seed_nodes, self.chunk_indptr, self.chunk_indices, list(reversed(self.fanouts)), self.replace,
             chunk_features)
         return frontiers[-1], seed_nodes, self._blocks(seeds, frontiers, srcs, dsts), x
@@ -193,14 +218,33 @@ _pipeline_streams = []
 _event_sets = {}  # streams of a pipeline -> spare (seeds ready, batch done) event lists
 
 
+OVERLAP_PROBE_BYTES = 1 << 30  # what the probe's long fill writes at most (a fill of some 300 us)
+
+
+def _overlap_scratch():
+    """The buffer streams_overlap fills: OVERLAP_PROBE_BYTES, or an eighth of the free device memory
+    if that is less; None when even 16 MiB cannot be had (the probe is skipped then)."""
+    try:
+        free = torch.cuda.mem_get_info()[0]
+        nbytes = min(OVERLAP_PROBE_BYTES, free // 8)
+        if nbytes < (16 << 20):
+            return None
+        return torch.empty(nbytes // 4, dtype=torch.float32, device="cuda")
+    except torch.cuda.OutOfMemoryError:
+        return None
+
+
 def streams_overlap(a, b, scratch=None):
     """Whether work on stream `b` can run while stream `a` is busy.  HIP spreads a process's streams
     over a few hardware queues (four by default), and two streams that land on the same queue run
     their kernels in submission order however independent they are.  Measured, not looked up: a
-    long fill is enqueued on `a`, a tiny one on `b`, and the host watches which finishes when."""
+    long fill is enqueued on `a`, a tiny one on `b`, and the host watches which finishes when.
+    Without memory for the long fill nothing can be measured and the answer is True."""
     import time
     if scratch is None:
-        scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB: a fill of some 300 us
+        scratch = _overlap_scratch()
+        if scratch is None:
+            return True
     tiny = torch.empty(64, dtype=torch.float32, device="cuda")
     done_a, done_b = torch.cuda.Event(), torch.cuda.Event()
     votes = 0
@@ -227,13 +271,15 @@ def pipeline_streams(n):
     it (at most four), so pipelines that come and go should not each bring new streams.
     A new stream joins only if it overlaps with every stream already chosen (streams_overlap):
     in a process that has made other streams before, freshly made ones may share a hardware queue.
-    After a few candidates without luck the next one is taken as it is."""
+    After a few candidates without luck, or when there is no memory to measure with, the next one
+    is taken as it is."""
     if len(_pipeline_streams) < n:
-        scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda") if _pipeline_streams or n > 1 else None
+        scratch = _overlap_scratch() if _pipeline_streams or n > 1 else None
         rejected = []  # kept alive until the choice is made, so that new candidates are new streams
         while len(_pipeline_streams) < n:
             candidate = torch.cuda.Stream()
-            if len(rejected) < 6 and not all(streams_overlap(s, candidate, scratch) for s in _pipeline_streams):
+            if (scratch is not None and len(rejected) < 6
+                    and not all(streams_overlap(s, candidate, scratch) for s in _pipeline_streams)):
                 rejected.append(candidate)
                 continue
             _pipeline_streams.append(candidate)

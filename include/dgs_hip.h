@@ -232,10 +232,13 @@ dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
  *              out_rows / out_cols and of `indices`)
  *   indptr   : view of N+1 offsets, elem_bytes 4 or 8
  *   indices  : view of E ids, elem_bytes == id_bytes
+ *   n_edges  : (dgs_sample_count) entries of the edge array the offsets point into
+ *              (indices.total); a row whose offsets leave [0, n_edges] is flagged
  *   nnz_dev  : device int64[2]; [0] receives the number of emitted edges,
- *              [1] flags: bit 0 = some row has degree >= 2^32, bit 1 = some
- *              seed id is not a row of the graph (the reference does not check;
- *              here the id is tested before it addresses indptr).  Flagged
+ *              [1] flags: bit 0 = some row has degree >= 2^32 or offsets outside
+ *              the edge array, bit 1 = some seed id is not a row of the graph (the
+ *              reference checks neither; here an id is tested before it addresses
+ *              indptr, and offsets before the fill uses them).  Flagged
  *              rows emit nothing; the caller reports DGS_ERR_RANGE.
  *              Every num_picks is served, as by the reference's reservoir
  *              kernel (src/cuda/rowwise_sampling.cu:42-99).
@@ -256,7 +259,7 @@ dgs_status dgs_split_index(dgs_view v, int64_t row_elems, const void* index,
  */
 size_t dgs_sample_workspace_bytes(int64_t n_seeds);
 dgs_status dgs_sample_count(const void* seeds, int32_t id_bytes, int64_t n_seeds,
-                            dgs_view indptr, int64_t num_picks, int32_t replace,
+                            dgs_view indptr, int64_t n_edges, int64_t num_picks, int32_t replace,
                             int64_t* nnz_dev, int64_t* nnz_host, void* workspace,
                             size_t workspace_bytes, void* stream);
 dgs_status dgs_sample_fill(const void* seeds, int32_t id_bytes, int64_t n_seeds,
@@ -544,10 +547,20 @@ dgs_status dgs_ticket_wait_words(void* ticket, const int64_t* words, int32_t n_w
 dgs_status dgs_stream_wait_words(void* stream, const int64_t* words, int32_t n_words);
 dgs_status dgs_ticket_release(void* ticket);
 /*
- * *idle = 1 when everything enqueued on `stream` so far has finished (also when the handle no
- * longer names a live stream: a destroyed stream has drained), else 0.  Never blocks.
+ * *idle = 1 when everything enqueued on `stream` so far has finished, else 0.  Never blocks.
+ * A handle that no longer names a live stream counts as drained (the runtime's "invalid handle"
+ * answer, and only that one, is taken as idle); any other failure of the query is DGS_ERR_HIP and
+ * stays visible to the caller's next HIP call.  Meant for streams the caller knows to be alive;
+ * to learn whether earlier work has finished without holding on to a stream, record a ticket
+ * behind it and ask dgs_ticket_query.
  */
 dgs_status dgs_stream_query(void* stream, int32_t* idle);
+/*
+ * *reached = 1 when the point a ticket marks has been reached, else 0.  Never blocks and does not
+ * retire the ticket.  A ticket belongs to the library, not to the stream it was recorded on, so
+ * the answer is well defined whatever has become of that stream since.
+ */
+dgs_status dgs_ticket_query(void* ticket, int32_t* reached);
 
 #ifdef __cplusplus
 }

@@ -33,7 +33,7 @@ def test_struct_layouts_match_the_header():
     pkg = load_pkg()
     assert ctypes.sizeof(pkg.capi.View) == 40      # 2 pointers + 2 int64 + 2 int32
     assert ctypes.sizeof(pkg.capi.Segments) == 8 * 8 + 8 * 8 + 8
-    assert pkg.capi.lib.dgs_abi_version() == 2
+    assert pkg.capi.lib.dgs_abi_version() == 3
 
 
 def test_store_split_matches_oracle(oracle):
@@ -80,25 +80,40 @@ def test_operator_surface_is_registered():
         torch.ops.dgs_ops._CAPI_set_nccl(2, [0] * 16, 1)
 
 
-def test_torch_dispatch_is_lightened_for_custom_class_arguments():
-    # importing the package opts torch.ScriptObject out of the __torch_function__ lookup (a miss
-    # costs two C++ exceptions per ChunkTensor argument per call) and binds the operators that
-    # take ChunkTensors to their C++ entry; DGS_PLAIN_TORCH_DISPATCH=1 leaves torch alone
+def test_torch_dispatch_is_left_alone_unless_asked():
+    # importing the package changes nothing of torch: torch.ScriptObject has no __torch_function__
+    # entry and every torch.ops.dgs_ops name is the packet torch made (schemas reachable);
+    # lighten_torch_dispatch() opts torch.ScriptObject out of the lookup (a miss costs two C++
+    # exceptions per ChunkTensor argument per call), lighten_torch_dispatch(False) takes that back;
+    # the package's own calls go to the packets' C++ entries without touching the packets
     import subprocess
     import sys
-    import torch
-    load_pkg()
-    assert vars(torch.ScriptObject)["__torch_function__"] is torch._C._disabled_torch_function_impl
-    assert type(torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor).__name__ == "builtin_function_or_method"
-    assert type(torch.ops.dgs_ops._CAPI_sample_neighbors).__name__ == "OpOverloadPacket"
-    code = ("import importlib, os, sys, torch; sys.path.insert(0, %r); importlib.import_module('dist-gpu-sampling_amd');"
-            "print('__torch_function__' in vars(torch.ScriptObject),"
-            " type(torch.ops.dgs_ops._CAPI_sample_neighbors_with_chunk_tensor).__name__)"
+    code = ("import importlib, os, sys, torch; sys.path.insert(0, %r);"
+            "had = '__torch_function__' in vars(torch.ScriptObject);"
+            "dgs = importlib.import_module('dist-gpu-sampling_amd');"
+            "name = '_CAPI_sample_neighbors_with_chunk_tensor';"
+            "print(had, '__torch_function__' in vars(torch.ScriptObject), type(getattr(torch.ops.dgs_ops, name)).__name__,"
+            " 'ChunkTensor' in str(getattr(torch.ops.dgs_ops, name).default._schema));"
+            "print(dgs.lighten_torch_dispatch(), vars(torch.ScriptObject).get('__torch_function__') is torch._C._disabled_torch_function_impl);"
+            "print(dgs.lighten_torch_dispatch(False), type(getattr(torch.ops.dgs_ops, name)).__name__);"
+            "print(type(getattr(dgs.fast_ops, name)).__name__, callable(dgs.fast_ops._CAPI_tensor_relabel))"
             % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-    out = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, DGS_PLAIN_TORCH_DISPATCH="1"),
+    env = {k: v for k, v in os.environ.items() if k != "DGS_LIGHT_TORCH_DISPATCH"}
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    lines = [line.split() for line in out.stdout.strip().splitlines()]
+    assert lines[0] == ["False", "False", "OpOverloadPacket", "True"]
+    assert lines[1] == ["True", "True"]
+    assert lines[2] == ["False", "OpOverloadPacket"]
+    assert lines[3] == ["builtin_function_or_method", "True"]
+    # asked for through the environment: in place after the import
+    code = ("import importlib, sys, torch; sys.path.insert(0, %r); importlib.import_module('dist-gpu-sampling_amd');"
+            "print('__torch_function__' in vars(torch.ScriptObject))"
+            % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    out = subprocess.run([sys.executable, "-c", code], env=dict(env, DGS_LIGHT_TORCH_DISPATCH="1"),
                          capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stderr
-    assert out.stdout.split() == ["False", "OpOverloadPacket"]
+    assert out.stdout.split() == ["True"]
 
 
 def test_no_gpu_means_a_loud_error_not_a_fallback():
@@ -111,14 +126,36 @@ def test_no_gpu_means_a_loud_error_not_a_fallback():
 
 
 def test_sampler_cache_size_formula():
-    # chunktensor_sampler.py:40-42: int(min(total_bytes * cache_rate // num_gpus, available_mem))
-    import inspect
+    # chunktensor_sampler.py:40-42: int(min(total_bytes * cache_rate // num_gpus, available_mem)), then
+    # chunk_tensor.cc:57-68: that many bytes / element size elements in HBM, at most all of them.
+    # Values worked out by hand, not by the formula's own text; the GPU suite checks the same numbers
+    # on real stores (test_gpu_store_gather.py::test_create_chunktensor_capacity).
+    import ctypes
+    import torch
     pkg = load_pkg()
-    src = inspect.getsource(pkg.create_chunktensor)
-    assert "total_size * cache_rate // num_gpus" in src
+    for total, rate, avail, want_bytes in [(4000, 1.0, 10 ** 9, 4000), (4000, 0.5, 10 ** 9, 2000), (4000, 0.3, 10 ** 9, 1200),
+                                           (4000, 0.333, 10 ** 9, 1332), (4000, 0.0, 10 ** 9, 0), (4000, 1.0, 1001, 1001),
+                                           (4001, 0.5, 10 ** 9, 2000), (979_611_600, 0.4, 1 << 40, 391_844_640)]:
+        got = pkg.cached_bytes_per_gpu(total, 1, avail, rate)
+        assert got == want_bytes and isinstance(got, int), (total, rate, avail, got)
+        for elem_bytes in (4, 8):
+            dev, host = ctypes.c_int64(), ctypes.c_int64()
+            pkg.capi.check(pkg.capi.lib.dgs_store_split(total // elem_bytes, elem_bytes, got, ctypes.byref(dev),
+                                                        ctypes.byref(host)))
+            assert dev.value == min(want_bytes // elem_bytes, total // elem_bytes)
+            assert dev.value + host.value == total // elem_bytes
     with pytest.raises(ValueError):
-        import torch
         pkg.create_chunktensor(torch.zeros(4), 2, 100)
+
+
+def test_query_entry_points_check_their_arguments():
+    # no GPU needed: null arguments are refused before any runtime call
+    import ctypes
+    capi = load_pkg().capi
+    flag = ctypes.c_int32(7)
+    assert capi.lib.dgs_stream_query(None, None) == capi.DGS_ERR_INVALID
+    assert capi.lib.dgs_ticket_query(None, ctypes.byref(flag)) == capi.DGS_ERR_INVALID
+    assert b"ticket_query" in capi.lib.dgs_last_error()
 
 
 def test_placement_host_arithmetic(oracle):

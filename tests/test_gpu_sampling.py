@@ -172,6 +172,24 @@ def test_neighbour_ids_outside_the_graph_are_refused(pkg, last_hop):
     ip_ct = pkg.create_chunktensor(torch.from_numpy(bad_ptr), 1, 1 << 40)
     with pytest.raises(RuntimeError, match="offsets outside"):
         pkg.ChunkTensorSampler([8], ip_ct, ix_ct).sample_blocks(None, torch.tensor([30]))
+    # the per-hop operators refuse such a row as well, before their fill reads through the offsets:
+    # stores, plain tensors, weighted picks, any fanout (group, wave and global fills)
+    seeds = torch.tensor([5, 30, 7]).cuda()
+    d_ptr, d_ix = torch.from_numpy(bad_ptr).cuda(), torch.from_numpy(indices).cuda()
+    d_w = torch.rand(indices.size, device="cuda")
+    for k in (8, 100, 3000):
+        for replace in (False, True):
+            with pytest.raises(RuntimeError, match="offsets outside"):
+                pkg.ChunkTensorSampler([k], ip_ct, ix_ct, replace=replace, fused=False).sample_blocks(None, seeds)
+            with pytest.raises(RuntimeError, match="offsets outside"):
+                pkg.ops._CAPI_sample_neighbors(seeds, d_ptr, d_ix, k, replace)
+    with pytest.raises(RuntimeError, match="offsets outside"):
+        pkg.ops._CAPI_sample_neighbors_with_probs(seeds, d_ptr, d_ix, d_w, 8, False)
+    # a row that ends exactly at the end of the edge array is fine
+    last = torch.tensor([n - 1]).cuda()
+    rows, cols = pkg.ops._CAPI_sample_neighbors(last, torch.from_numpy(indptr).cuda(), d_ix, 100, False)
+    assert cols.cpu().numpy().tolist() == indices[indptr[n - 1]:].tolist()
+    torch.cuda.synchronize()
 
 
 def test_capped_feature_buffer_gives_the_same_batch(pkg, oracle, graph, last_hop):
@@ -286,6 +304,19 @@ def test_node_tables_move_to_new_streams(pkg, oracle, graph):
         assert np.array_equal(_np(p.result()[0]), want[i % 4])
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() - base <= 4 * 8 * (indptr.size - 1) + (64 << 20)
+    # a stream's owner can give its table up (before destroying the stream, say): the memory goes
+    # back, and a stream that comes later gets a table of its own again
+    assert ip_ct._CAPI_node_table_count() == 4
+    released = 0
+    for st in streams:
+        released += int(ip_ct._CAPI_release_node_table(st.cuda_stream))
+    assert released >= 1 and ip_ct._CAPI_node_table_count() == 4 - released
+    assert not ip_ct._CAPI_release_node_table(streams[0].cuda_stream)  # gone already, or never had one
+    with torch.cuda.stream(streams[0]):
+        f, _, _ = sampler.sample_blocks(None, torch.from_numpy(seeds), batch=2)
+        assert np.array_equal(_np(f), want[2])
+        assert ip_ct._CAPI_release_node_table(0)  # 0: the current stream
+    torch.cuda.synchronize()
 
 
 def test_sample_with_chunk_tensor_tiers(pkg, oracle, graph):
@@ -706,6 +737,42 @@ def test_unique_relabel_ids_beyond_32_bits(pkg, oracle):
     assert _np(outs[0]).tolist() == [0, -1, -1]
 
 
+@pytest.mark.parametrize("n", [3000, 70000])
+def test_unique_relabel_of_a_tensor_on_both_sides_with_ids_the_table_cannot_hold(pkg, oracle, n):
+    # The upstream loop passes its picked neighbours as a mapping AND as a requiring tensor (the same
+    # device memory), and such a tensor is relabelled through the slot words its ids were given on
+    # insertion.  An id the table in use cannot hold gets no slot: the attempt on one-word slots
+    # (ids below 2^32 - 1) is void and repeated on the two-array table, and a negative id, which no
+    # table holds, makes the call fail cleanly.  Above 2048 ids, so that the table lives in HBM.
+    rng = np.random.default_rng(n)
+    seeds = rng.permutation(5000)[:64].astype(np.int64)
+    cols = rng.integers(0, 40000, size=n).astype(np.int64)
+    cols[::97] += 2 ** 33                      # ids beyond the one-word slots, spread over the list
+    cols[5] = cols[n - 1] = 2 ** 32 - 1        # the smallest such id, twice
+    rows = rng.choice(seeds, size=n).astype(np.int64)
+    want_u, (want_r, want_c) = oracle.unique_relabel([seeds, cols], [rows, cols])
+    d_seeds, d_cols, d_rows = _dev(seeds), _dev(cols), _dev(rows)
+    u, outs = pkg.ops._CAPI_tensor_relabel([d_seeds, d_cols], [d_rows, d_cols])
+    assert np.array_equal(_np(u), want_u) and np.array_equal(_np(outs[0]), want_r) and np.array_equal(_np(outs[1]), want_c)
+    u, outs = pkg.capi.unique_relabel([d_seeds, d_cols], [d_rows, d_cols])
+    assert np.array_equal(_np(u), want_u) and np.array_equal(_np(outs[0]), want_r) and np.array_equal(_np(outs[1]), want_c)
+    # the void attempt alone (what runs before the host has seen the overflow word): every output is
+    # a rank of the list or -1, nothing else was read
+    u, outs = pkg.capi.unique_relabel([d_seeds, d_cols], [d_rows, d_cols], packed_table=True, retry=False)
+    got = _np(outs[1])
+    assert ((got >= -1) & (got < n + 64)).all()
+    # a negative id among the mapped ones: no table holds it
+    bad = cols.copy()
+    bad[n // 2] = -7
+    d_bad = _dev(bad)
+    with pytest.raises(RuntimeError, match="rejected an id"):
+        pkg.ops._CAPI_tensor_relabel([d_seeds, d_bad], [d_rows, d_bad])
+    torch.cuda.synchronize()
+    # and the store is fine afterwards
+    u, outs = pkg.ops._CAPI_tensor_relabel([d_seeds, d_cols], [d_rows, d_cols])
+    assert np.array_equal(_np(u), want_u) and np.array_equal(_np(outs[1]), want_c)
+
+
 def test_pipeline_streams_do_not_share_a_hardware_queue(pkg):
     # a process that has made streams before (here: six of them) still gets pipeline streams that
     # run side by side; streams that share a hardware queue would run their batches one after the other
@@ -756,6 +823,43 @@ def test_batch_loop_of_the_extension_directly(pkg, oracle, graph):
     loop._CAPI_close()  # closing twice is fine
     with pytest.raises(RuntimeError, match="closed"):
         loop._CAPI_push(_dev(batches[0]), False, -1)
+
+
+def test_batch_loop_closed_with_batches_pending(pkg, graph):
+    # closing a loop gives up what was pushed and not popped: nothing is pending afterwards, a pop
+    # raises instead of waiting for a batch that will never come, and so does a push
+    indptr, indices = graph
+    big = 1 << 40
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    streams = pkg.pipeline_streams(2)
+    triples = []
+    for st in streams:
+        triples += [st.stream_id, st.device_index, st.device_type]
+    loop = torch.classes.dgs_classes.BatchLoop(ip_ct, ix_ct, None, [4, 6], False, None, triples, False, False, [])
+    rng = np.random.default_rng(4)
+    for i in range(6):  # more than the two streams take: some are begun, some still queued
+        loop._CAPI_push(_dev(rng.integers(0, 20000, size=200).astype(np.int64)), i < 2, -1)
+    frontiers, _, _, _, _ = loop._CAPI_pop()
+    assert frontiers[-1].numel() > 0 and loop._CAPI_pending() == 5
+    loop._CAPI_close()
+    assert loop._CAPI_pending() == 0
+    with pytest.raises(RuntimeError, match="closed"):
+        loop._CAPI_pop()
+    with pytest.raises(RuntimeError, match="closed"):
+        loop._CAPI_push(_dev(np.arange(10, dtype=np.int64)), True, -1)
+    torch.cuda.synchronize()
+    # a pipeline whose iteration is abandoned while its loop gets closed underneath ends, too
+    sampler = pkg.ChunkTensorSampler([6, 4], ip_ct, ix_ct)
+    pipe = pkg.BatchPipeline(sampler, None, inflight=2)
+    it = pipe([_dev(rng.integers(0, 20000, size=200).astype(np.int64)) for _ in range(5)])
+    next(it)
+    for entry in sampler._loops.values():
+        entry["loop"]._CAPI_close()
+    with pytest.raises(RuntimeError, match="closed"):
+        next(it)
+    it.close()
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("native_loop", [True, False])

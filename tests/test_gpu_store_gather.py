@@ -36,6 +36,28 @@ def test_readme_demo(pkg):
     assert pkg.ops._CAPI_get_current_allocated() == before
 
 
+def test_create_chunktensor_capacity(pkg):
+    # chunktensor_sampler.py:40-42 + chunk_tensor.cc:57-73 on real stores: the device slice holds
+    # int(min(total_bytes * cache_rate // 1, available_mem)) // element size elements (at most all),
+    # the host slice the rest; numbers worked out by hand for a [1000, 25] float32 tensor (100 000 B)
+    t = torch.arange(25000, dtype=torch.float32).reshape(1000, 25)
+    for rate, avail, want_dev in [(1.0, 1 << 40, 25000), (0.5, 1 << 40, 12500), (0.25, 1 << 40, 6250), (0.0, 1 << 40, 0),
+                                  (0.333, 1 << 40, 8325), (1.0, 30001, 7500), (0.1, 5000, 1250), (2.0, 1 << 40, 25000)]:
+        before = pkg.ops._CAPI_get_current_allocated()
+        ct = pkg.create_chunktensor(t, 1, avail, cache_rate=rate)
+        dev, host = ct._CAPI_get_sub_device_tensor(), ct._CAPI_get_host_tensor()
+        assert (dev.numel(), host.numel()) == (want_dev, 25000 - want_dev), (rate, avail)
+        assert pkg.ops._CAPI_get_current_allocated() - before == 4 * want_dev
+        assert torch.equal(dev.cpu(), t.reshape(-1)[:want_dev]) and torch.equal(host, t.reshape(-1)[want_dev:])
+        idx = torch.tensor([0, 999, 333, 332, 334, 500], device="cuda")  # rows around every boundary above
+        assert torch.equal(ct._CAPI_index(idx).cpu(), t[idx.cpu()])
+        del ct, dev, host
+    # an int64 store, as the harness makes for indptr / indices
+    t8 = torch.arange(1001, dtype=torch.int64)
+    ct = pkg.create_chunktensor(t8, 1, 1 << 40, cache_rate=0.4)
+    assert ct._CAPI_get_sub_device_tensor().numel() == 400  # 8008 * 0.4 // 1 = 3203 bytes -> 400 elements
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.int64, torch.int32, torch.bfloat16, torch.uint8,
                                    torch.float64, torch.bool])
 @pytest.mark.parametrize("rows,dim", [(257, 100), (64, 128), (1000, 1), (33, 7), (50, 256)])

@@ -1,6 +1,7 @@
 """The entry point that allocates nothing (dgs_sample_neighbors_static) against the entry point it is
-a variant of (dgs_sample_neighbors with a caller workspace): bit-exact rows, columns, edge count and
-flags, on calls that follow each other on one GPU and share the library's static scratch."""
+a variant of (dgs_sample_neighbors with a caller workspace) and against the CPU oracle: bit-exact
+rows, columns, edge count and flags, on calls that follow each other on one GPU and share the
+library's static scratch; and that such a call leaves every allocation count where it was."""
 import numpy as np
 import pytest
 import torch
@@ -24,7 +25,7 @@ def _static_call(capi, seeds, ipv, ixv, k, replace, rng_seed, rng_stream):
 
 
 @pytest.mark.parametrize("id_dtype,ptr_dtype", [(np.int64, np.int64), (np.int32, np.int64)])
-def test_static_entry_point_matches_the_workspace_one(id_dtype, ptr_dtype):
+def test_static_entry_point_matches_the_workspace_one(oracle, id_dtype, ptr_dtype):
     capi = load_pkg().capi
     rng = np.random.default_rng(77)
     indptr, indices = powerlaw_graph(rng, 30000, 20, 4000, id_dtype=id_dtype, ptr_dtype=ptr_dtype)
@@ -40,6 +41,44 @@ def test_static_entry_point_matches_the_workspace_one(id_dtype, ptr_dtype):
         assert got_flags == want_flags == 0
         assert got_r.numel() == want_r.numel() and got_c.numel() == want_c.numel()
         assert torch.equal(got_r, want_r) and torch.equal(got_c, want_c), (n_seeds, k, replace)
+        o_r, o_c = oracle.sample_neighbors(seeds.cpu().numpy(), indptr, indices, k, replace, 0xFEED5EED, 4)
+        assert np.array_equal(got_r.cpu().numpy(), o_r) and np.array_equal(got_c.cpu().numpy(), o_c)
+
+
+def test_static_entry_point_allocates_nothing(oracle):
+    # after a first call (which looks the scratch symbol's address up), calls through the C ABI with
+    # the caller's own output buffers leave the library's, torch's and the device's allocation
+    # counts where they were, whatever the input size
+    pkg = load_pkg()
+    capi = pkg.capi
+    rng = np.random.default_rng(78)
+    indptr, indices = powerlaw_graph(rng, 20000, 20, 2000)
+    ip, ix = _dev(indptr), _dev(indices)
+    ipv, ixv = capi.tensor_view(ip), capi.tensor_view(ix)
+    k, n_max = 12, 30000
+    rows = torch.empty(n_max * k, dtype=torch.int64, device="cuda")
+    cols = torch.empty(n_max * k, dtype=torch.int64, device="cuda")
+    nnz = torch.empty(2, dtype=torch.int64, device="cuda")
+    all_seeds = _dev(rng.integers(0, 20000, size=n_max))
+    stream = capi.stream_ptr()
+
+    def call(n):
+        capi.check(capi.lib.dgs_sample_neighbors_static(all_seeds.data_ptr(), 8, n, ipv, ixv, k, 0, 21, 3,
+                                                        rows.data_ptr(), cols.data_ptr(), nnz.data_ptr(), stream))
+    for n in (100, n_max):  # warm-up: resolves the symbol on this device, loads the kernels
+        call(n)
+    torch.cuda.synchronize()
+    before = (capi.lib.dgs_current_allocated(), torch.cuda.memory_allocated(), torch.cuda.memory_reserved(),
+              torch.cuda.mem_get_info()[0])
+    for n in (n_max, 17, 4097):
+        call(n)
+        torch.cuda.synchronize()
+        after = (capi.lib.dgs_current_allocated(), torch.cuda.memory_allocated(), torch.cuda.memory_reserved(),
+                 torch.cuda.mem_get_info()[0])
+        assert after == before, (n, before, after)
+    cnt = int(nnz[0].item())
+    o_r, o_c = oracle.sample_neighbors(all_seeds[:4097].cpu().numpy(), indptr, indices, k, False, 21, 3)
+    assert cnt == o_r.size and np.array_equal(rows[:cnt].cpu().numpy(), o_r) and np.array_equal(cols[:cnt].cpu().numpy(), o_c)
 
 
 def test_static_entry_point_rejects_what_does_not_fit():
