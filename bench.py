@@ -24,6 +24,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+PCIE_PEAK_GBPS = 64.0   # PCIe Gen5 x16, one direction
 GATHER_SOURCE = os.path.join(ROOT, "dist-gpu-sampling_amd", "csrc", "gather.hip")
 GATHER_TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gather_flat_kernel_c1_pmc.txt")
 
@@ -327,11 +328,11 @@ LARGE = {
 }
 
 
-def run_large(args, dgs):
-    """Benchmark configurations 2 to 4, built on the device.  For the two-tier case (c3) the tiers
-    are also timed separately: device tier against HBM, host tier against PCIe Gen5 x16."""
-    cfg = LARGE[args.workload]
-    scale = args.scale
+def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8):
+    """Benchmark configurations 2 to 4, built on the device; returns the result record.  For the
+    two-tier case (c3) the tiers are also timed separately: device tier against HBM, host tier
+    against PCIe Gen5 x16."""
+    cfg = LARGE[name]
     n, e = int(cfg["nodes"] * scale), int(cfg["edges"] * scale)
     dim, fanouts, batch = cfg["dim"], cfg["fanouts"], cfg["batch"]
     gen = torch.Generator(device="cuda").manual_seed(cfg["seed"])
@@ -358,7 +359,7 @@ def run_large(args, dgs):
         m = min(chunk, host.numel() - a)
         stage[:m].normal_(generator=gen)
         host[a: a + m].copy_(stage[:m])
-    del stage
+    del stage, dev, host
     torch.cuda.synchronize()
     t_gen = time.perf_counter() - t0
     sampler = dgs.ChunkTensorSampler(fanouts, ct_ip, ct_ix, replace=cfg["replace"])
@@ -366,32 +367,72 @@ def run_large(args, dgs):
     if cfg["train_frac"] < 1.0:  # seeds come from a fixed uniform subset of the nodes
         pool = torch.randperm(n, generator=gen, device="cuda")[: int(n * cfg["train_frac"])].to(torch.int32)
     seeds = []
-    for _ in range(args.steps + args.warmup):
+    for _ in range(steps + warmup):
         r = torch.randint(0, n if pool is None else pool.numel(), (batch,), generator=gen, device="cuda")
         seeds.append(r.to(torch.int32) if pool is None else pool[r])
     dgs.set_rng_state(cfg["seed"], 0)
     # the two-tier case gathers tens of GB per batch: one batch at a time
-    inflight = args.inflight if cfg["hbm_rows"] >= 1.0 else 1
-    run_batches(sampler, seeds[:args.warmup], ct_x, inflight)
+    two_tier = cfg["hbm_rows"] < 1.0
+    inflight = inflight if not two_tier else 1
+    run_batches(sampler, seeds[:warmup], ct_x, inflight)
+    if inflight > 1:  # the allocator's per-stream pools see every buffer size before anything is timed
+        run_batches(sampler, (seeds * 4)[:4 * inflight + warmup], ct_x, inflight)
     torch.cuda.synchronize()
     frontiers = []  # the first few, for the gather leg below; of the other batches only the lengths are kept
+
     def keep(r):
-        if len(frontiers) < 8:
+        if len(frontiers) < stage_batches:
             frontiers.append(r[0])
-        return r[0].numel(), sum(b.src_local.numel() for b in r[2])
+        return {"frontier": r[0].numel(),
+                "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]}
     resident = torch.cuda.memory_allocated()
     torch.cuda.reset_peak_memory_stats()
     t0 = time.perf_counter()
-    results = run_batches(sampler, seeds[args.warmup:], ct_x, inflight, keep)
+    results = run_batches(sampler, seeds[warmup:], ct_x, inflight, keep)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     peak_batch_bytes = torch.cuda.max_memory_allocated() - resident
-    rows = sum(r[0] for r in results)
-    edges = sum(r[1] for r in results)
-    frontier = frontiers[-1]
+    rows = sum(r["frontier"] for r in results)
+    edges = sum(sum(h[1] for h in r["hops"]) for r in results)
     row_bytes = dim * eb
+
+    def total_bytes(all_stats):
+        bs = bu = bg = 0
+        for st in all_stats:
+            a, b, c = algorithmic_bytes(st, dim, eb, w_id=4, w_ptr=8)
+            bs, bu, bg = bs + a, bu + b, bg + c
+        return bs, bu, bg
+    bs, bu, bg = total_bytes(results)
+    # one batch at a time on one stream, call to result (what upstream's own loop, num_workers=0, sees)
+    ms_alone = None
+    if inflight > 1:
+        n_alone = min(steps, 10)
+        run_batches(sampler, seeds[:2], ct_x, 1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_batches(sampler, seeds[warmup:warmup + n_alone], ct_x, 1, keep)
+        torch.cuda.synchronize()
+        ms_alone = 1e3 * (time.perf_counter() - t0) / n_alone
+    # stage split: the sampler alone (events on the launching stream around the fused call), then
     # the gather alone, once per kept frontier (a repeat of the same rows would be served by the
-    # 256 MB last-level cache), events on the launching stream, queued back to back
+    # 256 MB last-level cache), queued back to back
+    n_stage = min(steps, stage_batches)
+    sample_ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(n_stage)]
+    stage_stats = []
+    sampler.sample_blocks(None, seeds[0])
+    torch.cuda.synchronize()
+    for i in range(n_stage):
+        sample_ev[i][0].record()
+        r = sampler.sample_blocks(None, seeds[warmup + i])
+        sample_ev[i][1].record()
+        stage_stats.append({"frontier": r[0].numel(),
+                            "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]})
+        del r
+    torch.cuda.synchronize()
+    ms_sample = float(np.mean([a.elapsed_time(b) for a, b in sample_ev]))
+    sbs, sbu, _ = total_bytes(stage_stats)
+    sampler_gbps = (sbs + sbu) / n_stage / (ms_sample * 1e-3) / 1e9
+    frontier = frontiers[-1]
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in frontiers]
     ct_x._CAPI_index(frontiers[-1][:1024])
     torch.cuda.synchronize()
@@ -402,26 +443,44 @@ def run_large(args, dgs):
         del x
     torch.cuda.synchronize()
     t_mixed = sum(a.elapsed_time(b) for a, b in ev) * 1e-3
-    gather_gbps = sum(f.numel() for f in frontiers) * (2 * row_bytes + 4) / t_mixed / 1e9
+    gather_bytes = sum(f.numel() for f in frontiers) * (2 * row_bytes + 4)
+    gather_gbps = gather_bytes / t_mixed / 1e9
     t_mixed /= len(frontiers)
+    step_gbps = (bs + bu + bg) / elapsed / 1e9
     out = {
         "metric": "sampled edges/s (sampling + relabel + feature gather per batch), 1 MI355X",
-        "value": edges / elapsed, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": 1e3 * elapsed / args.steps, "higher_is_better": True, "scaling": "weak",
+        "value": edges / elapsed, "unit": "edges/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": 1e3 * elapsed / steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {cfg['graph']} graph, {n} nodes / {e} edges CSC int64+int32, "
+        "config": {"workload": f"{name}: {cfg['graph']} graph, {n} nodes / {e} edges CSC int64+int32, "
                                f"features {str(cfg['feat_dtype']).split('.')[-1]} x{dim} ({n * row_bytes / 1e9:.1f} GB), "
                                f"{int(100 * cfg['hbm_rows'])}% of rows in HBM, batch {batch}, fanouts {fanouts}, "
                                f"{'with' if cfg['replace'] else 'without'} replacement", "scale": scale,
                    "batches_in_flight": inflight},
-        "avg_frontier_rows": rows / args.steps, "avg_edges_per_batch": edges / args.steps,
+        "ms_per_batch_alone": ms_alone,
+        "edges_per_s": edges / elapsed,
+        "avg_frontier_rows": rows / steps, "avg_edges_per_batch": edges / steps,
+        "ms_sample_relabel": ms_sample,
         "gather_ms": 1e3 * t_mixed, "gather_GBps": gather_gbps, "graph_gen_s": t_gen,
+        "step_algorithmic_GBps": step_gbps, "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
+        "stages": [
+            {"stage": "sampling + relabel of every hop (fused sampler kernels, one batch alone on one stream)",
+             "bound": "hbm", "achieved": sampler_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": sampler_gbps / HBM_PEAK_GBPS, "algorithmic_bytes": (sbs + sbu) / n_stage, "avg_us": 1e3 * ms_sample},
+            {"stage": "feature gather of the last frontier (gather_flat_kernel), both tiers as the store holds them",
+             "bound": "hbm", "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": gather_gbps / HBM_PEAK_GBPS, "algorithmic_bytes": gather_bytes / len(frontiers),
+             "avg_us": 1e6 * t_mixed},
+            {"stage": "whole step as timed", "bound": "hbm", "achieved": step_gbps, "peak": HBM_PEAK_GBPS,
+             "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes": (bs + bu + bg) / steps,
+             "avg_us": 1e6 * elapsed / steps},
+        ],
         # torch allocations of the batches in flight at their peak (outputs, workspaces, kept frontiers),
         # beyond what was resident before the timed loop; the stores themselves are not torch memory
         "peak_batch_bytes": peak_batch_bytes,
         "gather_buffer_cap_bytes": int(torch.ops.dgs_ops._CAPI_get_gather_buffer_cap()),
     }
-    if cfg["hbm_rows"] < 1.0:
+    if two_tier:
         local, _, host_ids = ct_x._CAPI_split_index(frontier)
         t_local = time_call(lambda: ct_x._CAPI_local_index(local), 5)
         t_host = time_call(lambda: ct_x._CAPI_host_index(host_ids), 3)
@@ -430,8 +489,9 @@ def run_large(args, dgs):
         out.update({
             "frontier_rows_device_tier": local.numel(), "frontier_rows_host_tier": host_ids.numel(),
             "device_tier_gather_GBps": dev_gbps, "device_tier_ms": 1e3 * t_local,
+            "device_tier_hbm_frac": dev_gbps / HBM_PEAK_GBPS,
             "host_tier_gather_GBps": host_gbps, "host_tier_ms": 1e3 * t_host,
-            "host_tier_peak_GBps": 64.0, "host_tier_pcie_frac": host_gbps / 64.0,
+            "host_tier_peak_GBps": PCIE_PEAK_GBPS, "host_tier_pcie_frac": host_gbps / PCIE_PEAK_GBPS,
             "roofline": {"bound": "hbm", "kernel": "gather_flat_kernel (_CAPI_local_index, device tier)",
                          "achieved": dev_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": dev_gbps / HBM_PEAK_GBPS, "traffic": None},
@@ -440,7 +500,16 @@ def run_large(args, dgs):
         out["roofline"] = {"bound": "hbm", "kernel": "gather_flat_kernel (_CAPI_index)", "achieved": gather_gbps,
                            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gather_gbps / HBM_PEAK_GBPS,
                            "traffic": None}
-    print(json.dumps(out), flush=True)
+    return out
+
+
+def release_everything():
+    """Between workloads: pipelines (and their samplers' worker threads), cached blocks."""
+    import gc
+    _pipelines.clear()
+    gc.collect()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
 
 
 def main():
@@ -457,6 +526,11 @@ def main():
                     help="largest feature buffer the fused operator allocates ahead of a batch's sizes "
                          "(the library's default when not given)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="with --workload c1: do not also run c1w, c2, c4 and c3 after the headline")
+    ap.add_argument("--other-steps", type=int, default=20, help="timed batches of each other workload")
+    ap.add_argument("--other-budget-s", type=float, default=300.0,
+                    help="no further workload is started once this much time has gone into them")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a known-size kernel to scale "
@@ -474,7 +548,9 @@ def main():
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
     if args.workload in LARGE:
-        return run_large(args, dgs)
+        print(json.dumps(measure_large(args.workload, dgs, args.steps, args.warmup, args.inflight, args.scale)),
+              flush=True)
+        return
     cfg = WORKLOADS[args.workload]
     t0 = time.perf_counter()
     indptr, indices, feats, _ = make_graph(cfg)
@@ -545,11 +621,19 @@ def main():
                                  if inflight > 1 else None)
     # what an unmodified upstream harness runs: per hop one sampling operator and one relabel
     # operator (each returns tensors of exact length, so each waits for its lengths), then _CAPI_index
+    # -- called through torch.ops.dgs_ops with torch as it is, which is what such a harness does
     per_hop = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, ct_probs, replace=cfg["replace"],
                                      fused=False)
+    per_hop.ops = torch.ops.dgs_ops
     ms_per_hop_ops = 1e3 * timed_steps(per_hop, batches, 1)[0] / args.steps
     # the same loop without its last line: the sampling and relabel operators alone
     ms_per_hop_ops_no_gather = 1e3 * timed_steps(per_hop, batches, 1, features=None)[0] / args.steps
+    # the same loop again with the package's two opt-in shortcuts through torch's Python front end
+    # (lighten_torch_dispatch, and the operators' C++ entries instead of their packets)
+    per_hop.ops = dgs.fast_ops
+    dgs.lighten_torch_dispatch(True)
+    ms_per_hop_ops_light = 1e3 * timed_steps(per_hop, batches, 1)[0] / args.steps
+    dgs.lighten_torch_dispatch(False)
 
     # Stage split and the dominant kernel's duration, on the same batches: events on torch's
     # current stream (the one the C ABI launches on) around the sampler call and around the
@@ -628,6 +712,7 @@ def main():
         "ms_per_step_handed_over_host_seeds": ms_handed_over_host_seeds,
         "ms_per_step_per_hop_ops": ms_per_hop_ops,
         "ms_per_step_per_hop_ops_no_gather": ms_per_hop_ops_no_gather,
+        "ms_per_step_per_hop_ops_light_dispatch": ms_per_hop_ops_light,
         "timings": {"ms_per_step_repeats": "the timed region run three more times (spread)",
                     "ms_per_batch_alone": "one batch at a time, one stream, call to result",
                     "ms_per_step_handed_over": "as the headline, each batch handed to the calling stream "
@@ -636,7 +721,12 @@ def main():
                     "ms_per_step_handed_over_host_seeds": "host seeds in, each batch handed to the calling stream",
                     "ms_per_step_per_hop_ops": "upstream's own loop: _CAPI_sample_neighbors_with_chunk_tensor + "
                                                "_CAPI_tensor_relabel per hop, then _CAPI_index, one batch at a time",
-                    "ms_per_step_per_hop_ops_no_gather": "that loop without _CAPI_index: the six operator calls alone"},
+                    "ms_per_step_per_hop_ops_no_gather": "that loop without _CAPI_index: the six operator calls alone",
+                    "ms_per_step_per_hop_ops_light_dispatch": "that loop (with _CAPI_index) after "
+                                                              "lighten_torch_dispatch(), operators called by their C++ entries",
+                    "what_an_unmodified_harness_sees": "ms_per_step_per_hop_ops (one batch at a time through the "
+                                                       "upstream operator names); the headline needs the added "
+                                                       "fused operator and batches in flight"},
         "sample_edges_per_s": stage_edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
         "ms_sample_relabel": ms_sample,
@@ -688,6 +778,72 @@ def main():
         cb = cpu_baseline(cfg, indptr, indices, feats, batches_cpu[args.warmup:], args.cpu_budget_s, probs)
         out["cpu_baseline"] = cb
         out["gpu_over_cpu"] = out["value"] / cb["value"]
+        # leg by leg, each GPU stage alone on one stream against the same stage of the CPU run
+        out["gpu_over_cpu_per_leg"] = {
+            "sampling_relabel": out["sample_edges_per_s"] / cb["sample_edges_per_s"],
+            "gather": out["gather_GBps"] / cb["gather_GBps"],
+            "note": "stage alone on the GPU (events around it) over the same stage on the CPU"}
+    if args.workload == "c1" and not args.no_other_workloads:
+        # The other benchmark configurations, after the headline and never at its cost: a leg that
+        # fails becomes {"error": ...}.  c1w reuses this graph (c1 + a float32 weight per edge).
+        others = {}
+        t_others = time.perf_counter()
+        k_other, w_other = args.other_steps, min(args.warmup, 3)
+
+        def guarded(name, fn):
+            if time.perf_counter() - t_others > args.other_budget_s:
+                others[name] = {"skipped": f"the {args.other_budget_s:.0f} s for the other workloads were used up"}
+                return
+            t0 = time.perf_counter()
+            try:
+                others[name] = fn()
+                others[name]["leg_wall_s"] = time.perf_counter() - t0
+            except Exception as err:  # noqa: BLE001 (whatever it is, the headline stands)
+                others[name] = {"error": f"{type(err).__name__}: {err}"[:500]}
+            release_everything()
+
+        def c1w_leg():
+            w = make_weights(cfg, indices.numel())
+            ct_w = dgs.create_chunktensor(w, 1, big)
+            smp = dgs.ChunkTensorSampler(cfg["fanouts"], ct_indptr, ct_indices, ct_w, replace=cfg["replace"])
+            some = batches[:k_other + args.warmup]
+            run_batches(smp, (some * 4)[:64], ct_feats, inflight, sizes)
+            torch.cuda.synchronize()
+            el, st = timed_steps(smp, some, inflight)
+            el_alone, _ = timed_steps(smp, some, 1)
+            ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(k_other)]
+            st_stats = []
+            for i in range(k_other):
+                ev[i][0].record()
+                r = smp.sample_blocks(None, some[args.warmup + i])
+                ev[i][1].record()
+                st_stats.append(sizes(r))
+                del r
+            torch.cuda.synchronize()
+            ms_s = float(np.mean([a.elapsed_time(b) for a, b in ev]))
+            wbs, wbu, wbg = total_bytes(st)
+            tbs, tbu, _ = total_bytes(st_stats)
+            w_edges = sum(sum(h[1] for h in x["hops"]) for x in st)
+            weight_bytes = 0  # every weight of every sampled row is read: not counted, as for the uniform picks
+            return {"config": {"workload": "c1w: c1 with a float32 weight per edge, weighted picks in every hop "
+                                           "(dgs_sample_blocks_weighted), then the same gather",
+                               "batches_in_flight": inflight},
+                    "steps": k_other, "ms_per_step": 1e3 * el / k_other, "ms_per_batch_alone": 1e3 * el_alone / k_other,
+                    "edges_per_s": w_edges / el, "gather_GBps": gather_gbps,
+                    "step_algorithmic_GBps": (wbs + wbu + wbg + weight_bytes) / el / 1e9,
+                    "step_hbm_frac": (wbs + wbu + wbg + weight_bytes) / el / 1e9 / HBM_PEAK_GBPS,
+                    "ms_sample_relabel": ms_s,
+                    "stages": [{"stage": "weighted sampling + relabel of every hop, one batch alone on one stream",
+                                "bound": "valu (the races), priced against hbm", "achieved": (tbs + tbu) / k_other / (ms_s * 1e-3) / 1e9,
+                                "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                "frac": (tbs + tbu) / k_other / (ms_s * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                "algorithmic_bytes": (tbs + tbu) / k_other, "avg_us": 1e3 * ms_s}]}
+
+        guarded("c1w", c1w_leg)
+        for name in ("c2", "c4", "c3"):
+            guarded(name, lambda name=name: measure_large(name, dgs, k_other, w_other, 3))
+        out["other_workloads"] = others
+        out["other_workloads_wall_s"] = time.perf_counter() - t_others
     print(json.dumps(out), flush=True)
 
 
