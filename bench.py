@@ -460,6 +460,9 @@ def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8
         "ms_per_batch_alone": ms_alone,
         "edges_per_s": edges / elapsed,
         "avg_frontier_rows": rows / steps, "avg_edges_per_batch": edges / steps,
+        # per hop, in hop order: seeds, sampled edges, frontier size afterwards (averages over the timed batches)
+        "avg_hops": [[float(np.mean([r["hops"][h][j] for r in results])) for j in range(3)]
+                     for h in range(len(fanouts))],
         "ms_sample_relabel": ms_sample,
         "gather_ms": 1e3 * t_mixed, "gather_GBps": gather_gbps, "graph_gen_s": t_gen,
         "step_algorithmic_GBps": step_gbps, "step_hbm_frac": step_gbps / HBM_PEAK_GBPS,
@@ -525,6 +528,9 @@ def main():
     ap.add_argument("--gather-buffer-cap-gib", type=float, default=None,
                     help="largest feature buffer the fused operator allocates ahead of a batch's sizes "
                          "(the library's default when not given)")
+    ap.add_argument("--node-table-max-nodes", type=int, default=None,
+                    help="graphs above this many nodes sample on a per-call hash table instead of persistent "
+                         "node tables (the library's default when not given)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with --workload c1: do not also run c1w, c2, c4 and c3 after the headline")
@@ -547,6 +553,8 @@ def main():
         args.inflight = 3 if args.workload in LARGE else 4
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
+    if args.node_table_max_nodes is not None:
+        torch.ops.dgs_ops._CAPI_set_node_table_max_nodes(args.node_table_max_nodes)
     if args.workload in LARGE:
         print(json.dumps(measure_large(args.workload, dgs, args.steps, args.warmup, args.inflight, args.scale)),
               flush=True)

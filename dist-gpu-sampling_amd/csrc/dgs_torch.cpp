@@ -89,6 +89,11 @@ std::pair<uint64_t, uint32_t> next_rng(uint32_t calls = 1) {
 // for the frontier's size and allocates exactly (see PendingBlocks::Begin).
 std::atomic<int64_t> g_gather_buffer_cap{int64_t(2) << 30};
 
+// Node tables (8 bytes per node and stream, persistent) for the fused operators: graphs up to this
+// many nodes get them, larger ones build a hash table per call in the call's workspace.
+// -1: every graph that dgs_node_table_bytes accepts (below 8 GiB per table).
+std::atomic<int64_t> g_node_table_max_nodes{-1};
+
 // What the error bits of a sampling call mean (include/dgs_hip.h, sizes_dev / nnz_dev flags).
 void check_sampling_flags(int64_t flags, const char* who, int hop) {
   if (flags == 0) return;
@@ -246,6 +251,8 @@ class ChunkTensor : public torch::CustomClassHolder {
     const int64_t n_nodes = total_ - 1;
     const size_t bytes = dgs_node_table_bytes(n_nodes);
     if (bytes == 0 || bytes > (size_t(8) << 30)) return {nullptr, 0u};
+    const int64_t max_nodes = g_node_table_max_nodes.load();
+    if (max_nodes >= 0 && n_nodes > max_nodes) return {nullptr, 0u};
     auto it = node_tables_.find(stream);
     if (it == node_tables_.end()) {
       if (node_tables_.size() >= kMaxNodeTables) {
@@ -1085,6 +1092,10 @@ void SetGatherBufferCap(int64_t bytes) {
 }
 int64_t GetGatherBufferCap() { return g_gather_buffer_cap.load(); }
 
+// Largest graph (nodes) whose fused calls use persistent node tables; -1: no limit of its own.
+void SetNodeTableMaxNodes(int64_t nodes) { g_node_table_max_nodes.store(nodes < 0 ? -1 : nodes); }
+int64_t GetNodeTableMaxNodes() { return g_node_table_max_nodes.load(); }
+
 int64_t GetCurrentAllocated() { return dgs_current_allocated(); }
 
 // upstream nccl::GetUniqueId / nccl::SetNCCL (src/nccl_context.cc:17-34): there is no
@@ -1159,6 +1170,8 @@ TORCH_LIBRARY(dgs_ops, m) {
       .def("_CAPI_sample_blocks_submit", &dgs::SampleBlocksSubmit)
       .def("_CAPI_set_gather_buffer_cap", &dgs::SetGatherBufferCap)
       .def("_CAPI_get_gather_buffer_cap", &dgs::GetGatherBufferCap)
+      .def("_CAPI_set_node_table_max_nodes", &dgs::SetNodeTableMaxNodes)
+      .def("_CAPI_get_node_table_max_nodes", &dgs::GetNodeTableMaxNodes)
       // not in upstream: node renumbering (hottest rows first) for the positional stores
       .def("_CAPI_renumber_csc", &dgs::RenumberCSC)
       // not in upstream: the sampling generator's (seed, stream)

@@ -136,6 +136,11 @@ __device__ __forceinline__ int64_t seeds_of(const Hop& h) {
 __device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h.index == 0 ? s : 0; }
 // rank of the first id this hop can add: later hops append behind their seeds
 __device__ __forceinline__ int64_t first_rank(const Hop& h, int64_t s) { return h.index == 0 ? 0 : s; }
+// the wave-local search for repeated draws of a row (fill_rows): entries per wave, and the longest
+// row, in multiples of the fanout, that is searched (k draws from 4 k positions repeat one in nine)
+constexpr int kFoldSlotBits = 7;
+constexpr int kFoldSlots = 1 << kFoldSlotBits;
+constexpr int kFoldMaxRowPerPick = 4;
 constexpr int kRelabelItems = 4;  // padded picks per thread in relabel_tile
 __host__ __device__ __forceinline__ int relabel_groups(int k) { return (k + kRelabelItems - 1) / kRelabelItems; }
 
@@ -327,30 +332,38 @@ __device__ __forceinline__ void mark_lost(const Hop& h, uint32_t displaced) {
   if (displaced != kNoPosition) h.lost[displaced] = 1;
 }
 
-// What becomes of padded position p: with a pick (edge `edge` of the graph) the picked id goes
-// into the table and p's slot word is recorded; without one the position is marked empty.
-// Returns false when the picked id is one the table cannot hold (the position then stays empty
-// and the caller marks the row bad): the id is checked before it addresses anything.
+// The slot word of padded position p, which holds a pick of neighbour id `col`: the id goes into
+// the table (or, in a bucketed hop, into the word itself).  Returns false, and the word of an empty
+// position, when the id is one the table cannot hold (the caller marks the row bad): the id is
+// checked before it addresses anything.
+template <typename IdT, typename TableT>
+__device__ __forceinline__ bool place_pick(const Hop& h, const TableT& table, IdT col, int64_t p, bool look_first,
+                                           uint32_t* word) {
+  *word = kInvalidSlot;
+  if (!table.holds(col)) return false;
+  if (h.bucketed) {
+    *word = uint32_t(col) | kFirstBit;  // a first occurrence until the bucketed pass says otherwise; the table is left alone
+    return true;
+  }
+  bool first;
+  uint32_t displaced;
+  uint32_t w = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
+  if (h.index != 0) {
+    if (first) w |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
+    mark_lost(h, displaced);
+  }
+  *word = w;
+  return true;
+}
+
+// What becomes of padded position p: with a pick (edge `edge` of the graph) the picked id is placed
+// and p's slot word recorded; without one the position is marked empty.
 template <typename IdT, typename TableT>
 __device__ __forceinline__ bool emit_pick(const Hop& h, const TableT& table, const TierView<IdT>& indices, int64_t p,
                                           bool have, int64_t edge, bool look_first) {
   uint32_t word = kInvalidSlot;
   bool ok = true;
-  if (have) {
-    const IdT col = indices.at(edge);
-    ok = table.holds(col);
-    if (ok && h.bucketed) {
-      word = uint32_t(col) | kFirstBit;  // a first occurrence until the bucketed pass says otherwise; the table is left alone
-    } else if (ok) {
-      bool first;
-      uint32_t displaced;
-      word = table.insert_min(col, uint32_t(p), &first, &displaced, look_first);
-      if (h.index != 0) {
-        if (first) word |= kFirstBit;  // provisional: cleared by flag() if the position gets lost
-        mark_lost(h, displaced);
-      }
-    }
-  }
+  if (have) ok = place_pick<IdT>(h, table, indices.at(edge), p, look_first, &word);
   h.slot[p] = word;
   return ok;
 }
@@ -377,6 +390,15 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   const int l = int(gid % G);
   // a launch sized far beyond the hop: blocks past its end wait for nothing but the length
   if (!EARLY && vb != 0 && vb * (kBlock / G) >= seeds_of(h)) return;
+  // the wave's table for the search for repeated draws (below) is emptied here, where every lane
+  // of the wave is still present
+  __shared__ unsigned long long fold_lds[kBlock / kWave][kFoldSlots];
+  const bool fold = replace && !h.bucketed;
+  if (fold) {
+    unsigned long long* offers = fold_lds[threadIdx.x / kWave];
+#pragma unroll
+    for (int q = 0; q < kFoldSlots / kWave; ++q) offers[q * kWave + (threadIdx.x & (kWave - 1))] = ~0ull;
+  }
   // the hop's length, what the previous hop found, and this group's seed id, requested together
   // (the seed list has room for s_max ids whatever the length turns out to be)
   const IdT seed = i < h.s_max ? static_cast<const IdT*>(h.seeds)[i] : IdT(0);
@@ -406,8 +428,47 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   }
   uint32_t pos;
   const bool have = pick_position<G>(deg, k, replace, l, group_lane0, words, &pos);
+  const bool live = l < k && have;
+  const int64_t p = h.pos_base + seed_part(h, s) + i * k + l;
+  // Draws with replacement repeat positions: on a row shorter than k most slots do.  Only the
+  // lowest slot of each position reads the edge array and goes to the table; a repeat can never be
+  // its id's smallest position, so it takes its leader's id and slot word (without the first bit)
+  // and touches nothing.  Repeats are found through a small table of the wave's own in LDS: every
+  // slot of the row offers (position, lane) to the entry its position hashes to, the smallest
+  // offer stays, and a slot that then reads its own position with a lower lane of its row has found
+  // its leader.  Two positions that meet in one entry cost a missed repeat, never a wrong one.
+  // Long rows (whose draws rarely repeat) skip the search.
+  int leader = l;
+  if (fold) {
+    unsigned long long* offers = fold_lds[threadIdx.x / kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool search = live && deg <= uint32_t(kFoldMaxRowPerPick * k);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint32_t entry = ((pos + uint32_t(group_lane0) * 0x9E3779B1u) * 0x85EBCA6Bu) >> (32 - kFoldSlotBits);
+    if (search) atomicMin(&offers[entry], (static_cast<unsigned long long>(pos) << 8) | uint32_t(lane));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (search) {
+      const unsigned long long best = offers[entry];
+      const int best_lane = int(best & 255u);
+      if (uint32_t(best >> 8) == pos && best_lane < lane && best_lane >= group_lane0) leader = best_lane - group_lane0;
+    }
+  }
+  uint32_t word = kInvalidSlot;
   bool pick_ok = true;
-  if (l < k) pick_ok = emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, have, b + pos, look_first);
+  if (live && leader == l) pick_ok = place_pick<IdT>(h, table, indices.at(b + pos), p, look_first, &word);
+  if (fold) {
+    const uint32_t leader_word = __shfl(word, leader, G);
+    const int leader_ok = __shfl(int(pick_ok), leader, G);
+    if (live && leader != l) {
+      word = leader_word == kInvalidSlot ? kInvalidSlot : (leader_word & ~kFirstBit);
+      pick_ok = leader_ok != 0;
+    }
+  }
+  if (l < k) h.slot[p] = word;
   constexpr uint64_t group_mask = G == 64 ? ~uint64_t(0) : ((uint64_t(1) << (G & 63)) - 1);
   const bool picks_ok = ((__ballot(!pick_ok) >> group_lane0) & group_mask) == 0;
   if (l == 0)
