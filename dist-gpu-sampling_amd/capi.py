@@ -56,7 +56,7 @@ SIGNATURES = {
                                         ctypes.POINTER(c_vp), ctypes.POINTER(c_i64)]),
     "dgs_current_allocated": (c_i64, []),
     "dgs_gather_rows": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i32, c_vp, c_vp]),
-    "dgs_gather_rows_dyn": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_i32, c_vp, c_vp]),
+    "dgs_gather_rows_dyn": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i32, c_vp, c_vp]),
     "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
     "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_workspace_bytes": (c_sz, [c_i64]),
@@ -324,7 +324,7 @@ def unique_relabel(mapping, requiring, packed_table=True, polled=False, retry=Tr
 
 def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_seed, first_stream,
                   feature_view=None, feature_row_elems=None, feature_dtype=None, node_table=None, epoch=0,
-                  probs_view=None):
+                  probs_view=None, gather_expected=0):
     """All hops in one call (picks by the edge weights `probs_view` when given).  Returns [(frontier, src_local, dst_local) per hop], the gathered
     rows of the last frontier when a feature view is given, and the per-hop error flags.
     `node_table` is an int64 device tensor of dgs_node_table_bytes(n_nodes) bytes filled with -1."""
@@ -362,7 +362,8 @@ def sample_blocks(seeds, indptr_view, indices_view, hop_fanouts, replace, rng_se
     if feature_view is not None:
         x = torch.empty((smax[hops], feature_row_elems), dtype=feature_dtype, device=seeds.device)
         check(lib.dgs_gather_rows_dyn(feature_view, feature_row_elems, frontier.data_ptr(), w, smax[hops],
-                                      sizes.data_ptr() + 8 * hops, x.data_ptr(), TIER_ANY, None, stream_ptr()))
+                                      sizes.data_ptr() + 8 * hops, gather_expected, x.data_ptr(), TIER_ANY, None,
+                                      stream_ptr()))
     sz = read_i64(sizes, 3 * hops + 1)
     result = [(frontier[:sz[h + 1]], s[:sz[hops + 1 + h]], d[:sz[hops + 1 + h]]) for h, (s, d) in enumerate(bufs)]
     if x is not None:

@@ -48,16 +48,22 @@ __device__ __forceinline__ const char* resolve(const char* dev, const char* host
 // (cpr + kChunksPerBlock) * cpr < 2^32, guaranteed by kMaxFlatChunksPerRow).
 // Rows [row_lo, row_hi) are the ones the launch may read; the range is not empty.
 //
-// The kChunksPerBlock output chunks from chunk c0 on (c0 < total_chunks); returns whether an
-// index outside [row_lo, row_hi) was met.
+// The kChunksPerBlock output chunks from chunk c0 on; returns whether an index outside
+// [row_lo, row_hi) was met.
 // Three passes, each over all of the thread's chunks, so that nothing but the row ids, then
 // nothing but the chunks themselves, is alive across the waits: the row ids (all requested
 // before any is used), the loads, the stores.
+// `readable_chunks` bounds the ids that may be read (the index array holds that many rows' ids
+// whatever the count turns out to be); the number of chunks that count is `total_chunks`, or, when
+// `n_rows_dev` is given, is read from the device here, together with the ids: a block of a launch
+// that is about as large as the work does not wait for the count before it asks for its ids.
 template <int VEC, int TIER, typename IndexT>
 __device__ __forceinline__ bool gather_tile(const char* __restrict__ dev, const char* __restrict__ host,
                                             int64_t thr_bytes, int64_t row_bytes, uint32_t cpr, uint32_t magic,
-                                            const IndexT* __restrict__ index, int64_t total_chunks, int64_t row_lo,
-                                            int64_t row_hi, char* __restrict__ out, int64_t c0) {
+                                            const IndexT* __restrict__ index, int64_t readable_chunks,
+                                            int64_t total_chunks, const int64_t* __restrict__ n_rows_dev,
+                                            int64_t row_lo, int64_t row_hi, char* __restrict__ out, int64_t c0,
+                                            int64_t* counted_chunks) {
   using C = typename Chunk<VEC>::type;
   bool bad = false;
   const int64_t row0 = c0 / cpr;
@@ -71,19 +77,27 @@ __device__ __forceinline__ bool gather_tile(const char* __restrict__ dev, const 
     const uint32_t lc = rem0 + t;
     const uint32_t q = cpr == 1 ? lc : __umulhi(lc, magic);
     off[u] = (lc - q * cpr) * uint32_t(VEC);
-    src[u] = c0 + t < total_chunks ? int64_t(index0[q]) : row_lo;  // past the end: some row, never stored
+    src[u] = c0 + t < readable_chunks ? int64_t(index0[q]) : row_lo;  // past the end: some row, never stored
   }
+  if (n_rows_dev) {  // row count decided on the device; one that exceeds the output's rows gathers nothing
+    const int64_t rows = *n_rows_dev;
+    total_chunks = rows >= 0 && rows * cpr <= readable_chunks ? rows * cpr : 0;
+  }
+  *counted_chunks = total_chunks;
+  if (c0 >= total_chunks) return false;  // whole blocks leave together
   // An id outside [row_lo, row_hi) is replaced by row_lo before it addresses anything (the
   // launcher guarantees that row_lo is a row the tier holds), and what was read for it is
-  // dropped: no branch around the loads, so all of them are in flight together.
+  // dropped: no branch around the loads, so all of them are in flight together.  The same goes
+  // for the ids behind the last chunk that counts (whatever the index array holds there).
   C val[kGatherUnroll];
   bool in_range[kGatherUnroll];
 #pragma unroll
   for (int u = 0; u < kGatherUnroll; ++u) {
+    const bool counts = c0 + u * kGatherThreads + threadIdx.x < total_chunks;
     in_range[u] = src[u] >= row_lo && src[u] < row_hi;
-    if (!in_range[u]) {
+    if (!in_range[u] || !counts) {
       src[u] = row_lo;
-      bad |= c0 + u * kGatherThreads + threadIdx.x < total_chunks;
+      bad |= counts;
     }
     const int64_t g = src[u] * row_bytes + int64_t(off[u]);
     val[u] = *reinterpret_cast<const C*>(resolve<TIER>(dev, host, thr_bytes, g));
@@ -100,29 +114,28 @@ __device__ __forceinline__ bool gather_tile(const char* __restrict__ dev, const 
   return bad;
 }
 
-// STRIDE: the grid is smaller than the tile count (capped launch) and blocks stride over the
-// tiles; otherwise a block has exactly one tile and no loop in its instruction stream.
+// STRIDE: the grid is smaller than the tile count (a launch sized for fewer rows than the output
+// holds) and blocks stride over the tiles; otherwise a block has exactly one tile and no loop in
+// its instruction stream.  `total_chunks` is the launch's worst case: what the index array and the
+// output hold.
 template <int VEC, int TIER, typename IndexT, bool STRIDE>
 __global__ __launch_bounds__(kGatherThreads) void gather_flat_kernel(
     const char* __restrict__ dev, const char* __restrict__ host, int64_t thr_bytes,
     int64_t row_bytes, uint32_t cpr, uint32_t magic, const IndexT* __restrict__ index,
     int64_t total_chunks, const int64_t* __restrict__ n_rows_dev, int64_t row_lo, int64_t row_hi,
     int64_t* __restrict__ bad_index, char* __restrict__ out) {
-  if (n_rows_dev) {  // row count decided on the device; one that exceeds the output's rows gathers nothing
-    const int64_t rows = *n_rows_dev;
-    total_chunks = rows >= 0 && rows * cpr <= total_chunks ? rows * cpr : 0;
-  }
-  bool bad = false;
-  if (STRIDE) {
-    for (int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock; c0 < total_chunks;
-         c0 += int64_t(gridDim.x) * kChunksPerBlock)
-      bad |= gather_tile<VEC, TIER, IndexT>(dev, host, thr_bytes, row_bytes, cpr, magic, index, total_chunks, row_lo,
-                                            row_hi, out, c0);
-  } else {
-    const int64_t c0 = int64_t(blockIdx.x) * kChunksPerBlock;
-    if (c0 < total_chunks)
-      bad = gather_tile<VEC, TIER, IndexT>(dev, host, thr_bytes, row_bytes, cpr, magic, index, total_chunks, row_lo,
-                                           row_hi, out, c0);
+  const int64_t first = int64_t(blockIdx.x) * kChunksPerBlock;
+  if (first >= total_chunks) return;
+  int64_t counted;
+  bool bad = gather_tile<VEC, TIER, IndexT>(dev, host, thr_bytes, row_bytes, cpr, magic, index, total_chunks,
+                                            total_chunks, n_rows_dev, row_lo, row_hi, out, first, &counted);
+  if (STRIDE) {  // the count is known from here on
+    for (int64_t c0 = first + int64_t(gridDim.x) * kChunksPerBlock; c0 < counted;
+         c0 += int64_t(gridDim.x) * kChunksPerBlock) {
+      int64_t unused;
+      bad |= gather_tile<VEC, TIER, IndexT>(dev, host, thr_bytes, row_bytes, cpr, magic, index, counted, counted,
+                                            nullptr, row_lo, row_hi, out, c0, &unused);
+    }
   }
   if (bad && bad_index) *bad_index = 1;
 }
@@ -158,7 +171,7 @@ __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
 
 template <int VEC, int TIER, typename IndexT>
 dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index, int64_t n,
-                         const int64_t* n_dev, int64_t* bad_index, void* out, hipStream_t st) {
+                         const int64_t* n_dev, int64_t n_expected, int64_t* bad_index, void* out, hipStream_t st) {
   const int64_t cpr = row_bytes / VEC;
   const int64_t thr_bytes = v.threshold * v.elem_bytes;
   // rows the tier holds whole: the device tier the rows that end at or before the boundary, the
@@ -172,7 +185,13 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
     const int64_t total_chunks = n * cpr;
     const int64_t tiles = (total_chunks + kChunksPerBlock - 1) / kChunksPerBlock;
     int64_t blocks = tiles;
-    if (n_dev != nullptr && blocks > kMaxDynGrid) blocks = kMaxDynGrid;
+    if (n_dev != nullptr) {
+      // a count read on the device: the launch is sized for the rows the caller expects (all of
+      // them when it says nothing), and blocks stride should there be more
+      if (n_expected > 0 && n_expected < n) blocks = (n_expected * cpr + kChunksPerBlock - 1) / kChunksPerBlock;
+      if (blocks > kMaxDynGrid) blocks = kMaxDynGrid;
+      if (blocks > tiles) blocks = tiles;
+    }
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;
     const uint32_t magic = cpr > 1 ? uint32_t((uint64_t(1) << 32) / uint64_t(cpr)) + 1u : 0u;
     int64_t lds = debug_option(DGS_DEBUG_GATHER_LDS_BYTES);
@@ -202,22 +221,22 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
 
 template <int VEC, int TIER>
 dgs_status dispatch_index(const dgs_view& v, int64_t row_bytes, const void* index,
-                          int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t* bad, void* out,
-                          hipStream_t st) {
-  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, bad, out, st)
-                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, bad, out, st);
+                          int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t n_expected, int64_t* bad,
+                          void* out, hipStream_t st) {
+  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, n_expected, bad, out, st)
+                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, n_expected, bad, out, st);
 }
 
 template <int TIER>
 dgs_status dispatch_vec(int vec, const dgs_view& v, int64_t row_bytes, const void* index,
-                        int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t* bad, void* out,
-                        hipStream_t st) {
+                        int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t n_expected, int64_t* bad,
+                        void* out, hipStream_t st) {
   switch (vec) {
-    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
-    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
-    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
-    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
-    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
   }
 }
 
@@ -318,7 +337,8 @@ __global__ __launch_bounds__(kSplitThreads) void split_scatter_kernel(
 
 namespace {
 dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_t index_bytes, int64_t n,
-                        const int64_t* n_dev, void* out, int32_t tier, int64_t* bad, void* stream) {
+                        const int64_t* n_dev, int64_t n_expected, void* out, int32_t tier, int64_t* bad,
+                        void* stream) {
   using namespace dgs;
   DGS_REQUIRE(width_ok(index_bytes), DGS_ERR_INVALID, "gather: index width %d is not 4 or 8", index_bytes);
   DGS_REQUIRE(n >= 0 && row_elems > 0, DGS_ERR_INVALID, "gather: n=%lld row_elems=%lld", (long long)n,
@@ -342,9 +362,9 @@ dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_
   const int vec = pick_vec(v, row_bytes, out, tier);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (tier) {
-    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
-    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
-    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, bad, out, st);
+    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
   }
 }
 }  // namespace
@@ -352,14 +372,15 @@ dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_
 DGS_API dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
                                    int32_t index_bytes, int64_t n, void* out, int32_t tier,
                                    int64_t* bad_index, void* stream) {
-  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, out, tier, bad_index, stream);
+  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, 0, out, tier, bad_index, stream);
 }
 
 DGS_API dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
                                        int32_t index_bytes, int64_t n_max, const int64_t* n_rows_dev,
-                                       void* out, int32_t tier, int64_t* bad_index, void* stream) {
+                                       int64_t n_expected, void* out, int32_t tier, int64_t* bad_index,
+                                       void* stream) {
   DGS_REQUIRE(n_rows_dev != nullptr, DGS_ERR_INVALID, "gather_dyn: null n_rows_dev");
-  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, out, tier, bad_index, stream);
+  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, n_expected, out, tier, bad_index, stream);
 }
 
 DGS_API size_t dgs_split_index_workspace_bytes(int64_t n) {

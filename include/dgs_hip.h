@@ -179,17 +179,20 @@ dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
 
 /*
  * Same gather with the row count read from device memory when the kernel runs:
- * `n_rows_dev` points to an int64; the launch is sized for n_max rows and `out` must
- * hold n_max rows.  A count above n_max (or below 0) gathers nothing at all, so a
- * caller may offer a buffer smaller than the worst case and gather again, exactly,
- * when the count turns out not to fit.  Lets a caller enqueue the gather of a frontier
- * whose length a previous kernel on the same stream is still computing.  No
- * counterpart in the reference (which reads every length back to the host first).
+ * `n_rows_dev` points to an int64; `index` must hold n_max readable ids (whatever the count turns
+ * out to be, the kernel may read all of them) and `out` n_max rows.  A count above n_max (or
+ * below 0) gathers nothing at all, so a caller may offer a buffer smaller than the worst case and
+ * gather again, exactly, when the count turns out not to fit.  Lets a caller enqueue the gather
+ * of a frontier whose length a previous kernel on the same stream is still computing.
+ * `n_expected` sizes the launch: the number of rows the caller expects (the previous batch's
+ * count plus a margin, say); 0 or less, or more than n_max: n_max.  It is a hint only: any count
+ * up to n_max is gathered in full, by blocks that loop when there are more rows than expected.
+ * No counterpart in the reference (which reads every length back to the host first).
  */
 dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
                                int32_t index_bytes, int64_t n_max,
-                               const int64_t* n_rows_dev, void* out, int32_t tier,
-                               int64_t* bad_index, void* stream);
+                               const int64_t* n_rows_dev, int64_t n_expected, void* out,
+                               int32_t tier, int64_t* bad_index, void* stream);
 
 /*
  * Stable partition of an index list into (device-resident rows, host-resident

@@ -287,12 +287,49 @@ def test_gather_dyn_leaves_a_buffer_alone_that_is_too_small(pkg, dim):
     idx = torch.randint(0, rows, (100,), device="cuda")
     out = torch.full((n_max + 1, dim), -3.0, device="cuda")
     for count, written in ((41, 0), (100, 0), (-1, 0), (40, 40), (7, 7), (0, 0)):
-        out.fill_(-3.0)
-        n_dev = torch.tensor([count], dtype=torch.int64, device="cuda")
-        capi.check(capi.lib.dgs_gather_rows_dyn(st.view, dim, idx.data_ptr(), 8, n_max, n_dev.data_ptr(), out.data_ptr(),
-                                                capi.TIER_ANY, None, capi.stream_ptr()))
-        assert torch.equal(out[:written].cpu(), full[idx[:written].cpu()]), count
-        assert (out[written:] == -3.0).all().item(), count
+        for expected in (0, 1, 7, 40, 1000):  # how many rows the launch is sized for: a hint, never a limit
+            out.fill_(-3.0)
+            n_dev = torch.tensor([count], dtype=torch.int64, device="cuda")
+            capi.check(capi.lib.dgs_gather_rows_dyn(st.view, dim, idx.data_ptr(), 8, n_max, n_dev.data_ptr(), expected,
+                                                    out.data_ptr(), capi.TIER_ANY, None, capi.stream_ptr()))
+            assert torch.equal(out[:written].cpu(), full[idx[:written].cpu()]), (count, expected)
+            assert (out[written:] == -3.0).all().item(), (count, expected)
+    st.close()
+
+
+@pytest.mark.parametrize("dtype,dim", [(torch.float32, 100), (torch.bfloat16, 128), (torch.float32, 3)])
+def test_gather_dyn_with_more_rows_than_expected(pkg, dtype, dim):
+    # a launch sized for far fewer rows than turn up (its blocks loop), for about as many, and for
+    # more: the same rows come out; the ids behind the count are readable but never used (they
+    # name no row of the store here), and a bad id inside the count is still refused
+    capi = pkg.capi
+    rows = 30000
+    full = torch.randn((rows, dim)).to(dtype)
+    st = capi.Store(rows * dim, full.element_size(), rows * dim * full.element_size() // 3)  # both tiers
+    st.load(full)
+    view = st.view
+    n_max = 50000
+    idx = torch.randint(0, rows, (n_max,), device="cuda", dtype=torch.int32)
+    bad = torch.zeros(1, dtype=torch.int64, device="cuda")
+    out = torch.empty((n_max, dim), dtype=dtype, device="cuda")
+    for count in (0, 1, 999, 20011, n_max):
+        tail = idx.clone()
+        tail[count:] = 2 ** 31 - 1  # what lies behind the count is no row id at all
+        for expected in (0, 1, 300, count, count + count // 4 + 1024, 10 ** 9):
+            out.fill_(-3.0)
+            bad.zero_()
+            n_dev = torch.tensor([count], dtype=torch.int64, device="cuda")
+            capi.check(capi.lib.dgs_gather_rows_dyn(view, dim, tail.data_ptr(), 4, n_max, n_dev.data_ptr(), expected,
+                                                    out.data_ptr(), capi.TIER_ANY, bad.data_ptr(), capi.stream_ptr()))
+            assert torch.equal(out[:count].cpu(), full[idx[:count].cpu().long()]), (count, expected)
+            assert (out[count:] == -3.0).all().item() and bad.item() == 0, (count, expected)
+    tail = idx.clone()
+    tail[17] = rows  # one past the last row, inside the count
+    n_dev = torch.tensor([100], dtype=torch.int64, device="cuda")
+    capi.check(capi.lib.dgs_gather_rows_dyn(view, dim, tail.data_ptr(), 4, n_max, n_dev.data_ptr(), 50, out.data_ptr(),
+                                            capi.TIER_ANY, bad.data_ptr(), capi.stream_ptr()))
+    assert bad.item() == 1 and (out[17] == 0).all().item()
+    assert torch.equal(out[18:100].cpu(), full[idx[18:100].cpu().long()])
     st.close()
 
 
