@@ -179,8 +179,12 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0, probs=None
             "ms_gather": 1e3 * t_gather / done}
 
 
-def device_powerlaw_csc(n, e, max_deg, one_frac, id_dtype, gen, sort_by_degree):
-    """Power-law CSC built on the device (the large workloads never exist on the host)."""
+def device_powerlaw_csc(n, e, max_deg, one_frac, id_dtype, gen, sort_by_degree, sources="uniform"):
+    """Power-law CSC built on the device (the large workloads never exist on the host).
+    sources="uniform": every edge's source is a uniform node (the benchmark configurations);
+    "by_degree": a node is a source in proportion to its in-degree, as in the symmetric graphs
+    that citation and co-purchase data are (the source of an edge is the row that holds a
+    uniformly drawn edge slot)."""
     u = torch.rand(n, generator=gen, device="cuda", dtype=torch.float64)
     raw = (1.0 - u).pow(-1.0 / 1.25)
     ones = torch.rand(n, generator=gen, device="cuda") < one_frac
@@ -204,9 +208,14 @@ def device_powerlaw_csc(n, e, max_deg, one_frac, id_dtype, gen, sort_by_degree):
     torch.cumsum(deg, 0, out=indptr[1:])
     e = int(indptr[-1].item())
     indices = torch.empty(e, dtype=id_dtype, device="cuda")
-    for a in range(0, e, 1 << 28):
-        b = min(e, a + (1 << 28))
-        indices[a:b] = torch.randint(0, n, (b - a,), generator=gen, device="cuda", dtype=id_dtype)
+    step = 1 << 28 if sources == "uniform" else 1 << 26
+    for a in range(0, e, step):
+        b = min(e, a + step)
+        if sources == "uniform":
+            indices[a:b] = torch.randint(0, n, (b - a,), generator=gen, device="cuda", dtype=id_dtype)
+        else:
+            slot = torch.randint(0, e, (b - a,), generator=gen, device="cuda")
+            indices[a:b] = (torch.searchsorted(indptr, slot, right=True) - 1).to(id_dtype)
     return indptr, indices
 
 
@@ -506,6 +515,79 @@ def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8
     return out
 
 
+def measure_placement(dgs, scale=1.0, steps=4, hbm_rows=0.4, seed=20240606):
+    """What "hottest rows first" is worth on a two-tier store: the c3 shapes (111 M nodes, 1.6 G
+    edges, f32 x256 rows, 40 % of the rows in HBM, 8192 seeds, fanouts [20,15,10]) on a graph whose
+    sources follow the in-degrees, once with the nodes in the arbitrary order they were generated
+    in and once renumbered by decreasing in-degree (placement.degree_order + renumber_csc; the
+    feature rows are random either way, so the placed store is filled afresh instead of
+    permuted).  Per variant: the share of sampled edges whose source row lies in the HBM slice
+    beside placement.expected_hit_rate, the frontier's rows per tier, host-tier bytes, step time."""
+    cfg = LARGE["c3"]
+    n, e = int(cfg["nodes"] * scale), int(cfg["edges"] * scale)
+    dim, fanouts, batch = cfg["dim"], cfg["fanouts"], cfg["batch"]
+    pl = dgs.placement
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    indptr, indices = device_powerlaw_csc(n, e, 30_000, 0.05, torch.int32, gen, sort_by_degree=False,
+                                          sources="by_degree")
+    hot_rows = int(n * hbm_rows)
+    row_bytes = dim * 4
+    seeds = [torch.randint(0, n, (batch,), generator=gen, device="cuda").to(torch.int32) for _ in range(steps + 1)]
+    out = {"config": {"workload": f"c3 shapes, sources drawn in proportion to in-degree: {n} nodes / {e} edges, "
+                                  f"f32 x{dim} rows, {int(100 * hbm_rows)}% of rows in HBM, batch {batch}, fanouts {fanouts}",
+                      "scale": scale, "steps": steps}}
+
+    def variant(ip, ix, seed_batches):
+        deg = ip[1:] - ip[:-1]
+        expected = pl.expected_hit_rate(deg, hot_rows)
+        ct_ip = store_from_device(dgs, ip, 1 << 62)
+        ct_ix = store_from_device(dgs, ix, 1 << 62)
+        ct_x = dgs.ChunkTensor([n, dim], torch.float32, hot_rows * row_bytes)
+        dev, host = ct_x._CAPI_get_sub_device_tensor(), ct_x._CAPI_get_host_tensor()
+        chunk = 1 << 26
+        for a in range(0, dev.numel(), chunk):
+            dev[a: a + chunk].normal_(generator=gen)
+        stage = torch.empty(chunk, device="cuda", dtype=torch.float32)
+        for a in range(0, host.numel(), chunk):
+            m = min(chunk, host.numel() - a)
+            stage[:m].normal_(generator=gen)
+            host[a: a + m].copy_(stage[:m])
+        del stage, dev, host
+        sampler = dgs.ChunkTensorSampler(fanouts, ct_ip, ct_ix, replace=False)
+        dgs.set_rng_state(seed, 0)
+        sampler.sample_blocks_and_index(None, seed_batches[0], ct_x)
+        torch.cuda.synchronize()
+        picks = hot_picks = rows = rows_hbm = 0
+        t0 = time.perf_counter()
+        results = [sampler.sample_blocks_and_index(None, sb, ct_x) for sb in seed_batches[1:]]
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        for frontier, _, blocks, x in results:
+            for b in blocks:
+                src = b.src_ids[b.src_local.long()]
+                picks += src.numel()
+                hot_picks += int((src < hot_rows).sum().item())
+            rows += frontier.numel()
+            rows_hbm += int((frontier < hot_rows).sum().item())
+        k = len(results)
+        return {"expected_hit_rate": expected, "measured_hit_rate_of_sampled_edges": hot_picks / max(picks, 1),
+                "frontier_rows": rows / k, "frontier_rows_in_hbm": rows_hbm / k,
+                "frontier_rows_in_host_memory": (rows - rows_hbm) / k,
+                "frontier_share_in_hbm": rows_hbm / max(rows, 1),
+                "host_tier_bytes_per_batch": (rows - rows_hbm) / k * row_bytes,
+                "ms_per_step": 1e3 * elapsed / k,
+                "host_tier_GBps_if_it_bounds_the_step": (rows - rows_hbm) * row_bytes / elapsed / 1e9}
+
+    out["unplaced"] = variant(indptr, indices, seeds)
+    release_everything()
+    order = pl.degree_order(indptr)
+    new_ip, new_ix, rank = pl.renumber_csc(indptr, indices, order)
+    del indptr, indices, order
+    out["placed_by_in_degree"] = variant(new_ip, new_ix, [rank[sb.long()] for sb in seeds])
+    out["step_time_ratio_unplaced_over_placed"] = out["unplaced"]["ms_per_step"] / out["placed_by_in_degree"]["ms_per_step"]
+    return out
+
+
 def release_everything():
     """Between workloads: pipelines (and their samplers' worker threads), cached blocks."""
     import gc
@@ -520,7 +602,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + sorted(LARGE))
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + sorted(LARGE) + ["c3_placement"])
     ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
     ap.add_argument("--inflight", type=int, default=None,
                     help="batches in flight on as many streams (1 = one blocking call per batch); default 4 for "
@@ -550,11 +632,14 @@ def main():
     dgs = importlib.import_module("dist-gpu-sampling_amd")
     torch.cuda.set_device(0)
     if args.inflight is None:
-        args.inflight = 3 if args.workload in LARGE else 4
+        args.inflight = 4 if args.workload in WORKLOADS else 3
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
     if args.node_table_max_nodes is not None:
         torch.ops.dgs_ops._CAPI_set_node_table_max_nodes(args.node_table_max_nodes)
+    if args.workload == "c3_placement":
+        print(json.dumps(measure_placement(dgs, args.scale, min(args.steps, 8))), flush=True)
+        return
     if args.workload in LARGE:
         print(json.dumps(measure_large(args.workload, dgs, args.steps, args.warmup, args.inflight, args.scale)),
               flush=True)
@@ -850,6 +935,11 @@ def main():
         guarded("c1w", c1w_leg)
         for name in ("c2", "c4", "c3"):
             guarded(name, lambda name=name: measure_large(name, dgs, k_other, w_other, 3))
+        # what the hottest-rows-first placement buys where a node's popularity follows its degree
+        # (the benchmark's own c3 draws sources uniformly: there the hot prefix catches its row share)
+        guarded("c3_placement", lambda: measure_placement(dgs))
+        if "error" not in others.get("c3", {"error": 1}) and "error" not in others["c3_placement"]:
+            others["c3"]["placement"] = others.pop("c3_placement")
         out["other_workloads"] = others
         out["other_workloads_wall_s"] = time.perf_counter() - t_others
     print(json.dumps(out), flush=True)

@@ -94,6 +94,68 @@ def test_placed_batch_is_the_same_batch(pkg):
     assert pl.expected_hit_rate(deg_new, hot_rows) > 0.5
 
 
+def test_hot_prefix_catches_the_share_of_picks_it_is_expected_to(pkg):
+    # A graph whose sources follow the in-degrees (a node is picked as a neighbour in proportion to
+    # its degree, as in symmetric power-law graphs).  With the nodes in arbitrary order the first
+    # 40 % of the rows catch 40 % of the sampled edges; renumbered by decreasing in-degree they catch
+    # what placement.expected_hit_rate says (the share of all degree that the prefix holds), which is
+    # far more.  Measured on the sampled edges of real batches, within 2 % either way.  The placed
+    # batch is gathered from a two-tier store whose rows were moved with placement.permute_rows and
+    # must hold the original rows of the nodes it names.
+    rng = np.random.default_rng(31)
+    n = 200_000
+    deg = np.minimum(np.floor(rng.pareto(1.25, size=n) * 5 + 1), 5000).astype(np.int64)
+    indptr = np.zeros(n + 1, dtype=np.int64)
+    indptr[1:] = np.cumsum(deg)
+    e = int(indptr[-1])
+    slot = rng.integers(0, e, size=e)
+    indices = (np.searchsorted(indptr, slot, side="right") - 1).astype(np.int32)  # source = row of a uniform edge slot
+    feats = torch.from_numpy(rng.standard_normal((n, 16)).astype(np.float32))
+    pl = pkg.placement
+    hot_rows = int(0.4 * n)
+    fanouts = [10, 10, 5]
+    seed_batches = [rng.integers(0, n, size=2048).astype(np.int32) for _ in range(4)]
+    big = 1 << 40
+
+    def run(ip, ix, x, batches):
+        ct_ip = pkg.create_chunktensor(ip.cpu(), 1, big)
+        ct_ix = pkg.create_chunktensor(ix.cpu(), 1, big)
+        ct_x = pkg.ChunkTensor(list(x.shape), x.dtype, pl.capacity_for_rows(x, rows=hot_rows))
+        ct_x._CAPI_load_from_tensor(x)
+        assert pl.rows_in_hbm(x, x.dtype, pl.capacity_for_rows(x, rows=hot_rows)) == hot_rows
+        sampler = pkg.ChunkTensorSampler(fanouts, ct_ip, ct_ix, seed=5)
+        picks = hot = 0
+        out = []
+        for b, sb in enumerate(batches):
+            frontier, _, blocks, rows = sampler.submit(None, torch.from_numpy(sb), ct_x, batch=b).result()
+            for blk in blocks:
+                src = blk.src_ids[blk.src_local.long()]
+                picks += src.numel()
+                hot += int((src < hot_rows).sum().item())
+            out.append((frontier, rows))
+        return hot / picks, picks, out
+
+    d_ip, d_ix = _dev(indptr), _dev(indices)
+    rate0, picks0, out0 = run(d_ip, d_ix, feats, seed_batches)
+    want0 = pl.expected_hit_rate(d_ip[1:] - d_ip[:-1], hot_rows)
+    assert picks0 > 500_000 and abs(want0 - 0.4) < 0.02 and abs(rate0 - want0) < 0.02, (rate0, want0)
+    order = pl.degree_order(d_ip)
+    new_ip, new_ix, rank = pl.renumber_csc(d_ip, d_ix, order)
+    new_feats = pl.permute_rows(feats, order.cpu())
+    rank_np = _np(rank)
+    rate1, picks1, out1 = run(new_ip, new_ix, new_feats, [rank_np[sb] for sb in seed_batches])
+    want1 = pl.expected_hit_rate(new_ip[1:] - new_ip[:-1], hot_rows)
+    assert want1 > 0.75 and abs(rate1 - want1) < 0.02, (rate1, want1)
+    assert rate1 > 1.8 * rate0
+    # the placed batches name the same kind of rows: what was gathered for new id r is the original row order[r]
+    order_cpu = order.cpu()
+    for frontier, rows in out1:
+        assert torch.equal(rows.cpu(), feats[order_cpu[frontier.cpu().long()]])
+        assert int((frontier < hot_rows).sum().item()) > 0.6 * frontier.numel()  # most of the frontier sits in HBM
+    for frontier, rows in out0:
+        assert torch.equal(rows.cpu(), feats[frontier.cpu().long()])
+
+
 def test_loading_factor_runs(pkg):
     n, d = 2_000_000, 32
     lines = []
