@@ -364,6 +364,71 @@ def test_sample_chi_square_uniform(pkg):
     assert ((counts - exp) ** 2 / exp).sum() < 72.05
 
 
+def _inclusion_statistic(picks, deg, k, rows):
+    """Chi-square statistic of the per-position inclusion counts of `rows` uniform k-subsets of
+    [0, deg) (cells are negatively correlated Bernoulli sums: scaled to deg - 1 dof)."""
+    counts = np.bincount(picks.ravel(), minlength=deg).astype(float)
+    p = k / deg
+    exp = rows * p
+    return ((counts - exp) ** 2).sum() / (exp * (1 - p)) * (deg - 1) / deg
+
+
+@pytest.mark.parametrize("deg,k,rows", [(400, 100, 3000), (6000, 3000, 60), (17000, 15, 20000)])
+def test_wave_and_global_fills_pick_uniform_subsets(pkg, deg, k, rows):
+    # the fills for fanouts above 64 (a wave per row, Floyd's set in LDS) and above 2048 (the set in
+    # the row's own output slots), and the group fill on a row of the benchmark graph's longest degree:
+    # distinct positions, every position included at rate k / deg
+    capi = pkg.capi
+    indptr = torch.arange(0, (rows + 1) * deg, deg, dtype=torch.int64, device="cuda")
+    indices = torch.arange(deg, dtype=torch.int64, device="cuda").repeat(rows)
+    seeds = torch.arange(rows, dtype=torch.int64, device="cuda")
+    r, c, flags = capi.sample_neighbors(seeds, capi.tensor_view(indptr), capi.tensor_view(indices), k, False, 4711, 6)
+    assert flags == 0 and c.numel() == rows * k
+    picks = _np(c).reshape(rows, k)
+    srt = np.sort(picks, axis=1)
+    assert (srt[:, 1:] != srt[:, :-1]).all() and picks.min() >= 0 and picks.max() < deg
+    stat = _inclusion_statistic(picks, deg, k, rows)
+    assert abs(stat - (deg - 1)) < 5 * np.sqrt(2 * (deg - 1)), stat
+    # with replacement through the same fills: independent uniform draws
+    r, c, flags = capi.sample_neighbors(seeds, capi.tensor_view(indptr), capi.tensor_view(indices), k, True, 4711, 7)
+    counts = np.bincount(_np(c), minlength=deg).astype(float)
+    exp = rows * k / deg
+    stat = ((counts - exp) ** 2 / exp).sum()
+    assert abs(stat - (deg - 1)) < 5 * np.sqrt(2 * (deg - 1)), stat
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_fused_path_picks_uniform_subsets(pkg, last_hop, replace):
+    # the fused sampler (both ways its last hop can take) on 6000 rows of degree 40 with fanout 10,
+    # then one of degree 17 000 with fanout 15: what comes out as picked ids (neighbour id = position)
+    # is a uniform subset, or with replacement independent draws whose repeats were folded inside
+    # the wave without changing a single pick
+    for deg, k, rows in ((40, 10, 6000), (17000, 15, 3000)):
+        n_nodes = max(rows, deg)
+        ptr = np.zeros(n_nodes + 1, dtype=np.int64)
+        ptr[1: rows + 1] = np.arange(1, rows + 1) * deg
+        ptr[rows + 1:] = rows * deg
+        indices = np.tile(np.arange(deg, dtype=np.int64), rows)
+        ip_ct = pkg.create_chunktensor(torch.from_numpy(ptr), 1, 1 << 40)
+        ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+        sampler = pkg.ChunkTensorSampler([k], ip_ct, ix_ct, replace=replace, seed=99)
+        frontier, _, blocks = sampler.sample_blocks(None, torch.arange(rows, dtype=torch.int64), batch=3)
+        blk = blocks[0]
+        picked = _np(blk.src_ids[blk.src_local])
+        owner = _np(blk.dst_ids[blk.dst_local])
+        assert picked.size == rows * k and np.array_equal(owner, np.repeat(np.arange(rows), k))
+        picks = picked.reshape(rows, k)
+        if replace:
+            counts = np.bincount(picked, minlength=deg).astype(float)
+            exp = rows * k / deg
+            stat = ((counts - exp) ** 2 / exp).sum()
+        else:
+            srt = np.sort(picks, axis=1)
+            assert (srt[:, 1:] != srt[:, :-1]).all()
+            stat = _inclusion_statistic(picks, deg, k, rows)
+        assert abs(stat - (deg - 1)) < 5 * np.sqrt(2 * (deg - 1)), (deg, k, replace, stat)
+
+
 @pytest.mark.parametrize("dtype", [np.int64, np.int32])
 @pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (5000, 10 ** 6), (100000, 3000), (300000, 10 ** 9)])
 def test_unique_relabel_parity(pkg, oracle, dtype, n, hi):

@@ -165,6 +165,159 @@ def test_floyd_every_subset_equally_often(oracle):
     assert chi2 < 43.82  # chi-square 19 dof, p = 0.001
 
 
+def _subset_picks(oracle, deg, k, trials, replace=False):
+    """[trials, k] picked positions of independent rows of degree `deg` (neighbour id = position).
+    Small cases are one call over `trials` rows (draws are keyed by the row id); rows too long for
+    that many copies are drawn one call at a time from a single row under `trials` different seeds."""
+    if deg * trials <= 30_000_000:
+        indptr = np.arange(0, (trials + 1) * deg, deg, dtype=np.int64)
+        indices = np.tile(np.arange(deg, dtype=np.int32), trials)
+        _, cols = oracle.sample_neighbors(np.arange(trials, dtype=np.int32), indptr, indices, k, replace, 777, 2)
+        return cols.reshape(trials, k).astype(np.int64)
+    indptr = np.array([0, deg], dtype=np.int64)
+    indices = np.arange(deg, dtype=np.int32)
+    row = np.zeros(1, dtype=np.int32)
+    out = np.empty((trials, k), dtype=np.int64)
+    for t in range(trials):
+        _, cols = oracle.sample_neighbors(row, indptr, indices, k, replace, 1000 + t, 2)
+        out[t] = cols
+    return out
+
+
+@pytest.mark.parametrize("deg,k,trials", [(1000, 15, 20000), (17000, 15, 15000), (30000, 20, 12000), (5000, 3000, 600)])
+def test_floyd_is_a_uniform_subset_on_long_rows(oracle, deg, k, trials):
+    # The degrees of the benchmark graphs' tails (17 k, 30 k), where the bounded draw works on
+    # large ranges, and a fanout in the thousands.  A uniform k-subset includes every position with
+    # probability p = k / deg and every pair with k (k - 1) / (deg (deg - 1)).  A wrong range of a
+    # step's draw, a wrong replacement position, or a biased reduction shows in one of:
+    picks = _subset_picks(oracle, deg, k, trials)
+    assert picks.min() >= 0 and picks.max() < deg
+    srt = np.sort(picks, axis=1)
+    assert (srt[:, 1:] != srt[:, :-1]).all()  # distinct positions in every row
+    p = k / deg
+    # (1) inclusion counts per position: trials Bernoulli(p) each, negatively correlated across
+    # positions; sum (c - E)^2 / (E (1 - p)) * (deg - 1) / deg is chi-square with deg - 1 dof
+    counts = np.bincount(picks.ravel(), minlength=deg).astype(float)
+    exp = trials * p
+    stat = ((counts - exp) ** 2).sum() / (exp * (1 - p)) * (deg - 1) / deg
+    dof = deg - 1
+    assert abs(stat - dof) < 5 * math.sqrt(2 * dof), (stat, dof)
+    # (2) Floyd treats the last k positions differently (they are what a repeated draw is replaced
+    # by) and the first deg - k are only ever drawn: both blocks must be included at the common rate
+    for lo, hi in ((deg - k, deg), (0, k), (deg - 2 * k, deg - k) if deg >= 3 * k else (0, deg - k)):
+        got = counts[lo:hi].sum()
+        want = trials * p * (hi - lo)
+        sd = math.sqrt(want * (1 - p))  # an upper bound: the counts are negatively correlated
+        assert abs(got - want) < 5 * sd, (lo, hi, got, want)
+    # (3) pairs: neighbouring positions, mirrored positions, and (first, last) k positions
+    member = np.zeros((trials, deg), dtype=bool) if deg * trials <= 40_000_000 else None
+    p2 = k * (k - 1) / (deg * (deg - 1))
+    if member is not None:
+        member[np.arange(trials)[:, None], picks] = True
+        both_adjacent = (member[:, 1:] & member[:, :-1]).sum()
+        both_mirrored = (member[:, : deg // 2] & member[:, ::-1][:, : deg // 2]).sum()
+        for got, pairs in ((both_adjacent, deg - 1), (both_mirrored, deg // 2)):
+            want = trials * pairs * p2
+            assert abs(got - want) < 5 * math.sqrt(want) + 1, (got, want)
+    else:
+        # without the membership matrix: count adjacent pairs from the sorted picks
+        both_adjacent = (srt[:, 1:] - srt[:, :-1] == 1).sum()
+        want = trials * (deg - 1) * p2
+        assert abs(both_adjacent - want) < 5 * math.sqrt(want) + 1, (both_adjacent, want)
+    # (4) the order of the output slots: slot j holds a draw from [0, deg - k + j] (or that top
+    # position itself), so it never exceeds deg - k + j, and it is that top position exactly when the
+    # draw repeated an earlier slot or hit the top by itself: probability (j + 1) / (deg - k + j + 1)
+    tops = deg - k + np.arange(k)
+    assert (picks <= tops[None, :]).all()
+    at_top = (picks == tops[None, :]).sum(axis=0).astype(float)
+    want_top = trials * (np.arange(k) + 1) / (tops + 1)
+    z = (at_top.sum() - want_top.sum()) / math.sqrt(want_top.sum())
+    assert abs(z) < 5, (at_top.sum(), want_top.sum())
+
+
+def test_replace_draws_are_uniform_on_a_long_row(oracle):
+    # with replacement on a row of degree 30 000: 3 M independent draws, 100 expected per position
+    deg, k = 30000, 3_000_000
+    picks = _subset_picks(oracle, deg, k, 1, replace=True).ravel()
+    counts = np.bincount(picks, minlength=deg).astype(float)
+    exp = k / deg
+    stat = ((counts - exp) ** 2 / exp).sum()
+    assert abs(stat - (deg - 1)) < 5 * math.sqrt(2 * (deg - 1)), stat
+    # consecutive draws are independent: how often draw j + 1 lands in the same hundredth of the row as draw j
+    same = (picks[1:] // 300 == picks[:-1] // 300).sum()
+    assert abs(same - (k - 1) / 100) < 5 * math.sqrt((k - 1) / 100)
+
+
+@pytest.mark.parametrize("n", [65537, 65535, 2 ** 16 + 2 ** 15 + 1, 2 ** 31 - 1, 2 ** 31 + 12345, 3 * 2 ** 30, 2 ** 32 - 5])
+def test_bounded_accepts_the_same_number_of_words_for_every_value(oracle, n):
+    # Lemire's reduction maps word w to v = floor(w n / 2^32) and must accept, for EVERY v, exactly
+    # floor(2^32 / n) of the words that map to it (that is what makes it unbiased); the words that
+    # map to v are the integers of [v 2^32 / n, (v + 1) 2^32 / n).  Counted by brute force over all
+    # of them, for values at both ends and in the middle of the range, with n on either side of
+    # 2^16 and 2^31, where the rejection zone 2^32 mod n is small, large, or nearly all of n.
+    import ctypes
+    lib = oracle.lib()
+    per_value = 2 ** 32 // n
+    words = np.zeros(4, dtype=np.uint32)
+    ptr = ctypes.c_void_p(words.ctypes.data)
+    # a word that is accepted whatever happens and maps to a value no tested word maps to
+    marker_value = n // 3 + 7
+    marker = next(w for w in range(-(-(marker_value << 32) // n), -(-((marker_value + 1) << 32) // n))
+                  if (w * n) % 2 ** 32 >= 2 ** 32 % n)
+    values = [0, 1, 2, n // 2, n - 2, n - 1] + [int(x) for x in np.random.default_rng(n % 1000).integers(0, n, size=6)]
+    zone = 2 ** 32 % n
+    for v in values:
+        if v == marker_value:
+            continue
+        lo = -(-(v << 32) // n)          # ceil(v 2^32 / n)
+        hi = -(-((v + 1) << 32) // n)    # ceil((v + 1) 2^32 / n)
+        assert hi - lo in (per_value, per_value + 1)
+        accepted = 0
+        for w in range(lo, hi):
+            words[:] = (w, marker, marker, marker)
+            got = lib.oracle_bounded(ptr, ctypes.c_uint32(n))
+            assert got in (v, marker_value)
+            accepted += got == v
+        assert accepted == per_value, (n, v, accepted, per_value)
+        # (the rejected word, when there is one, is the one whose product falls in the zone)
+        assert (hi - lo == per_value + 1) == any((w * n) % 2 ** 32 < zone for w in range(lo, hi))
+
+
+@pytest.mark.parametrize("n", [65537, 2 ** 31 + 12345, 3 * 2 ** 30])
+def test_bounded_draws_follow_the_contract_near_the_powers_of_two(oracle, n):
+    # The draws themselves (Philox words, not hand-made ones), 400 k of them.  The contract accepts
+    # the fourth word of a block unconditionally, so a value v comes up with probability
+    #   (1 - q^3) / n + q^3 * (words that map to v) / 2^32,   q = (2^32 mod n) / 2^32:
+    # uniform but for q^3, which is 2e-15 at n = 65537 (and less on any real row), 1/8 just above
+    # 2^31 (where nearly every value has two words, so the skew stays invisible) and 1/64 at
+    # n = 3 * 2^30, where every third value has two words and the other two one: that residue class
+    # must come up 1/3 + (1/64)(1/2 - 1/3) of the time, no more (a dropped rejection would give
+    # 1/2) and no less (a fifth word, or none, would give 1/3).
+    import ctypes
+    lib = oracle.lib()
+    draws = np.array([lib.oracle_draw(ctypes.c_uint64(31337), ctypes.c_uint32(9), ctypes.c_int64(j >> 10),
+                                      ctypes.c_uint32(j & 1023), ctypes.c_uint32(n)) for j in range(400_000)],
+                     dtype=np.int64)
+    assert draws.min() >= 0 and draws.max() < n
+    q3 = (2 ** 32 % n / 2 ** 32) ** 3
+    cells = 64
+    edges = [c * n // cells for c in range(cells + 1)]
+    words_into = np.array([-(-(edges[c + 1] << 32) // n) - -(-(edges[c] << 32) // n) for c in range(cells)], dtype=float)
+    sizes = np.diff(np.array(edges, dtype=float))
+    exp = draws.size * ((1 - q3) * sizes / n + q3 * words_into / 2 ** 32)
+    counts = np.bincount(np.searchsorted(np.array(edges[1:]), draws, side="right"), minlength=cells).astype(float)
+    stat = ((counts - exp) ** 2 / exp).sum()
+    assert stat < cells - 1 + 5 * math.sqrt(2 * (cells - 1)), (n, stat)
+    if n == 3 * 2 ** 30:
+        counts = np.bincount(draws % 3, minlength=3).astype(float)
+        share = np.array([0.5, 0.25, 0.25])  # words per value: 2, 1, 1, repeating
+        exp = draws.size * ((1 - q3) / 3 + q3 * share)
+        stat = ((counts - exp) ** 2 / exp).sum()
+        assert stat < 2 + 5 * math.sqrt(4), (counts, exp, stat)
+        uniform = draws.size / 3
+        assert ((counts - uniform) ** 2 / uniform).sum() > 10  # the contract's skew is there, and it is this one
+
+
 def test_floyd_definition_by_hand(oracle):
     # restate Floyd from the textbook with the oracle's draw() and compare picks
     deg, k, seed, stream, row = 37, 10, 4242, 3, 0
