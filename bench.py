@@ -148,9 +148,23 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0, probs=None
         yield from batches
         while True:
             yield torch.randint(0, cfg["nodes"], (cfg["batch"],), generator=extra, dtype=torch.int64)
+    # the checker's unique/relabel is sequential (upstream's algorithm in a fixed order); the timed
+    # leg uses the all-threads variant, held against the sequential one on the first batch, once
+    # for the result and once for what it costs
+    first = batches[0].numpy()
+    t0 = time.perf_counter()
+    want = oracle.sample_blocks(first, ip, ix, cfg["fanouts"], cfg["replace"], 1, 0, probs=pr)
+    t_sequential = time.perf_counter() - t0
+    got = oracle.sample_blocks(first, ip, ix, cfg["fanouts"], cfg["replace"], 1, 0, probs=pr, parallel_relabel=True)
+    same = np.array_equal(want[0], got[0]) and all(
+        all(np.array_equal(x, y) for x, y in zip(a, b)) for a, b in zip(want[2], got[2]))
+    if not same:
+        raise RuntimeError("cpu baseline: the all-threads relabel differs from the sequential one")
+    del want, got
     for b in more():
         t0 = time.perf_counter()
-        frontier, _, blocks = oracle.sample_blocks(b.numpy(), ip, ix, cfg["fanouts"], cfg["replace"], 1, 0, probs=pr)
+        frontier, _, blocks = oracle.sample_blocks(b.numpy(), ip, ix, cfg["fanouts"], cfg["replace"], 1, 0, probs=pr,
+                                                   parallel_relabel=True)
         t1 = time.perf_counter()
         x = torch.index_select(feats, 0, torch.from_numpy(frontier))
         t2 = time.perf_counter()
@@ -169,14 +183,16 @@ def cpu_baseline(cfg, indptr, indices, feats, batches, budget_s=12.0, probs=None
     return {"value": edges / total, "unit": "edges/s", "cores": threads, "kind": "port",
             "host_cpus": os.cpu_count(), "omp_threads": threads, "torch_threads": torch.get_num_threads(),
             "threads_per_leg": {"sampling": f"{threads} (OpenMP over the seed rows)",
-                                "unique/relabel": "1 (the identity-hash table with sequential inserts, as "
-                                                  "upstream's algorithm orders them)",
+                                "unique/relabel": f"{threads} (tables sharded by id, one per thread; the sequential "
+                                                  "restatement of upstream's table is the checker, and this one "
+                                                  "was held against it on the first batch)",
                                 "gather": f"{torch.get_num_threads()} (torch.index_select)"},
             "sample": f"{done} batches of {cfg['batch']} seeds, fanouts {cfg['fanouts']}, same graph/features "
                       f"({total:.1f} s of CPU work): oracle sampling+relabel, torch.index_select gather",
             "sample_edges_per_s": edges / t_sample, "gather_GBps": gather_bytes / t_gather / 1e9,
             "ms_per_batch": 1e3 * total / done, "ms_sample_relabel": 1e3 * t_sample / done,
-            "ms_gather": 1e3 * t_gather / done}
+            "ms_gather": 1e3 * t_gather / done,
+            "ms_sample_relabel_with_sequential_relabel": 1e3 * t_sequential}
 
 
 def device_powerlaw_csc(n, e, max_deg, one_frac, id_dtype, gen, sort_by_degree, sources="uniform"):

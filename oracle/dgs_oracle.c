@@ -33,6 +33,7 @@
  * Build: see oracle/Makefile (gcc -O2 -fopenmp -shared).
  */
 #include <math.h>
+#include <omp.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -525,5 +526,127 @@ ORACLE_API int64_t oracle_unique_relabel(const void* mapping, int64_t n_map,
     store_int(relabel_out, i, id_bytes, s < 0 ? -1 : slot_local[s]);
   }
   free(t.key); free(t.val); free(slot_local);
+  return tot;
+}
+
+/*
+ * The same result on all host threads, for the TIMED CPU baseline only (the checker stays the
+ * sequential restatement above, and tests/test_oracle.py holds this one against it): a fair
+ * multi-core CPU figure needs all three legs on all cores, and upstream's table, an identity
+ * hash filled by racing threads, has no sequential order a CPU port could keep to.
+ * Keys are sharded by a mixing hash; thread t owns shard t, walks the whole mapping list in
+ * order and inserts the keys of its shard into its own linear-probing table, so the first
+ * insertion of a key carries its smallest index and no two threads write one table.  First
+ * occurrences are flagged, counted per contiguous stretch of the list, and ranked in input
+ * order, which makes the output independent of the sharding: it is the first-occurrence-ordered
+ * unique list and its ranks, as above.
+ */
+static inline uint64_t mix64(uint64_t x) {
+  x ^= x >> 33; x *= 0xff51afd7ed558ccdull; x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ull; x ^= x >> 33;
+  return x;
+}
+
+typedef struct { int64_t* key; int64_t* first; int64_t* rank; uint64_t mask; } shard_t;
+
+static inline int64_t shard_find(const shard_t* sh, int64_t key, uint64_t h) {
+  uint64_t pos = (h >> 8) & sh->mask;
+  for (;;) {
+    if (sh->key[pos] == key) return (int64_t)pos;
+    if (sh->key[pos] == -1) return -1;
+    pos = (pos + 1) & sh->mask;
+  }
+}
+
+ORACLE_API int64_t oracle_unique_relabel_parallel(const void* mapping, int64_t n_map,
+                                                  const void* requiring, int64_t n_req,
+                                                  int id_bytes, void* unique_out,
+                                                  void* relabel_out) {
+  int n_threads = 1;
+#pragma omp parallel
+  {
+#pragma omp single
+    n_threads = omp_get_num_threads();
+  }
+  const int n_shards = n_threads;
+  shard_t* shards = (shard_t*)malloc(sizeof(shard_t) * (size_t)n_shards);
+  const int64_t cap = up_power(2 * (n_map / n_shards + 1) + 16);
+  for (int t = 0; t < n_shards; ++t) {
+    shards[t].key = (int64_t*)malloc(sizeof(int64_t) * (size_t)cap);
+    shards[t].first = (int64_t*)malloc(sizeof(int64_t) * (size_t)cap);
+    shards[t].rank = (int64_t*)malloc(sizeof(int64_t) * (size_t)cap);
+    shards[t].mask = (uint64_t)cap - 1;
+  }
+  unsigned char* flag = (unsigned char*)malloc((size_t)(n_map > 0 ? n_map : 1));
+  int64_t* stretch_count = (int64_t*)calloc((size_t)n_threads + 1, sizeof(int64_t));
+  int overfull = 0;
+#pragma omp parallel num_threads(n_threads)
+  {
+    const int t = omp_get_thread_num();
+    shard_t* mine = &shards[t];
+    int64_t held = 0;
+    for (int64_t i = 0; i < cap; ++i) { mine->key[i] = -1; mine->rank[i] = -1; }  /* (a lookup of -1 lands on an empty slot: rank -1) */
+    /* pass 1: this thread's keys, in list order: the first insertion is the smallest index */
+    for (int64_t i = 0; i < n_map; ++i) {
+      const int64_t key = load_int(mapping, i, id_bytes);
+      const uint64_t h = mix64((uint64_t)key);
+      if ((int)(h % (uint64_t)n_shards) != t) continue;
+      uint64_t pos = (h >> 8) & mine->mask;
+      for (;;) {
+        if (mine->key[pos] == key) break;
+        if (mine->key[pos] == -1) {
+          if (++held > cap - 1) { overfull = 1; break; }  /* cannot happen for a mixing hash; checked anyway */
+          mine->key[pos] = key; mine->first[pos] = i; mine->rank[pos] = -1;
+          break;
+        }
+        pos = (pos + 1) & mine->mask;
+      }
+      if (overfull) break;
+    }
+#pragma omp barrier
+    /* pass 2: flags and counts per contiguous stretch of the list */
+    const int64_t lo = n_map * t / n_threads, hi = n_map * (t + 1) / n_threads;
+    int64_t c = 0;
+    if (!overfull) {
+      for (int64_t i = lo; i < hi; ++i) {
+        const int64_t key = load_int(mapping, i, id_bytes);
+        const uint64_t h = mix64((uint64_t)key);
+        const shard_t* sh = &shards[h % (uint64_t)n_shards];
+        const int64_t s = shard_find(sh, key, h);
+        flag[i] = (unsigned char)(s >= 0 && sh->first[s] == i);
+        c += flag[i];
+      }
+    }
+    stretch_count[t + 1] = c;
+#pragma omp barrier
+#pragma omp single
+    for (int q = 0; q < n_threads; ++q) stretch_count[q + 1] += stretch_count[q];
+    /* pass 3: ranks in input order; every key is ranked by the one thread that holds its first index */
+    int64_t r = stretch_count[t];
+    if (!overfull) {
+      for (int64_t i = lo; i < hi; ++i) {
+        if (!flag[i]) continue;
+        const int64_t key = load_int(mapping, i, id_bytes);
+        const uint64_t h = mix64((uint64_t)key);
+        shard_t* sh = &shards[h % (uint64_t)n_shards];
+        sh->rank[shard_find(sh, key, h)] = r;
+        store_int(unique_out, r, id_bytes, key);
+        ++r;
+      }
+    }
+#pragma omp barrier
+    if (!overfull) {
+#pragma omp for schedule(static)
+      for (int64_t i = 0; i < n_req; ++i) {
+        const int64_t key = load_int(requiring, i, id_bytes);
+        const uint64_t h = mix64((uint64_t)key);
+        const shard_t* sh = &shards[h % (uint64_t)n_shards];
+        const int64_t s = shard_find(sh, key, h);
+        store_int(relabel_out, i, id_bytes, s < 0 ? -1 : sh->rank[s]);
+      }
+    }
+  }
+  const int64_t tot = overfull ? -1 : stretch_count[n_threads];
+  for (int t = 0; t < n_shards; ++t) { free(shards[t].key); free(shards[t].first); free(shards[t].rank); }
+  free(shards); free(flag); free(stretch_count);
   return tot;
 }

@@ -36,6 +36,7 @@ def lib():
         _lib.oracle_draw.restype = ctypes.c_uint32
         _lib.oracle_sample_counts.restype = ctypes.c_int64
         _lib.oracle_unique_relabel.restype = ctypes.c_int64
+        _lib.oracle_unique_relabel_parallel.restype = ctypes.c_int64
         _lib.oracle_neg_log_u32.restype = ctypes.c_double
         _lib.oracle_weighted_key.restype = ctypes.c_double
         _lib.oracle_weight_quantum.restype = ctypes.c_uint64
@@ -219,8 +220,9 @@ def sample_counts(seeds, indptr, num_picks, replace):
 
 
 # -------------------------------------------------------- unique/relabel ----
-def unique_relabel(mapping, requiring):
-    """_CAPI_tensor_relabel(mapping_tensors, requiring_relabel_tensors)."""
+def unique_relabel(mapping, requiring, parallel=False):
+    """_CAPI_tensor_relabel(mapping_tensors, requiring_relabel_tensors).  `parallel`: the same
+    result computed on all host threads (sharded tables), for the timed CPU baseline."""
     mapping = [_ids(m) for m in mapping]
     requiring = [_ids(r) for r in requiring]
     dt = mapping[0].dtype if mapping else requiring[0].dtype
@@ -229,15 +231,16 @@ def unique_relabel(mapping, requiring):
     assert m.dtype == dt and r.dtype == dt
     uniq = np.empty(m.size, dtype=dt)
     rel = np.empty(r.size, dtype=dt)
-    tot = lib().oracle_unique_relabel(_p(m), _i64(m.size), _p(r), _i64(r.size),
-                                      ctypes.c_int(dt.itemsize), _p(uniq), _p(rel))
+    fn = lib().oracle_unique_relabel_parallel if parallel else lib().oracle_unique_relabel
+    tot = fn(_p(m), _i64(m.size), _p(r), _i64(r.size), ctypes.c_int(dt.itemsize), _p(uniq), _p(rel))
+    assert tot >= 0
     sizes = np.cumsum([x.size for x in requiring])[:-1]
     return uniq[:tot].copy(), [x.copy() for x in np.split(rel, sizes)]
 
 
 # --------------------------------------------------- multi-layer driver -----
 def sample_blocks(seed_nodes, indptr, indices, fanouts, replace=False, rng_seed=0,
-                  first_stream=0, probs=None):
+                  first_stream=0, probs=None, parallel_relabel=False):
     """ChunkTensorSampler.sample_blocks
     (oppo_bench/single_node/utils/chunktensor_sampler.py:93-118) with the DGL
     block replaced by the tuple (src_local, dst_local, n_src, n_dst, src_ids,
@@ -254,7 +257,7 @@ def sample_blocks(seed_nodes, indptr, indices, fanouts, replace=False, rng_seed=
         else:
             coo_row, coo_col = sample_neighbors(seeds, indptr, indices, fan_out, replace, rng_seed,
                                                 first_stream + hop)
-        frontier, (row_l, col_l) = unique_relabel([seeds, coo_col], [coo_row, coo_col])
+        frontier, (row_l, col_l) = unique_relabel([seeds, coo_col], [coo_row, coo_col], parallel=parallel_relabel)
         blocks.insert(0, (col_l, row_l, frontier.size, seeds.size, frontier, seeds))
         seeds = frontier
     return frontier, _ids(seed_nodes), blocks

@@ -377,6 +377,30 @@ def test_unique_relabel_vs_numpy(oracle, dtype):
         assert uniq.dtype == dtype and rl.dtype == dtype
 
 
+@pytest.mark.parametrize("dtype", [np.int64, np.int32])
+def test_parallel_unique_relabel_is_the_sequential_one(oracle, dtype):
+    # the all-threads variant that the benchmark's CPU baseline times gives the sequential
+    # restatement's results, bit for bit: sizes around the shard and thread counts, many repeats, few
+    # repeats, absent and negative ids to look up, nothing at all
+    rng = np.random.default_rng(17)
+    for n, hi in [(0, 10), (1, 10), (7, 3), (100, 1000), (5000, 300), (200000, 50000), (200000, 2 ** 30), (1 << 20, 1 << 21)]:
+        mapping = [rng.integers(0, hi, size=n // 3).astype(dtype), rng.integers(0, hi, size=n - n // 3).astype(dtype)]
+        requiring = [rng.integers(-3, hi + 5, size=n // 2 + 3).astype(dtype), mapping[1]]
+        want_u, want_r = oracle.unique_relabel(mapping, requiring)
+        got_u, got_r = oracle.unique_relabel(mapping, requiring, parallel=True)
+        assert np.array_equal(got_u, want_u)
+        for a, b in zip(got_r, want_r):
+            assert np.array_equal(a, b)
+    # and through the multi-layer driver
+    indptr, indices = _toy_graph(rng, 3000, 40)
+    seeds = rng.integers(0, 3000, size=500).astype(np.int64)
+    a = oracle.sample_blocks(seeds, indptr, indices, [5, 4, 3], False, 3, 1)
+    b = oracle.sample_blocks(seeds, indptr, indices, [5, 4, 3], False, 3, 1, parallel_relabel=True)
+    assert np.array_equal(a[0], b[0])
+    for x, y in zip(a[2], b[2]):
+        assert all(np.array_equal(p, q) for p, q in zip(x, y))
+
+
 def test_relabel_absent_key(oracle):
     uniq, (r,) = oracle.unique_relabel([np.array([5, 3, 5], dtype=np.int64)],
                                        [np.array([3, 9, 5], dtype=np.int64)])
