@@ -93,6 +93,8 @@ SIGNATURES = {
     "dgs_ticket_stream_wait": (ctypes.c_int, [c_vp, c_vp]),
     "dgs_ticket_wait": (ctypes.c_int, [c_vp]),
     "dgs_ticket_wait_words": (ctypes.c_int, [c_vp, c_vp, c_i32]),
+    "dgs_ticket_sync": (ctypes.c_int, [c_vp]),
+    "dgs_ticket_sync_words": (ctypes.c_int, [c_vp, c_vp, c_i32]),
     "dgs_stream_wait_words": (ctypes.c_int, [c_vp, c_vp, c_i32]),
     "dgs_ticket_release": (ctypes.c_int, [c_vp]),
     "dgs_stream_query": (ctypes.c_int, [c_vp, ctypes.POINTER(c_i32)]),

@@ -34,6 +34,7 @@
 #include <string>
 #include <thread>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -48,6 +49,26 @@ void check(dgs_status s) {
 }
 
 void* current_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+// A ticket (an event recorded on a stream) that several parties look at: the host thread that
+// waits for a batch's lengths, the next batch's gather waiting its turn, the owner of a node table.
+// Every event between two kernels costs the GPU about 6 us of idling, so a batch records ONE, behind
+// its last launch, and shares it; it goes back to the library's pool when the last holder lets go.
+struct SharedTicket {
+  void* handle = nullptr;
+  SharedTicket() = default;
+  SharedTicket(const SharedTicket&) = delete;
+  SharedTicket& operator=(const SharedTicket&) = delete;
+  ~SharedTicket() {
+    if (handle != nullptr) dgs_ticket_release(handle);
+  }
+};
+using TicketRef = std::shared_ptr<SharedTicket>;
+TicketRef record_ticket(void* stream) {
+  auto t = std::make_shared<SharedTicket>();
+  check(dgs_ticket_record(stream, &t->handle));
+  return t;
+}
 
 #define DGS_CHECK_GPU(x) TORCH_CHECK((x).device().is_cuda(), #x " must be a GPU tensor")
 
@@ -135,11 +156,7 @@ class ChunkTensor : public torch::CustomClassHolder {
     // without a copy, the kernels write it through its device mapping)
     bad_index_ = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
   }
-  ~ChunkTensor() override {
-    for (auto& entry : node_tables_)
-      if (entry.second.done != nullptr) dgs_ticket_release(entry.second.done);
-    dgs_store_destroy(store_);
-  }
+  ~ChunkTensor() override { dgs_store_destroy(store_); }
 
   // Raises if a gather that has run since the last check met an index outside the rows it may
   // read (those output rows were zero-filled).  Gathers are asynchronous, so the error surfaces
@@ -259,12 +276,11 @@ class ChunkTensor : public torch::CustomClassHolder {
         auto pick = node_tables_.end();
         for (auto jt = node_tables_.begin(); jt != node_tables_.end(); ++jt) {
           int32_t finished = 1;  // a table that was handed out and never used has nothing pending
-          if (jt->second.done != nullptr) check(dgs_ticket_query(jt->second.done, &finished));
+          if (jt->second.done) check(dgs_ticket_query(jt->second.done->handle, &finished));
           if (finished && (pick == node_tables_.end() || jt->second.last_use < pick->second.last_use)) pick = jt;
         }
         if (pick == node_tables_.end()) return {nullptr, 0u};
         NodeTable taken = std::move(pick->second);
-        pick->second.done = nullptr;
         node_tables_.erase(pick);
         // the memory came from another stream's pool: it must not be handed out again while
         // this stream still uses it
@@ -285,14 +301,12 @@ class ChunkTensor : public torch::CustomClassHolder {
     t.last_use = ++uses_;
     return {t.entries.data_ptr(), ++t.epoch};
   }
-  // Marks the end of a call that used `stream`'s table: everything enqueued on the stream so far.
+  // Says when the call that just used `stream`'s table will have finished with it: at `done`, a
+  // ticket recorded on the stream behind the call's last launch that reads the table (or later).
   // (Called with enqueue_lock() held.)
-  void node_table_used(void* stream) {
+  void node_table_used(void* stream, TicketRef done) {
     auto it = node_tables_.find(stream);
-    if (it == node_tables_.end()) return;
-    if (it->second.done != nullptr) dgs_ticket_release(it->second.done);
-    it->second.done = nullptr;
-    check(dgs_ticket_record(stream, &it->second.done));
+    if (it != node_tables_.end()) it->second.done = std::move(done);
   }
   // Gives up the node table of a stream (0: the current stream), e.g. before the stream is
   // destroyed; returns whether there was one.  Kernels of earlier calls that still use the table
@@ -302,7 +316,6 @@ class ChunkTensor : public torch::CustomClassHolder {
     void* key = stream_handle != 0 ? reinterpret_cast<void*>(static_cast<intptr_t>(stream_handle)) : current_stream();
     auto it = node_tables_.find(key);
     if (it == node_tables_.end()) return false;
-    if (it->second.done != nullptr) dgs_ticket_release(it->second.done);
     node_tables_.erase(it);
     return true;
   }
@@ -336,7 +349,7 @@ class ChunkTensor : public torch::CustomClassHolder {
     torch::Tensor entries;
     uint32_t epoch = 0;
     uint64_t last_use = 0;
-    void* done = nullptr;  // ticket behind the last call that used the table (null: never used)
+    TicketRef done;  // ticket behind the last call that used the table (none: never used)
   };
   uint64_t uses_ = 0;
   std::atomic<int64_t> frontier_hint_{0};
@@ -608,18 +621,17 @@ class PendingBlocks : public torch::CustomClassHolder {
  public:
   PendingBlocks() = default;
   ~PendingBlocks() override {
-    if (ticket_ != nullptr) dgs_ticket_wait(ticket_);  // never leave a ticket behind
+    // a batch nobody finished: its kernels still write the pinned words, which must outlive them
+    if (!finished_ && end_) dgs_ticket_sync(end_->handle);
   }
 
   BlocksResult Finish() {
     TORCH_CHECK(!finished_, "PendingBlocks: already finished");
     finished_ = true;
+    // the lengths are mirrored into the pinned words when the last hop's compaction has run, well
+    // before the batch's end: the words are polled, and the batch's ticket only bounds the wait
     dgs_status ws_status = DGS_OK;
-    if (ticket_ != nullptr) {
-      void* t = ticket_;
-      ticket_ = nullptr;
-      ws_status = dgs_ticket_wait_words(t, pinned_.data_ptr<int64_t>(), 3 * hops_ + 1);
-    }
+    if (end_) ws_status = dgs_ticket_sync_words(end_->handle, pinned_.data_ptr<int64_t>(), 3 * hops_ + 1);
     check(gather_status_);
     check(ws_status);
     const int64_t* sizes_host = pinned_.data_ptr<int64_t>();
@@ -646,6 +658,7 @@ class PendingBlocks : public torch::CustomClassHolder {
         x_ = torch::empty({rows, features_->elem_stride()}, x_.options());
         check(dgs_gather_rows(features_->view(), features_->elem_stride(), all_.data_ptr(), width_, rows,
                               x_.data_ptr(), DGS_TIER_ANY, features_->bad_index_word(), current_stream()));
+        gathered_late_ = true;
       }
     }
     return std::make_tuple(frontier, src_, dst_, features_ ? x_ : torch::empty({0}, seeds_.options()), seeds_);
@@ -759,13 +772,12 @@ class PendingBlocks : public torch::CustomClassHolder {
       check(dgs_sample_blocks_weighted(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), probs->view(),
                                        fanouts.data(), hops, replace, rng.first, rng.second, table.first,
                                        table.second, p->all_.data_ptr(), outs.data(), sizes_dev.data_ptr<int64_t>(),
-                                       p->pinned_.data_ptr<int64_t>(), &p->ticket_, ws.data_ptr(), ws_bytes, st));
+                                       p->pinned_.data_ptr<int64_t>(), nullptr, ws.data_ptr(), ws_bytes, st));
     else
       check(dgs_sample_blocks(p->seeds_.data_ptr(), w, n, indptr->view(), indices->view(), fanouts.data(), hops,
                               replace, rng.first, rng.second, table.first, table.second, p->all_.data_ptr(),
                               outs.data(), sizes_dev.data_ptr<int64_t>(), p->pinned_.data_ptr<int64_t>(),
-                              &p->ticket_, ws.data_ptr(), ws_bytes, st));
-    if (table.first != nullptr) indptr->node_table_used(st);  // the last launch above is the table's last reader
+                              nullptr, ws.data_ptr(), ws_bytes, st));
     if (features) {
       const auto xopt = torch::TensorOptions().dtype(features->dtype()).device(dev);
       const int64_t row_bytes = features->elem_stride() * static_cast<int64_t>(c10::elementSize(features->dtype()));
@@ -796,12 +808,25 @@ class PendingBlocks : public torch::CustomClassHolder {
                                                 features->bad_index_word(), st);
       }
     }
+    // the batch's one ticket, behind its last launch: it bounds the wait for the lengths, tells the
+    // next batch's gather when this one's is through, and the graph when its node table is free again
+    p->end_ = record_ticket(st);
+    if (table.first != nullptr) indptr->node_table_used(st, p->end_);
     return p;
   }
 
   // The stream the batch was begun on, and a way to mark the batch's buffers as used on another
   // stream (so that the allocator does not hand them out again while that stream still reads them).
   c10::Stream stream() const { return stream_; }
+  // The ticket behind everything the batch has enqueued: the one recorded by Begin, unless Finish
+  // had to enqueue a gather of its own afterwards (a fresh one then).
+  TicketRef last_ticket() {
+    if (gathered_late_) {
+      end_ = record_ticket(c10::hip::HIPStreamMasqueradingAsCUDA(stream_).stream());
+      gathered_late_ = false;
+    }
+    return end_;
+  }
   void RecordStream(const c10::Stream& consumer) {
     // (the frontier and the edge lists are, or are views of, the tensors in owned_)
     for (const torch::Tensor* t : {&seeds_, &x_})
@@ -812,7 +837,8 @@ class PendingBlocks : public torch::CustomClassHolder {
  private:
   int hops_ = 0;
   bool finished_ = false;
-  void* ticket_ = nullptr;
+  TicketRef end_;               // recorded behind the last launch of Begin
+  bool gathered_late_ = false;  // Finish enqueued a gather behind end_
   dgs_status gather_status_ = DGS_OK;
   torch::Tensor pinned_, seeds_, all_, x_;
   std::vector<torch::Tensor> owned_;  // the allocations behind all_, src_, dst_ and the device-side lengths
@@ -848,7 +874,7 @@ class BatchLoop : public torch::CustomClassHolder {
     for (size_t i = 0; i < streams.size(); i += 3)
       streams_.push_back(c10::Stream::unpack3(streams[i], static_cast<c10::DeviceIndex>(streams[i + 1]),
                                                static_cast<c10::DeviceType>(streams[i + 2])));
-    done_.assign(streams_.size() + 1, nullptr);
+    done_.assign(streams_.size() + 1, TicketRef());
     worker_ = std::thread([this] { Work(); });
   }
   ~BatchLoop() override { Close(); }
@@ -907,11 +933,7 @@ class BatchLoop : public torch::CustomClassHolder {
     if (hand_over_) {
       // the calling thread's stream waits for everything the batch has enqueued (Finish may just have
       // added a gather), and the batch's buffers are marked as used there
-      void* ticket = nullptr;
-      check(dgs_ticket_record(stream_handle(item.batch->stream()), &ticket));
-      const dgs_status ws = dgs_ticket_stream_wait(current_stream(), ticket);
-      dgs_ticket_release(ticket);
-      check(ws);
+      check(dgs_ticket_stream_wait(current_stream(), item.batch->last_ticket()->handle));
       item.batch->RecordStream(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().unwrap());
     }
     return result;
@@ -944,10 +966,7 @@ class BatchLoop : public torch::CustomClassHolder {
       if (item.seeds_ready) dgs_ticket_release(item.seeds_ready);
     unbegun.clear();
     unclaimed.clear();  // batches nobody asked for: their destructors wait for their kernels' lengths
-    for (void*& t : done_) {
-      if (t) dgs_ticket_release(t);
-      t = nullptr;
-    }
+    for (TicketRef& t : done_) t.reset();
   }
 
  private:
@@ -987,18 +1006,14 @@ class BatchLoop : public torch::CustomClassHolder {
           check(ws);
         }
         const bool turn = turn_ && features_ && n > 1;
-        void* gather_after = turn && index > 0 ? done_[(index - 1) % (n + 1)] : nullptr;
+        const TicketRef before = turn && index > 0 ? done_[(index - 1) % (n + 1)] : TicketRef();
+        void* gather_after = before ? before->handle : nullptr;
         std::pair<uint64_t, uint32_t> own{0, 0};
         if (!rng_.empty()) own = {static_cast<uint64_t>(rng_[0]), static_cast<uint32_t>(item.first_stream)};
         item.batch = PendingBlocks::Begin(item.seeds, indptr_, indices_, fanouts_, replace_, features_, probs_,
                                           rng_.empty() ? nullptr : &own, gather_after);
-        if (turn) {
-          // the slot's old ticket belongs to a batch that was popped long ago (at most n are in flight)
-          void*& slot = done_[index % (n + 1)];
-          if (slot) dgs_ticket_release(slot);
-          slot = nullptr;
-          check(dgs_ticket_record(raw, &slot));
-        }
+        // (the slot's old ticket belongs to a batch that was popped long ago: at most n are in flight)
+        if (turn) done_[index % (n + 1)] = item.batch->last_ticket();
       } catch (const std::exception& err) {
         item.error = err.what();
       }
@@ -1019,7 +1034,7 @@ class BatchLoop : public torch::CustomClassHolder {
   std::vector<c10::Stream> streams_;
   bool hand_over_, turn_;
   std::vector<int64_t> rng_;
-  std::vector<void*> done_;  // ring of tickets behind the last batches' last launches (worker thread only)
+  std::vector<TicketRef> done_;  // ring of the last batches' tickets (worker thread only)
   std::mutex mutex_;
   std::condition_variable wake_worker_, wake_caller_;
   std::deque<Item> input_, output_;

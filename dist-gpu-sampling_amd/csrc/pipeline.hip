@@ -1325,18 +1325,16 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
   DGS_REQUIRE(node_table == nullptr || (node_table_epoch >= 1 && node_table_epoch < 0xfffffff0u), DGS_ERR_INVALID,
               "sample_blocks: node table epoch %u outside 1..2^32-17 (refill the table with 0xFF and restart at 1)",
               node_table_epoch);
-  DGS_REQUIRE((sizes_host == nullptr) == (sizes_ticket == nullptr), DGS_ERR_INVALID,
-              "sample_blocks: sizes_host and sizes_ticket go together");
+  DGS_REQUIRE(sizes_ticket == nullptr || sizes_host != nullptr, DGS_ERR_INVALID,
+              "sample_blocks: a sizes_ticket needs sizes_host");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n_seeds == 0) {  // nothing to launch: every size is zero
     // a fill kernel, not a memset node: the call may be recorded into a graph
     hipLaunchKernelGGL(zero_sizes_kernel, dim3(1), dim3(64), 0, st, sizes_dev, 3 * n_hops + 1);
     DGS_LAUNCH_CHECK();
-    if (sizes_host) {
+    if (sizes_host)
       for (int i = 0; i < 3 * n_hops + 1; ++i) sizes_host[i] = 0;
-      return dgs_ticket_record(st, sizes_ticket);
-    }
-    return DGS_OK;
+    return sizes_ticket ? dgs_ticket_record(st, sizes_ticket) : DGS_OK;
   }
   DGS_REQUIRE(seeds != nullptr && frontier != nullptr, DGS_ERR_INVALID, "sample_blocks: null seeds or frontier");
   DGS_REQUIRE(workspace != nullptr && workspace_bytes >= need, DGS_ERR_WORKSPACE,

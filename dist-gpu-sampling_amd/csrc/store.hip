@@ -307,17 +307,31 @@ static hipError_t poll_words(const int64_t* words, int32_t n_words, StillRunning
 }
 }  // namespace dgs
 
+DGS_API dgs_status dgs_ticket_sync_words(void* ticket, const int64_t* words, int32_t n_words) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_sync_words: null ticket");
+  DGS_REQUIRE(words != nullptr && n_words >= 1, DGS_ERR_INVALID, "ticket_sync_words: no words");
+  hipEvent_t ev = static_cast<hipEvent_t>(ticket);
+  const hipError_t e = dgs::poll_words(words, n_words, [ev] { return hipEventQuery(ev); });
+  if (e != hipSuccess) {
+    dgs::set_error("ticket_sync_words: %s", hipGetErrorString(e));
+    return DGS_ERR_HIP;
+  }
+  return DGS_OK;
+}
+
 DGS_API dgs_status dgs_ticket_wait_words(void* ticket, const int64_t* words, int32_t n_words) {
   DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_wait_words: null ticket");
   DGS_REQUIRE(words != nullptr && n_words >= 1, DGS_ERR_INVALID, "ticket_wait_words: no words");
-  hipEvent_t ev = static_cast<hipEvent_t>(ticket);
-  const hipError_t e = dgs::poll_words(words, n_words, [ev] { return hipEventQuery(ev); });
-  {
-    std::lock_guard<std::mutex> lock(dgs::g_event_mutex);
-    dgs::g_event_pool.push_back(ev);
-  }
+  const dgs_status s = dgs_ticket_sync_words(ticket, words, n_words);
+  dgs_ticket_release(ticket);
+  return s;
+}
+
+DGS_API dgs_status dgs_ticket_sync(void* ticket) {
+  DGS_REQUIRE(ticket != nullptr, DGS_ERR_INVALID, "ticket_sync: null ticket");
+  const hipError_t e = hipEventSynchronize(static_cast<hipEvent_t>(ticket));
   if (e != hipSuccess) {
-    dgs::set_error("ticket_wait_words: %s", hipGetErrorString(e));
+    dgs::set_error("ticket_sync: %s", hipGetErrorString(e));
     return DGS_ERR_HIP;
   }
   return DGS_OK;

@@ -421,12 +421,16 @@ typedef struct dgs_block_out {
  *                                                          not a row of the graph, 4 a picked neighbour id
  *                                                          is not a node (each checked before it addresses
  *                                                          anything; such rows emit nothing)
- *   sizes_host / ticket    : optional (both or neither).  sizes_host is pinned host memory
- *                            that the device can write (hipHostMalloc); the kernels mirror
+ *   sizes_host / ticket    : optional (a ticket only with sizes_host).  sizes_host is pinned host
+ *                            memory that the device can write (hipHostMalloc); the kernels mirror
  *                            sizes_dev into it, and *sizes_ticket marks the point on `stream`
  *                            after which it is complete -- before the last hop's edge lists are
  *                            written, so a caller can enqueue more work (a feature gather) and
  *                            only then call dgs_ticket_wait.  Saves the device-to-host copy.
+ *                            A caller that polls the words (dgs_stream_wait_words, or
+ *                            dgs_ticket_sync_words on a ticket of its own recorded later) passes
+ *                            sizes_host alone: every ticket is an event on the stream, and an
+ *                            event between two kernels costs the GPU some 6 us of idling.
  *   node_table / epoch     : optional persistent direct-address table of
  *                            dgs_node_table_bytes(n_nodes) bytes (n_nodes = indptr entries - 1,
  *                            < 2^31), filled with 0xFF bytes before its first use and then never
@@ -542,6 +546,14 @@ dgs_status dgs_ticket_wait(void* ticket);
  * which copies its lengths back with a blocking cudaMemcpy.
  */
 dgs_status dgs_ticket_wait_words(void* ticket, const int64_t* words, int32_t n_words);
+/*
+ * dgs_ticket_wait and dgs_ticket_wait_words for a ticket that more than one party looks at (the
+ * host thread that wants a batch's lengths, a later batch whose gather waits its turn, the owner
+ * of a node table): they block in the same way but leave the ticket valid; whoever lets go of it
+ * last calls dgs_ticket_release.
+ */
+dgs_status dgs_ticket_sync(void* ticket);
+dgs_status dgs_ticket_sync_words(void* ticket, const int64_t* words, int32_t n_words);
 /*
  * The same wait without a ticket (recording one costs the caller 1-4 us per call): polls the
  * words and gives up once `stream`, the stream the call was enqueued on, has drained.  For
