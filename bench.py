@@ -629,6 +629,9 @@ def main():
     ap.add_argument("--node-table-max-nodes", type=int, default=None,
                     help="graphs above this many nodes sample on a per-call hash table instead of persistent "
                          "node tables (the library's default when not given)")
+    ap.add_argument("--last-hop", type=int, default=0,
+                    help="how the fused sampler's last hop finds first occurrences (the library's test hook "
+                         "DGS_DEBUG_SAMPLER_BUCKETED): 0 by size, 1 always on the node table, 2 always the bucketed pass")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with --workload c1: do not also run c1w, c2, c4 and c3 after the headline")
@@ -651,6 +654,8 @@ def main():
         args.inflight = 4 if args.workload in WORKLOADS else 3
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
+    if args.last_hop:
+        dgs.capi.check(dgs.capi.lib.dgs_debug_set(dgs.capi.DEBUG_SAMPLER_BUCKETED, args.last_hop))
     if args.node_table_max_nodes is not None:
         torch.ops.dgs_ops._CAPI_set_node_table_max_nodes(args.node_table_max_nodes)
     if args.workload == "c3_placement":

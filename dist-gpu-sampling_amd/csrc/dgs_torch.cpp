@@ -122,6 +122,9 @@ void check_sampling_flags(int64_t flags, const char* who, int hop) {
   TORCH_CHECK((flags & 2) == 0, where, ": a seed id is not a row of the graph (outside 0 .. nodes - 1)");
   TORCH_CHECK((flags & 4) == 0, where, ": a neighbour id stored in the graph is not a node (outside 0 .. nodes - 1)");
   TORCH_CHECK((flags & 1) == 0, where, ": a seed row has a degree of 2^32 or more, or offsets outside the edge array");
+  TORCH_CHECK((flags & 8) == 0, where, ": the ids of this hop crowd one bucket of the on-chip pass that finds first "
+              "occurrences (more distinct ids in a bucket than its table holds); sample on the node table instead "
+              "(dgs_debug_set(DGS_DEBUG_SAMPLER_BUCKETED, 1))");
   TORCH_CHECK(false, where, ": error bits ", flags);
 }
 

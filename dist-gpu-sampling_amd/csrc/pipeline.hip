@@ -123,7 +123,10 @@ struct Hop {
   int32_t k;
   int32_t index;            // hop number
   uint32_t rng_stream;
-  int32_t bucketed;         // non-zero: first occurrences come from the bucketed pass (see Buckets)
+  int32_t bucketed;         // non-zero: first occurrences come from the bucketed pass (see Buckets) ...
+  int32_t pad1_;
+  int64_t bucket_pos_cap;   // ... as long as the hop's padded positions (seeds * k) are no more than this: decided on the device
+  int* bucket_overflow;     // set by the pass when a bucket held more ids than its LDS table takes (the call fails)
 };
 
 // (written without a conditional so that the read is not moved behind a test)
@@ -131,6 +134,13 @@ __device__ __forceinline__ int64_t seeds_of(const Hop& h) {
   const int64_t on_device = *h.n_seeds;
   const int64_t use_device = h.n_seeds_host >> 63;  // all ones when the count lives on the device
   return (on_device & use_device) | (h.n_seeds_host & ~use_device);
+}
+// Whether this hop finds its first occurrences by the bucketed pass.  Its worst case may be far
+// beyond what the pass has room for (it grows with the product of the fanouts, the hop does not),
+// so the host only says whether the hop is eligible and every kernel decides from the hop's real
+// length, the same way.  (A bucketed hop is never hop 0: its positions are seeds * k.)
+__device__ __forceinline__ bool bucketed_now(const Hop& h, int64_t s) {
+  return h.bucketed != 0 && s * h.k <= h.bucket_pos_cap;
 }
 // the first seed_part positions of hop 0 are the caller's seeds themselves
 __device__ __forceinline__ int64_t seed_part(const Hop& h, int64_t s) { return h.index == 0 ? s : 0; }
@@ -166,8 +176,15 @@ constexpr int kBucketRange = 8192;                   // ids per bucket at most: 
 constexpr int kMaxBucketTiles = 2048;                // tiles a bucket's block can walk (its LDS index of them)
 constexpr int64_t kBucketedMaxNodes = int64_t(kMaxBuckets) * kBucketRange;
 constexpr int64_t kBucketedMinPicks = int64_t(1) << 18;  // worst-case picks of the hop below which the table is cheaper
-constexpr int64_t kBucketedMaxUnits = int64_t(kMaxBucketTiles - 2) * kBucketTile;  // so that the tiles fit that index; bounds the extra workspace too
 constexpr uint32_t kRankBit = 0x40000000u;
+// Graphs with more nodes than kBucketedMaxNodes: buckets by a hash of the id, and a bucket's ids
+// are told apart in an open-addressing table in LDS (ids + smallest order values, 128 KB of the
+// CU's 160 KB) instead of an array indexed by the id's high bits.  A bucket may hold up to half as
+// many units as the table has slots on average, which bounds the hop the pass accepts.
+constexpr int kHashBlock = 1024;
+constexpr int kHashSlots = 16384;
+constexpr uint32_t kHashEmpty = 0xffffffffu;         // no id: ids are below 2^31
+constexpr int kErrBucketOverflow = 8;                // hop flag bit: a bucket's ids did not fit its LDS table
 
 struct Buckets {
   uint2* items;      // [tiles_max][kBucketTile] (id, order value), every tile's units in bucket order
@@ -176,7 +193,25 @@ struct Buckets {
   int32_t front_tiles;
   int32_t log_buckets;
   uint32_t n_nodes;
+  int32_t hashed;    // buckets by a hash of the id, ids told apart in an LDS hash table (any node count)
+  int32_t hash_slots;  // slots of that table the kernels use: kHashSlots (a test hook makes it small, so that small inputs fill it)
 };
+// Buckets of the hop.  The direct form's count follows from the node count (host); the hashed
+// form's follows from the hop's real size, on the device: as few buckets as keep a bucket's units
+// within its table's slots on average (a bucket that is fuller than that goes over its units in
+// parts), because every bucket costs its block a fixed chain of waits: a hop that fits 256 buckets
+// is one block per CU, all at once.
+constexpr int kMinHashLogBuckets = 8;
+__device__ __forceinline__ int log_buckets_of(const Buckets& b, const Hop& h, int64_t s) {
+  if (!b.hashed) return b.log_buckets;
+  const int64_t units = s + s * h.k;  // at most: short rows leave padded positions empty, ids repeat
+  int lb = kMinHashLogBuckets;
+  while (lb < b.log_buckets && (int64_t(b.hash_slots) << lb) < units) ++lb;
+  return lb;
+}
+__device__ __forceinline__ uint32_t bucket_of(const Buckets& b, int log_buckets, uint32_t id) {
+  return (b.hashed ? hash_id(id) : id) & uint32_t((1 << log_buckets) - 1);
+}
 
 // rank of the id at position p, given p's slot word
 template <typename TableT>
@@ -290,6 +325,7 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
   // is a first occurrence, else the position the table holds.  Two rounds of loads, each issued
   // for all of the thread's picks before any is used, and both before the block adds up its
   // prefix (whose barrier nothing here has to wait behind).
+  const bool bucketed = bucketed_now(h, s);
   bool live[kRelabelItems];
   bool known[kRelabelItems];  // bucketed hop: the word of a repeat may be the rank itself
   uint32_t at[kRelabelItems];
@@ -299,7 +335,7 @@ __device__ __forceinline__ void relabel_tile(const Hop& h, const TableT& table, 
     at[j] = uint32_t(p[j]);
     known[j] = false;
     if (live[j] && !(word[j] & kFirstBit)) {
-      if (h.bucketed) {
+      if (bucketed) {
         known[j] = (word[j] & kRankBit) != 0;
         at[j] = word[j] & (kRankBit - 1);
       } else {
@@ -338,10 +374,10 @@ __device__ __forceinline__ void mark_lost(const Hop& h, uint32_t displaced) {
 // checked before it addresses anything.
 template <typename IdT, typename TableT>
 __device__ __forceinline__ bool place_pick(const Hop& h, const TableT& table, IdT col, int64_t p, bool look_first,
-                                           uint32_t* word) {
+                                           bool bucketed, uint32_t* word) {
   *word = kInvalidSlot;
   if (!table.holds(col)) return false;
-  if (h.bucketed) {
+  if (bucketed) {
     *word = uint32_t(col) | kFirstBit;  // a first occurrence until the bucketed pass says otherwise; the table is left alone
     return true;
   }
@@ -360,10 +396,10 @@ __device__ __forceinline__ bool place_pick(const Hop& h, const TableT& table, Id
 // and p's slot word recorded; without one the position is marked empty.
 template <typename IdT, typename TableT>
 __device__ __forceinline__ bool emit_pick(const Hop& h, const TableT& table, const TierView<IdT>& indices, int64_t p,
-                                          bool have, int64_t edge, bool look_first) {
+                                          bool have, int64_t edge, bool look_first, bool bucketed) {
   uint32_t word = kInvalidSlot;
   bool ok = true;
-  if (have) ok = place_pick<IdT>(h, table, indices.at(edge), p, look_first, &word);
+  if (have) ok = place_pick<IdT>(h, table, indices.at(edge), p, look_first, bucketed, &word);
   h.slot[p] = word;
   return ok;
 }
@@ -393,8 +429,7 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   // the wave's table for the search for repeated draws (below) is emptied here, where every lane
   // of the wave is still present
   __shared__ unsigned long long fold_lds[kBlock / kWave][kFoldSlots];
-  const bool fold = replace && !h.bucketed;
-  if (fold) {
+  if (replace) {
     unsigned long long* offers = fold_lds[threadIdx.x / kWave];
 #pragma unroll
     for (int q = 0; q < kFoldSlots / kWave; ++q) offers[q * kWave + (threadIdx.x & (kWave - 1))] = ~0ull;
@@ -404,6 +439,8 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   const IdT seed = i < h.s_max ? static_cast<const IdT*>(h.seeds)[i] : IdT(0);
   const int64_t s = seeds_of(h);
   const bool look_first = look_before_insert(h, s);
+  const bool bucketed = bucketed_now(h, s);
+  const bool fold = replace && !bucketed;
   if (h.n_seeds_out && vb == 0 && threadIdx.x == 0) *h.n_seeds_out = s;
   if (i >= s) return;  // whole groups leave together
   const int group_lane0 = (threadIdx.x & (kWave - 1)) - l;
@@ -459,7 +496,7 @@ __device__ __forceinline__ void fill_rows(const Hop& h, int64_t vb, const TableT
   }
   uint32_t word = kInvalidSlot;
   bool pick_ok = true;
-  if (live && leader == l) pick_ok = place_pick<IdT>(h, table, indices.at(b + pos), p, look_first, &word);
+  if (live && leader == l) pick_ok = place_pick<IdT>(h, table, indices.at(b + pos), p, look_first, bucketed, &word);
   if (fold) {
     const uint32_t leader_word = __shfl(word, leader, G);
     const int leader_ok = __shfl(int(pick_ok), leader, G);
@@ -489,7 +526,7 @@ __global__ __launch_bounds__(kBlock) void hop_fill_kernel(Hop h, Hop prev, int64
   DGS_FOR_VIRTUAL_BLOCKS(vb, total) {
     if (vb < fill_blocks) {
       fill_rows<IdT, PtrT, TableT, G, !STRIDE>(h, vb, table, indptr, indices, replace, rng_seed);
-    } else if (vb < fill_blocks + relabel_count) {
+    } else if (!STRIDE && vb < fill_blocks + relabel_count) {  // (a striding launch is given no such blocks)
       relabel_tile<IdT, TableT, !STRIDE>(prev, table, vb - fill_blocks);
     } else {
       const int64_t i = (vb - fill_blocks - relabel_count) * kBlock + threadIdx.x;
@@ -576,7 +613,8 @@ __device__ __forceinline__ void fill_rows_weighted(const Hop& h, int64_t vb, con
   }
   bool pick_ok = true;
   if (i < s && l < k && !is_long)
-    pick_ok = emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, pick < deg, b + pick, look_first);
+    pick_ok = emit_pick<IdT>(h, table, indices, h.pos_base + seed_part(h, s) + i * k + l, pick < deg, b + pick, look_first,
+                             bucketed_now(h, s));
   const uint64_t row_mask = lanes == kWave ? ~uint64_t(0) : ((uint64_t(1) << lanes) - 1);
   const bool picks_ok = ((__ballot(!pick_ok) >> (mine * lanes)) & row_mask) == 0;
   if (i < s && l == 0)
@@ -615,6 +653,7 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
   const int64_t n_long = *h.long_count;
   const int64_t s = seeds_of(h);
   const bool look_first = look_before_insert(h, s);
+  const bool bucketed = bucketed_now(h, s);
   const int k = h.k;
   for (int64_t t = blockIdx.x; t < n_long; t += gridDim.x) {
     const int64_t i = h.long_rows[t];
@@ -625,12 +664,14 @@ __global__ __launch_bounds__(kLongBlock) void hop_fill_weighted_long_kernel(Hop 
     if (REPLACE) {
       draw_long_row(lds, probs, b, int64_t(deg), int64_t(k), rng_seed, h.rng_stream, row,
                     [&](int64_t j, int64_t pick) {
-                      if (!emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first)) h.row_cnt[i] = kBadPick;
+                      if (!emit_pick<IdT>(h, table, indices, p0 + j, true, b + pick, look_first, bucketed))
+                        h.row_cnt[i] = kBadPick;
                     });
     } else {
       const uint32_t pos = race_long_row(lds, probs, b, deg, k, rng_seed, h.rng_stream, row);
       const int l = threadIdx.x;  // wave 0 holds the winners
-      if (l < k && !emit_pick<IdT>(h, table, indices, p0 + l, pos < deg, b + pos, look_first)) h.row_cnt[i] = kBadPick;
+      if (l < k && !emit_pick<IdT>(h, table, indices, p0 + l, pos < deg, b + pos, look_first, bucketed))
+        h.row_cnt[i] = kBadPick;
     }
   }
 }
@@ -691,19 +732,22 @@ __global__ __launch_bounds__(kBlock) void bucket_sort_kernel(Hop h, Buckets b) {
   __shared__ int cnt[kMaxBuckets];     // units per bucket, then the next free place of every bucket in the stage
   __shared__ uint2 stage[kBucketTile];
   __shared__ int lds[kBlock / kWave];
-  const int buckets = 1 << b.log_buckets;
-  const int mine = buckets / kBlock;  // 2..8 consecutive buckets per thread
+  if (blockIdx.x == 0 && threadIdx.x == 0) *h.bucket_overflow = 0;  // (the per-bucket launch comes behind this one)
   for (int64_t tile = blockIdx.x; tile < b.tiles_max; tile += gridDim.x) {
     const TileOfUnits t = bucket_tile(b, tile);
     UnitsOfThread<IdT> units;
     units.load(h, t);
     const int64_t s = seeds_of(h);
+    if (!bucketed_now(h, s)) return;           // the hop outgrew the pass: it runs on the table
     if (!bucket_tile_live(h, t, s)) continue;  // whole blocks skip a tile together
+    const int log_buckets = log_buckets_of(b, h, s);
+    const int buckets = 1 << log_buckets;
+    const int mine = buckets / kBlock;  // 1..8 consecutive buckets per thread
     for (int j = threadIdx.x; j < buckets; j += kBlock) cnt[j] = 0;
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < kBucketTileItems; ++j)
-      if (units.valid(h, t, s, j)) atomicAdd(&cnt[units.id[j] & uint32_t(buckets - 1)], 1);
+      if (units.valid(h, t, s, j)) atomicAdd(&cnt[bucket_of(b, log_buckets, units.id[j])], 1);
     __syncthreads();
     int own[kMaxBuckets / kBlock];
     int sum = 0;
@@ -728,7 +772,7 @@ __global__ __launch_bounds__(kBlock) void bucket_sort_kernel(Hop h, Buckets b) {
 #pragma unroll
     for (int j = 0; j < kBucketTileItems; ++j) {
       if (units.valid(h, t, s, j)) {
-        const int to = atomicAdd(&cnt[units.id[j] & uint32_t(buckets - 1)], 1);
+        const int to = atomicAdd(&cnt[bucket_of(b, log_buckets, units.id[j])], 1);
         if (to >= 0 && to < kBucketTile) stage[to] = make_uint2(units.id[j], units.order[j]);
       }
     }
@@ -752,6 +796,7 @@ __global__ __launch_bounds__(kBlock) void bucket_first_kernel(Hop h, Buckets b) 
   const uint32_t range = (b.n_nodes + uint32_t(buckets) - 1) >> b.log_buckets;  // <= kBucketRange by the plan
   const uint32_t pos_begin = uint32_t(h.pos_base), pos_end = uint32_t(h.pos_base + h.len_max);
   const int64_t s = seeds_of(h);
+  if (!bucketed_now(h, s)) return;
   const int tiles = b.tiles_max < kMaxBucketTiles ? b.tiles_max : kMaxBucketTiles;
   const int64_t item_count = int64_t(b.tiles_max) * kBucketTile;
   for (int bucket = blockIdx.x; bucket < buckets; bucket += gridDim.x) {
@@ -828,6 +873,152 @@ __global__ __launch_bounds__(kBlock) void bucket_first_kernel(Hop h, Buckets b) 
       const uint32_t least = best[at];  // first occurrences keep the word the fill gave them
       if (least != it.y) h.slot[it.y] = least < pos_begin ? (least | kRankBit) : least;
     }
+    __syncthreads();
+  }
+}
+
+// The per-bucket kernel for graphs of any node count: as bucket_first_kernel, but a bucket's ids
+// are told apart in an open-addressing table in LDS (the id claims a slot with a compare-and-swap,
+// the slot's second word takes the smallest order value), since an array indexed by the id itself
+// would not fit.  Buckets are chosen by low bits of a hash of the id, slots by the next bits.
+// A bucket with more units than three quarters of the table's slots (its ids might not fit) is
+// gone over in parts, by yet other bits of the hash, one table's worth at a time.  Ids that crowd
+// one part all the same (more than kHashSlots distinct ones: not by chance) set the hop's overflow
+// word, which fails the call.
+__global__ __launch_bounds__(kHashBlock) void bucket_first_hashed_kernel(Hop h, Buckets b) {
+  __shared__ uint32_t owner[kHashSlots];
+  __shared__ uint32_t best[kHashSlots];
+  __shared__ int piece_at[kMaxBucketTiles];      // first unit of the tile's piece, as an index into items[]
+  __shared__ int piece_before[kMaxBucketTiles];  // units of the bucket in the tiles before
+  __shared__ int lds[kHashBlock / kWave];
+  __shared__ int overflow;
+  const uint32_t pos_begin = uint32_t(h.pos_base), pos_end = uint32_t(h.pos_base + h.len_max);
+  const int64_t s = seeds_of(h);
+  if (!bucketed_now(h, s)) return;
+  const int log_buckets = log_buckets_of(b, h, s);
+  const int buckets = 1 << log_buckets;
+  const int tiles = b.tiles_max < kMaxBucketTiles ? b.tiles_max : kMaxBucketTiles;
+  const int64_t item_count = int64_t(b.tiles_max) * kBucketTile;
+  for (int bucket = blockIdx.x; bucket < buckets; bucket += gridDim.x) {
+    if (threadIdx.x == 0) overflow = 0;
+    constexpr int kRounds = kMaxBucketTiles / kHashBlock;
+    int from[kRounds], upto[kRounds];
+#pragma unroll
+    for (int q = 0; q < kRounds; ++q) {
+      const int tile = q * kHashBlock + threadIdx.x;
+      from[q] = upto[q] = 0;
+      if (tile < tiles && bucket_tile_live(h, bucket_tile(b, tile), s)) {
+        const uint16_t* piece = b.piece + int64_t(tile) * (buckets + 1);
+        from[q] = piece[bucket];
+        upto[q] = piece[bucket + 1];
+      }
+    }
+    int total = 0;
+#pragma unroll
+    for (int q = 0; q < kRounds; ++q) {
+      if (q * kHashBlock >= tiles) break;  // the same for every thread
+      const int tile = q * kHashBlock + threadIdx.x;
+      const int count = from[q] <= upto[q] && upto[q] <= kBucketTile ? upto[q] - from[q] : 0;
+      int sum;
+      const int before = block_exclusive_scan<kHashBlock, int>(count, &sum, lds);
+      if (tile < tiles) {
+        piece_at[tile] = tile * kBucketTile + from[q];
+        piece_before[tile] = total + before;
+      }
+      total += sum;
+    }
+    // The table is as large as the bucket needs: at least twice its units (all of them may be
+    // distinct ids), all of the array when that is not enough; beyond three quarters of the array
+    // the bucket is split into parts.
+    const int capacity = b.hash_slots;
+    const int parts = total <= capacity * 3 / 4 ? 1 : (total + capacity / 2 - 1) / (capacity / 2);
+    int slots = capacity < 1024 ? capacity : 1024;
+    while (slots < 2 * (total / parts + 1) && slots < capacity) slots <<= 1;
+    const uint32_t slot_mask = uint32_t(slots - 1);
+    __syncthreads();  // piece_at / piece_before are complete
+    const auto unit = [&](int j) {
+      int lo = 0, hi = tiles - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (piece_before[mid] <= j) lo = mid; else hi = mid - 1;
+      }
+      const int64_t at = int64_t(piece_at[lo]) + (j - piece_before[lo]);
+      return at >= 0 && at < item_count ? b.items[at] : make_uint2(kHashEmpty, 0u);
+    };
+    // where an id's slot search starts, and which part it belongs to: bits of its hash that the
+    // choice of the bucket did not use
+    const auto home = [&](uint32_t hash) { return (hash >> log_buckets) & slot_mask; };
+    const auto part_of = [&](uint32_t hash) { return int((hash >> 23) % uint32_t(parts)); };
+    constexpr int kKept = 8;  // a thread's first units stay in registers across the passes
+    uint2 kept[kKept];
+#pragma unroll
+    for (int r = 0; r < kKept; ++r) {
+      const int j = threadIdx.x + r * kHashBlock;
+      kept[r] = j < total ? unit(j) : make_uint2(kHashEmpty, 0u);
+    }
+    for (int part = 0; part < parts; ++part) {
+      for (int j = threadIdx.x; j < slots; j += kHashBlock) {
+        owner[j] = kHashEmpty;
+        best[j] = 0xffffffffu;
+      }
+      __syncthreads();
+      // every unit of the part claims its id's slot (or finds it claimed by the same id) and offers its order value
+      uint32_t kept_slot[kKept];
+#pragma unroll
+      for (int r = 0; r < kKept; ++r) kept_slot[r] = kHashEmpty;
+      for (int j = threadIdx.x, r = 0; j < total; j += kHashBlock, ++r) {
+        uint2 it = make_uint2(kHashEmpty, 0u);
+        if (r < kKept) {
+#pragma unroll
+          for (int q = 0; q < kKept; ++q) if (q == r) it = kept[q];
+        } else {
+          it = unit(j);
+        }
+        if (it.x == kHashEmpty) continue;
+        const uint32_t hash = hash_id(it.x);
+        if (parts > 1 && part_of(hash) != part) continue;
+        uint32_t slot = home(hash);
+        bool placed = false;
+        for (int probes = 0; probes < slots; ++probes) {
+          uint32_t seen = owner[slot];
+          if (seen == kHashEmpty) seen = atomicCAS(&owner[slot], kHashEmpty, it.x);
+          if (seen == kHashEmpty || seen == it.x) {
+            placed = true;
+            break;
+          }
+          slot = (slot + 1) & slot_mask;
+        }
+        if (placed) atomicMin(&best[slot], it.y); else overflow = 1;
+        if (r < kKept) {
+#pragma unroll
+          for (int q = 0; q < kKept; ++q) if (q == r) kept_slot[q] = placed ? slot : kHashEmpty;
+        }
+      }
+      __syncthreads();
+      if (overflow == 0) {  // (an overflowing part's answers are void: the call fails, nothing is rewritten)
+        for (int j = threadIdx.x, r = 0; j < total; j += kHashBlock, ++r) {
+          uint2 it = make_uint2(kHashEmpty, 0u);
+          uint32_t slot = kHashEmpty;
+          if (r < kKept) {
+#pragma unroll
+            for (int q = 0; q < kKept; ++q) if (q == r) { it = kept[q]; slot = kept_slot[q]; }
+          } else {
+            it = unit(j);
+          }
+          if (it.x == kHashEmpty || it.y < pos_begin || it.y >= pos_end) continue;  // not a pick of this hop
+          const uint32_t hash = hash_id(it.x);
+          if (parts > 1 && part_of(hash) != part) continue;
+          if (slot == kHashEmpty) {  // beyond what the registers kept: find the id's slot again
+            slot = home(hash);
+            for (int probes = 0; probes < slots && owner[slot] != it.x; ++probes) slot = (slot + 1) & slot_mask;
+          }
+          const uint32_t least = best[slot];  // first occurrences keep the word the fill gave them
+          if (least != it.y) h.slot[it.y] = least < pos_begin ? (least | kRankBit) : least;
+        }
+      }
+      __syncthreads();
+    }
+    if (threadIdx.x == 0 && overflow != 0) *h.bucket_overflow = 1;
     __syncthreads();
   }
 }
@@ -941,6 +1132,7 @@ __device__ __forceinline__ void compact_tile(const Hop& h, int64_t tile, int64_t
     // (row tiles were scanned by the surplus blocks of the flag launch) and error bits
     edges = block_sum<kBlock, int64_t>(edges, lds64);
     bad = block_or<kBlock>(bad, lds);
+    if (h.bucketed != 0 && *h.bucket_overflow != 0) bad |= kErrBucketOverflow;
     if (threadIdx.x == 0) {
       *h.n_unique = rank0 + part;
       *h.nnz = edges;
@@ -1005,14 +1197,26 @@ struct Plan {
   uint32_t capacity = 0;     // hash table slots (one table for all hops)
   size_t table_bytes = 0;    // 0 for the direct table
   bool weighted = false;     // picks by edge weight: per-hop queues for long rows
-  bool bucketed = false;     // the last hop finds its first occurrences by the bucketed pass
+  bool bucketed = false;     // the last hop may find its first occurrences by the bucketed pass (if it turns out to fit)
+  bool bucket_hashed = false; // ... with ids told apart by an LDS hash table (graphs beyond kBucketedMaxNodes)
   bool bucket_space = false; // the workspace has room for that pass
+  int32_t bucket_front_tiles = 0;  // tiles over the frontier array as large as it can be before the last hop
+  int32_t bucket_pos_tiles = 0;    // tiles over the last hop's padded positions: all of them, or as many as there is room for
   int32_t log_buckets = 0;
+  int32_t hash_slots = kHashSlots;
   uint32_t n_nodes = 0;
 };
 
-// units (frontier ids + padded positions) the bucketed pass of the last hop handles at most
-inline int64_t bucket_units_max(const Plan& p) { return p.s_max[p.n_hops]; }
+// Tiles of the bucketed pass: the frontier before the last hop at its worst case, and as many of the
+// hop's padded positions as the per-bucket kernels can index (a hop beyond that runs on the table).
+inline void plan_bucket_tiles(Plan* p) {
+  const int64_t front = (p->s_max[p->n_hops - 1] + kBucketTile - 1) / kBucketTile;
+  const int64_t pos = (p->nnz_max[p->n_hops - 1] + kBucketTile - 1) / kBucketTile;
+  const int64_t room = int64_t(kMaxBucketTiles) - 2 - front;
+  p->bucket_space = p->n_hops >= 2 && room >= 1;
+  p->bucket_front_tiles = int32_t(front);
+  p->bucket_pos_tiles = int32_t(pos < room ? pos : (room > 0 ? room : 0));
+}
 
 dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, int32_t id_bytes,
                      int64_t n_nodes, bool have_node_table, Plan* p) {
@@ -1031,21 +1235,39 @@ dgs_status make_plan(int64_t n_seeds, const int64_t* fanouts, int32_t n_hops, in
     DGS_REQUIRE(p->s_max[h + 1] <= kMaxPositions, DGS_ERR_UNSUPPORTED,
                 "sample_blocks: worst-case frontier of hop %d exceeds 2^30 ids", h);
   }
-  // room for the bucketed pass whenever its size is bounded (whether it runs is decided below)
-  p->bucket_space = n_hops >= 2 && bucket_units_max(*p) <= kBucketedMaxUnits;
+  // room for the bucketed pass (whether a hop takes it is decided below and, from its real size, on the device)
+  plan_bucket_tiles(p);
   if (have_node_table) {
     DGS_REQUIRE(n_nodes >= 0 && n_nodes < 0x7fffffffLL, DGS_ERR_UNSUPPORTED,
                 "sample_blocks: a node table needs fewer than 2^31 nodes (have %lld)", (long long)n_nodes);
     p->kind = TableKind::kDirect;
-    // the bucketed pass: slot words are ids (the direct table's), ids fit the LDS arrays, and the
-    // hop is large enough for its two extra launches to cost less than the atomics they replace
-    // (test hook: 1 never, 2 whatever the size)
+    // the bucketed pass: slot words are ids (the direct table's), and the hop is large enough for
+    // its two extra launches to cost less than the atomics they replace.  Ids that fit the LDS
+    // array of a bucket (kBucketRange ids in each of at most kMaxBuckets buckets) index it directly;
+    // larger graphs take the hashed form.
+    // (test hook: 1 never, 2 whatever the size, 3 whatever the size and hashed whatever the graph,
+    // 4 like 3 with on-chip tables of 256 slots, so that small inputs fill them and go over their
+    // buckets in parts)
     const int64_t mode = debug_option(DGS_DEBUG_SAMPLER_BUCKETED);
     const bool large = p->nnz_max[n_hops - 1] >= kBucketedMinPicks;
-    p->bucketed = p->bucket_space && n_nodes >= 1 && n_nodes <= kBucketedMaxNodes && fanouts[n_hops - 1] >= 1 &&
-                  mode != 1 && (large || mode == 2);
+    p->bucket_hashed = n_nodes > kBucketedMaxNodes || mode == 3 || mode == 4;
+    // By size only the direct form runs.  The hashed form gives the same results on any graph and
+    // takes the atomics out of the hop just the same, but it does not pay: 111 M nodes, 944 k picks
+    // of mostly new ids: fill 64 -> 35 us and relabel 14 -> 12, against 19 + 22 us for its two
+    // launches (0.187-0.200 ms per step in flight against 0.191); R-MAT with two thirds repeats: every
+    // repeat costs a scattered 4-byte store where the table's look before the atomic gets cheaper
+    // (0.382 against 0.373 ms).  It runs when the test hook asks for it.
+    p->bucketed = p->bucket_space && n_nodes >= 1 && fanouts[n_hops - 1] >= 1 && mode != 1 &&
+                  (p->bucket_hashed ? mode >= 2 : (large || mode >= 2));
+    p->hash_slots = mode == 4 ? 256 : kHashSlots;
     int log_b = 0;
-    while ((1 << log_b) < kMinBuckets || (int64_t(kBucketRange) << log_b) < n_nodes) ++log_b;
+    if (p->bucket_hashed) {
+      // a bucket's LDS table takes kHashSlots ids: at most half as many units per bucket on average
+      const int64_t units = int64_t(p->bucket_front_tiles + p->bucket_pos_tiles) * kBucketTile;
+      while ((1 << log_b) < kMinBuckets || ((int64_t(kHashSlots) << log_b) < units && (1 << log_b) < kMaxBuckets)) ++log_b;
+    } else {
+      while ((1 << log_b) < kMinBuckets || (int64_t(kBucketRange) << log_b) < n_nodes) ++log_b;
+    }
     p->log_buckets = log_b;
     p->n_nodes = uint32_t(n_nodes);
   } else {
@@ -1095,20 +1317,39 @@ size_t layout(const Plan& p, const int64_t* fanouts, void* base, Hop* hops, void
     v.k = int32_t(fanouts[h]);
     v.index = h;
     v.bucketed = p.bucketed && h == p.n_hops - 1;
+    v.bucket_pos_cap = int64_t(p.bucket_pos_tiles) * kBucketTile;
     if (hops) hops[h] = v;
     pos_base += int64_t(len);
   }
   if (p.bucket_space) {
     Buckets b{};
-    b.front_tiles = int32_t((p.s_max[p.n_hops - 1] + kBucketTile - 1) / kBucketTile);
-    b.tiles_max = b.front_tiles + int32_t((p.nnz_max[p.n_hops - 1] + kBucketTile - 1) / kBucketTile);
+    b.front_tiles = p.bucket_front_tiles;
+    b.tiles_max = p.bucket_front_tiles + p.bucket_pos_tiles;
     b.items = c.take<uint2>(size_t(b.tiles_max) * kBucketTile);
     b.piece = c.take<uint16_t>(size_t(b.tiles_max) * (kMaxBuckets + 1));
+    int* overflow = c.take<int>(4);
     b.log_buckets = p.log_buckets;
     b.n_nodes = p.n_nodes;
+    b.hashed = p.bucket_hashed ? 1 : 0;
+    b.hash_slots = p.hash_slots;
     if (buckets) *buckets = b;
+    if (hops)
+      for (int h = 0; h < p.n_hops; ++h) hops[h].bucket_overflow = overflow;
   }
   return c.used + 256;
+}
+
+// The packed edge list of one hop as a launch of its own.
+template <typename IdT, typename TableT>
+void launch_relabel(const Hop& hop, const TableT& table, hipStream_t st) {
+  const int64_t blocks = relabel_blocks(hop.s_max, hop.k);
+  if (blocks <= 0) return;
+  if (is_capped(blocks))
+    hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT, true>), dim3(capped_grid(blocks)), dim3(kBlock), 0, st, hop,
+                       blocks, table);
+  else
+    hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT, false>), dim3(capped_grid(blocks)), dim3(kBlock), 0, st, hop,
+                       blocks, table);
 }
 
 template <typename IdT, typename PtrT, typename TableT, int G>
@@ -1117,12 +1358,18 @@ void launch_fill(const Hop& cur, const Hop& prev, int64_t relabel_count, uint4* 
                  uint64_t rng_seed, hipStream_t st) {
   const int64_t fill_blocks = (cur.s_max * G + kBlock - 1) / kBlock;
   const int64_t clear_blocks = (clear_n16 + kBlock - 1) / kBlock;
-  const int64_t total = fill_blocks + relabel_count + clear_blocks;
-  if (is_capped(total))
+  int64_t total = fill_blocks + relabel_count + clear_blocks;
+  if (is_capped(total)) {
+    // A launch that loops over its virtual blocks keeps the previous hop's edge list out of the
+    // loop: with it the kernel needs 85-90 vector registers and five waves fit a SIMD instead of
+    // seven (measured on a 136 k-row hop: 46 us against 39).  That list becomes a launch of its own,
+    // behind this one (the previous hop's table entries do not change any more: positions only grow).
+    total -= relabel_count;
     hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G, true>), dim3(capped_grid(total)), dim3(kBlock), 0, st,
-                       cur, prev, fill_blocks, relabel_count, clear_begin, clear_n16, table,
+                       cur, prev, fill_blocks, int64_t(0), clear_begin, clear_n16, table,
                        TierView<PtrT>(indptr), TierView<IdT>(indices), replace, rng_seed);
-  else
+    if (relabel_count > 0) launch_relabel<IdT>(prev, table, st);
+  } else
     hipLaunchKernelGGL((hop_fill_kernel<IdT, PtrT, TableT, G, false>), dim3(capped_grid(total)), dim3(kBlock), 0, st,
                        cur, prev, fill_blocks, relabel_count, clear_begin, clear_n16, table,
                        TierView<PtrT>(indptr), TierView<IdT>(indices), replace, rng_seed);
@@ -1188,7 +1435,11 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const Buckets& buckets, const Ta
       hipLaunchKernelGGL(bucket_sort_kernel<IdT>, dim3(capped_grid(buckets.tiles_max)), dim3(kBlock), 0, st, cur,
                          buckets);
       DGS_LAUNCH_CHECK();
-      hipLaunchKernelGGL(bucket_first_kernel, dim3(capped_grid(n_buckets)), dim3(kBlock), 0, st, cur, buckets);
+      if (buckets.hashed)
+        hipLaunchKernelGGL(bucket_first_hashed_kernel, dim3(capped_grid(n_buckets)), dim3(kHashBlock), 0, st, cur,
+                           buckets);
+      else
+        hipLaunchKernelGGL(bucket_first_kernel, dim3(capped_grid(n_buckets)), dim3(kBlock), 0, st, cur, buckets);
       DGS_LAUNCH_CHECK();
     }
 
@@ -1224,17 +1475,8 @@ dgs_status run_blocks(const Plan& p, Hop* hops, const Buckets& buckets, const Ta
     const dgs_status ts = dgs_ticket_record(st, sizes_ticket);
     if (ts != DGS_OK) return ts;
   }
-  const Hop& last = hops[p.n_hops - 1];
-  const int64_t last_blocks = relabel_blocks(last.s_max, last.k);
-  if (last_blocks > 0) {
-    if (is_capped(last_blocks))
-      hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT, true>), dim3(capped_grid(last_blocks)), dim3(kBlock), 0,
-                         st, last, last_blocks, table);
-    else
-      hipLaunchKernelGGL((hop_relabel_kernel<IdT, TableT, false>), dim3(capped_grid(last_blocks)), dim3(kBlock), 0,
-                         st, last, last_blocks, table);
-    DGS_LAUNCH_CHECK();
-  }
+  launch_relabel<IdT>(hops[p.n_hops - 1], table, st);
+  DGS_LAUNCH_CHECK();
   return DGS_OK;
 }
 
@@ -1314,7 +1556,7 @@ dgs_status sample_blocks_entry(const void* seeds, int32_t id_bytes, int64_t n_se
     p.weighted = true;
     // weighted picks: the fill is bound by the races, not by its atomics, and the bucketed pass
     // changes the step by a per cent either way (measured with three and four batches in flight)
-    if (debug_option(DGS_DEBUG_SAMPLER_BUCKETED) != 2) p.bucketed = false;
+    if (debug_option(DGS_DEBUG_SAMPLER_BUCKETED) < 2) p.bucketed = false;
   }
   const size_t need = probs != nullptr ? dgs_sample_blocks_weighted_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes)
                                        : dgs_sample_blocks_workspace_bytes(n_seeds, fanouts, n_hops, id_bytes);

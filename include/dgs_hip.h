@@ -59,7 +59,11 @@ int dgs_abi_version(void);
  *                                table finds its first occurrences: 0 by size (the bucketed LDS
  *                                pass for a large hop of uniform picks, the table's atomics
  *                                otherwise), 1 always the table, 2 the bucketed pass whatever
- *                                the size and the kind of picks
+ *                                the size and the kind of picks, 3 like 2 and in the form for
+ *                                graphs of any node count (buckets by a hash of the id, an LDS
+ *                                hash table per bucket) whatever the graph's size, 4 like 3 with
+ *                                those tables cut to 256 slots (small inputs then fill them and
+ *                                are gone over in parts)
  */
 enum {
   DGS_DEBUG_FORCE_SPLIT_TABLE = 0,
@@ -420,7 +424,12 @@ typedef struct dgs_block_out {
  *                                                          offsets outside the edge array, 2 a seed id is
  *                                                          not a row of the graph, 4 a picked neighbour id
  *                                                          is not a node (each checked before it addresses
- *                                                          anything; such rows emit nothing)
+ *                                                          anything; such rows emit nothing), 8 the last hop's
+ *                                                          bucketed pass met a bucket with more distinct ids
+ *                                                          than its on-chip table holds (the hop's results are
+ *                                                          void; ids that crowd one bucket of the library's
+ *                                                          hash: run the call again with
+ *                                                          DGS_DEBUG_SAMPLER_BUCKETED = 1)
  *   sizes_host / ticket    : optional (a ticket only with sizes_host).  sizes_host is pinned host
  *                            memory that the device can write (hipHostMalloc); the kernels mirror
  *                            sizes_dev into it, and *sizes_ticket marks the point on `stream`

@@ -24,11 +24,14 @@ def np_unique_first(x):
     return u[np.argsort(first, kind="stable")]
 
 
-LAST_HOP_MODES = ["last hop by size", "last hop bucketed"]
+LAST_HOP_MODES = ["last hop by size", "last hop bucketed", "last hop bucketed by hash", "last hop bucketed by hash in parts"]
 
 
 def set_last_hop_mode(pkg, mode):
     """How the fused sampler's last hop finds its first occurrences in this test: by size (small
-    test inputs then take the node table's atomics) or always through the bucketed LDS pass."""
+    test inputs then take the node table's atomics), always through the bucketed LDS pass, or
+    always through the form of that pass for graphs of any node count (buckets by a hash of the id),
+    or through that form with on-chip tables so small that buckets are gone over in parts."""
     capi = pkg.capi
-    capi.check(capi.lib.dgs_debug_set(capi.DEBUG_SAMPLER_BUCKETED, 2 if mode == LAST_HOP_MODES[1] else 0))
+    capi.check(capi.lib.dgs_debug_set(capi.DEBUG_SAMPLER_BUCKETED, {LAST_HOP_MODES[0]: 0, LAST_HOP_MODES[1]: 2,
+                                                                    LAST_HOP_MODES[2]: 3, LAST_HOP_MODES[3]: 4}[mode]))
