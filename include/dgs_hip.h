@@ -447,7 +447,12 @@ typedef struct dgs_block_out {
  *                            call that uses it, and do not share it between calls that may run
  *                            concurrently.  With NULL the call builds a hash table inside the
  *                            workspace instead (one extra clearing launch, slower inserts).
- * Fanouts above 64 are DGS_ERR_UNSUPPORTED here (use the per-hop entry points).
+ * Limits of this entry point (each is DGS_ERR_UNSUPPORTED, none is silent): fanouts above 64 (use
+ * the per-hop entry points, which take any fanout); a worst-case frontier S * prod(1 + k_h) above
+ * 2^30 ids (positions are 32-bit words with two flag bits); a node table for 2^31 nodes or more
+ * (dgs_node_table_bytes returns 0).  The operator layer above adds two of its own: it makes node
+ * tables only below 8 GiB each (larger graphs sample on the per-call hash table) and keeps at
+ * most four per graph, one per stream that samples from it.
  */
 dgs_status dgs_sample_blocks_plan(int64_t n_seeds, const int64_t* fanouts,
                                   int32_t n_hops, int64_t* seeds_max,
