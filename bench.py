@@ -351,6 +351,9 @@ LARGE = {
     "c4": dict(graph="rmat", nodes=1 << 26, edges=1 << 30, dim=64, feat_dtype=torch.float32,
                hbm_rows=1.0, batch=16384, fanouts=[50, 50], replace=True, train_frac=1.0, seed=20240605),
 }
+# batches in flight by default: the best of 2..5 measured on each (c2: 0.176-0.187 ms per step with four against
+# 0.189-0.194 with three; c4: three and four are level and three hold less memory; a two-tier c3 batch runs alone)
+LARGE_INFLIGHT = {"c2": 4, "c3": 3, "c4": 3}
 
 
 def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8):
@@ -622,7 +625,7 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="size factor of the c2/c3/c4 workloads (1.0 = full)")
     ap.add_argument("--inflight", type=int, default=None,
                     help="batches in flight on as many streams (1 = one blocking call per batch); default 4 for "
-                         "c0/c1/c1w and 3 for the large workloads (measured best of 2..4 on each)")
+                         "c0/c1/c1w/c2 and 3 for c3/c4 (measured best of 2..5 on each; c3 always runs one)")
     ap.add_argument("--gather-buffer-cap-gib", type=float, default=None,
                     help="largest feature buffer the fused operator allocates ahead of a batch's sizes "
                          "(the library's default when not given)")
@@ -651,7 +654,7 @@ def main():
     dgs = importlib.import_module("dist-gpu-sampling_amd")
     torch.cuda.set_device(0)
     if args.inflight is None:
-        args.inflight = 4 if args.workload in WORKLOADS else 3
+        args.inflight = LARGE_INFLIGHT.get(args.workload, 4)
     if args.gather_buffer_cap_gib is not None:
         dgs.set_gather_buffer_cap(int(args.gather_buffer_cap_gib * (1 << 30)))
     if args.last_hop:
@@ -955,7 +958,7 @@ def main():
 
         guarded("c1w", c1w_leg)
         for name in ("c2", "c4", "c3"):
-            guarded(name, lambda name=name: measure_large(name, dgs, k_other, w_other, 3))
+            guarded(name, lambda name=name: measure_large(name, dgs, k_other, w_other, LARGE_INFLIGHT[name]))
         # what the hottest-rows-first placement buys where a node's popularity follows its degree
         # (the benchmark's own c3 draws sources uniformly: there the hot prefix catches its row share)
         guarded("c3_placement", lambda: measure_placement(dgs))
