@@ -634,7 +634,8 @@ def main():
                          "node tables (the library's default when not given)")
     ap.add_argument("--last-hop", type=int, default=0,
                     help="how the fused sampler's last hop finds first occurrences (the library's test hook "
-                         "DGS_DEBUG_SAMPLER_BUCKETED): 0 by size, 1 always on the node table, 2 always the bucketed pass")
+                         "DGS_DEBUG_SAMPLER_BUCKETED): 0 by size, 1 always on the node table, 2 always the bucketed pass, "
+                         "3 / 4 its hashed form for graphs of any node count (16384- / 256-slot LDS tables)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with --workload c1: do not also run c1w, c2, c4 and c3 after the headline")
