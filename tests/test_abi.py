@@ -158,6 +158,46 @@ def test_query_entry_points_check_their_arguments():
     assert b"ticket_query" in capi.lib.dgs_last_error()
 
 
+def test_fused_plan_arithmetic_and_limits():
+    # host-only parts of the fused sampler's entry points: worst-case sizes by hand (hop h adds seeds * k picks
+    # to a frontier that already holds the seeds), and the limits stated beside dgs_sample_blocks
+    import ctypes
+    capi = load_pkg().capi
+    lib, c_i64 = capi.lib, capi.c_i64
+
+    def plan(n, fanouts):
+        fan = (c_i64 * max(len(fanouts), 1))(*fanouts)
+        smax, emax = (c_i64 * (len(fanouts) + 1))(), (c_i64 * max(len(fanouts), 1))()
+        return lib.dgs_sample_blocks_plan(n, fan, len(fanouts), smax, emax), list(smax), list(emax)
+
+    # benchmark configuration 1 in hop order: 1024 seeds, fanouts 5, 10, 15
+    assert plan(1024, [5, 10, 15]) == (0, [1024, 6144, 67584, 1081344], [5120, 61440, 1013760])
+    assert plan(0, [7]) == (0, [0, 0], [0])
+    assert plan(3, [0, 64]) == (0, [3, 3, 195], [0, 192])
+    st, _, _ = plan(10, [65])
+    assert st == capi.DGS_ERR_UNSUPPORTED and b"per-hop" in lib.dgs_last_error()
+    assert plan(10, [-1])[0] == capi.DGS_ERR_UNSUPPORTED
+    # 2^30 ids is the largest worst-case frontier: 2^24 seeds x (1 + 63) fits exactly, one seed more does not
+    assert plan(1 << 24, [63])[0] == 0
+    st, _, _ = plan((1 << 24) + 1, [63])
+    assert st == capi.DGS_ERR_UNSUPPORTED and b"2^30" in lib.dgs_last_error()
+    assert plan(16384, [50, 50, 50])[0] == capi.DGS_ERR_UNSUPPORTED
+    assert plan(10, [])[0] == capi.DGS_ERR_INVALID and plan(10, [1] * 9)[0] == capi.DGS_ERR_INVALID  # 1..8 hops
+    assert plan(-1, [3])[0] == capi.DGS_ERR_INVALID
+    fan = (c_i64 * 1)(3)
+    assert lib.dgs_sample_blocks_plan(10, fan, 1, None, None) == capi.DGS_ERR_INVALID
+    # the node table: 8 bytes per node below 2^31 - 1 nodes, none otherwise
+    assert lib.dgs_node_table_bytes(2449029) == 8 * 2449029 and lib.dgs_node_table_bytes(0) == 0
+    assert lib.dgs_node_table_bytes((1 << 31) - 2) == 8 * ((1 << 31) - 2) and lib.dgs_node_table_bytes((1 << 31) - 1) == 0
+    # workspaces: grow with the input, smaller for 4-byte ids, nothing for a plan that is refused
+    fan3 = (c_i64 * 3)(5, 10, 15)
+    small, large = (lib.dgs_sample_blocks_workspace_bytes(n, fan3, 3, 8) for n in (256, 1024))
+    assert 0 < small < large and lib.dgs_sample_blocks_workspace_bytes(1024, fan3, 3, 4) < large
+    assert lib.dgs_sample_blocks_weighted_workspace_bytes(1024, fan3, 3, 8) >= large
+    assert lib.dgs_sample_blocks_workspace_bytes(1024, (c_i64 * 1)(65), 1, 8) == 0
+    assert lib.dgs_sample_blocks_workspace_bytes(1024, fan3, 3, 2) == 0
+
+
 def test_placement_host_arithmetic(oracle):
     # the parts of the placement helpers that need no GPU: degree order, capacity <-> rows, hit rate
     import numpy as np
