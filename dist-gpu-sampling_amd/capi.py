@@ -104,6 +104,13 @@ SIGNATURES = {
 if not os.path.exists(LIB_PATH):
     raise ImportError(f"{LIB_PATH} is missing; build it with dist-gpu-sampling_amd/build.py")
 lib = ctypes.CDLL(LIB_PATH)
+# the signatures above are those of one version of include/dgs_hip.h; a library of another version
+# would take its arguments from the wrong places
+ABI_VERSION = 3
+lib.dgs_abi_version.restype = ctypes.c_int
+if lib.dgs_abi_version() != ABI_VERSION:
+    raise ImportError(f"{LIB_PATH} reports C ABI version {lib.dgs_abi_version()}, this binding is written for "
+                      f"{ABI_VERSION}; rebuild it with dist-gpu-sampling_amd/build.py")
 for _name, (_res, _args) in SIGNATURES.items():
     _f = getattr(lib, _name)
     _f.restype = _res

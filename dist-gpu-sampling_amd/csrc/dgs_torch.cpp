@@ -1189,6 +1189,10 @@ TORCH_LIBRARY(dgs_classes, m) {
 }
 
 TORCH_LIBRARY(dgs_ops, m) {
+  // an operator layer and a kernel library built from different headers would pass each other
+  // arguments in the wrong places: refuse to register on top of such a pair
+  TORCH_CHECK(dgs_abi_version() == DGS_ABI_VERSION, "libdgs_hip.so reports C ABI version ", dgs_abi_version(),
+              ", this operator layer was built against ", DGS_ABI_VERSION, ": rebuild both (build.py)");
   m.def("_CAPI_tensor_relabel", &dgs::TensorRelabel)
       .def("_CAPI_sample_neighbors", &dgs::SampleNeighbors)
       .def("_CAPI_sample_neighbors_with_chunk_tensor", &dgs::SampleNeighborsWithChunkTensor)

@@ -58,7 +58,7 @@ DGS_API const char* dgs_status_name(dgs_status s) {
   }
 }
 
-DGS_API int dgs_abi_version(void) { return 3; }
+DGS_API int dgs_abi_version(void) { return DGS_ABI_VERSION; }
 
 DGS_API dgs_status dgs_debug_set(int32_t option, int64_t value) {
   DGS_REQUIRE(option >= 0 && option < dgs::kDebugOptions, DGS_ERR_INVALID, "debug_set: unknown option %d", option);

@@ -41,7 +41,9 @@ enum {
 const char* dgs_last_error(void);
 /* Static name of a status code. */
 const char* dgs_status_name(dgs_status s);
-/* ABI version of this header (bumped on incompatible change). */
+/* ABI version of this header (bumped on incompatible change): a binding compares what the library
+ * it loaded reports with the DGS_ABI_VERSION it was written against, before any other call. */
+#define DGS_ABI_VERSION 3
 int dgs_abi_version(void);
 /*
  * Test hooks, process-wide: force code paths that small test inputs would not reach by

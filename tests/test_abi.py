@@ -33,7 +33,10 @@ def test_struct_layouts_match_the_header():
     pkg = load_pkg()
     assert ctypes.sizeof(pkg.capi.View) == 40      # 2 pointers + 2 int64 + 2 int32
     assert ctypes.sizeof(pkg.capi.Segments) == 8 * 8 + 8 * 8 + 8
-    assert pkg.capi.lib.dgs_abi_version() == 3
+    # header, library and binding name one version; the binding and the operator layer refuse a library of another
+    header = open(os.path.join(ROOT, "include", "dgs_hip.h")).read()
+    declared = int(re.search(r"#define DGS_ABI_VERSION (\d+)", header).group(1))
+    assert pkg.capi.lib.dgs_abi_version() == declared == pkg.capi.ABI_VERSION == 3
 
 
 def test_store_split_matches_oracle(oracle):
