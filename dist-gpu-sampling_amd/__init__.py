@@ -66,6 +66,7 @@ from .sampler import (  # noqa: E402
     ChunkTensorSampler,
     Block,
     PendingBatch,
+    SeedLoader,
     cached_bytes_per_gpu,
     create_chunktensor,
     create_dgs_communicator,
@@ -83,5 +84,5 @@ from . import loading_factor  # noqa: E402
 ChunkTensor = torch.classes.dgs_classes.ChunkTensor
 ops = torch.ops.dgs_ops
 
-__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "cached_bytes_per_gpu", "create_chunktensor",
+__all__ = ["capi", "placement", "loading_factor", "ops", "ChunkTensor", "ChunkTensorSampler", "BatchPipeline", "Block", "PendingBatch", "SeedLoader", "cached_bytes_per_gpu", "create_chunktensor",
            "create_dgs_communicator", "get_available_memory", "set_rng_state", "set_gather_buffer_cap", "pipeline_streams", "streams_overlap", "lighten_torch_dispatch", "fast_ops", "HIP_LIB", "TORCH_LIB"]

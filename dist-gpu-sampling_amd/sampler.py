@@ -444,3 +444,71 @@ class BatchPipeline:
                 yield self._hand_out(*queue.popleft(), consumer)
         finally:
             spare.append(events)
+
+
+class SeedLoader:
+    """Stands where upstream's training loop has `dgl.dataloading.DataLoader(graph, train_idx, sampler,
+    device='cuda', batch_size=..., shuffle=True, drop_last=False, num_workers=0, use_ddp=True,
+    use_uva=True)` (oppo_bench/single_node/chunktensor.py:123-139), with the same leading arguments:
+
+        for input_nodes, output_nodes, blocks in SeedLoader(graph, train_idx, sampler, batch_size=1024,
+                                                            shuffle=True):
+
+    cuts `indices` into batches of `batch_size` seed ids (a fresh random order per iteration with
+    `shuffle`, the short last batch left out with `drop_last`) and yields what
+    `graph_sampler.sample_blocks(graph, batch)` returns for each.  With `chunk_features` it yields a
+    fourth element, `chunk_features._CAPI_index(input_nodes)`: the loop's next line upstream (:151).
+    Upstream runs one batch at a time (`num_workers=0`); here a fused sampler's batches go through a
+    BatchPipeline with `inflight` of them on the GPU (1: one at a time), and a sampler that cannot
+    run fused (a fanout above 64) is called batch by batch.  `graph` is unused, as in the sampler.
+    `device` moves the seed ids there first (upstream passes 'cuda': batches of device ids are
+    ordered behind the caller's stream; host ids are uploaded by the operator on the batch's own
+    stream).  `generator` is the torch.Generator of the shuffle (CPU).  The DataLoader options that
+    only matter with several ranks or worker processes are accepted and change nothing here.
+    """
+
+    _INERT_OPTIONS = ("use_ddp", "ddp_seed", "use_uva", "use_prefetch_thread", "use_alternate_streams",
+                      "pin_prefetcher", "persistent_workers")
+
+    def __init__(self, graph, indices, graph_sampler, device=None, batch_size=1, shuffle=False, drop_last=False,
+                 num_workers=0, chunk_features=None, inflight=3, generator=None, **options):
+        unknown = sorted(set(options) - set(self._INERT_OPTIONS))
+        if unknown:
+            raise TypeError(f"SeedLoader: unknown option(s) {unknown}")
+        if num_workers != 0:
+            raise ValueError("SeedLoader: num_workers must be 0 (batches overlap on the GPU, not in worker processes)")
+        if batch_size < 1 or inflight < 1:
+            raise ValueError("SeedLoader: batch_size and inflight must be at least 1")
+        indices = torch.as_tensor(indices)
+        if indices.dim() != 1 or indices.dtype not in (torch.int32, torch.int64):
+            raise ValueError("SeedLoader: indices must be a 1-D int32 or int64 tensor")
+        self.indices = indices if device is None else indices.to(device)
+        self.graph_sampler = graph_sampler
+        self.chunk_features = chunk_features
+        self.batch_size = int(batch_size)
+        self.shuffle = bool(shuffle)
+        self.drop_last = bool(drop_last)
+        self.inflight = int(inflight)
+        self.generator = generator
+
+    def __len__(self):
+        n = self.indices.numel()
+        return n // self.batch_size if self.drop_last else -(-n // self.batch_size)
+
+    def _batches(self):
+        ids = self.indices
+        if self.shuffle:
+            ids = ids[torch.randperm(ids.numel(), generator=self.generator).to(ids.device)]
+        return list(ids.split(self.batch_size))[:len(self)]
+
+    def __iter__(self):
+        smp, feats = self.graph_sampler, self.chunk_features
+        batches = self._batches()
+        if getattr(smp, "fused", False) and self.inflight > 1:
+            yield from BatchPipeline(smp, feats, self.inflight)(batches)
+            return
+        for seeds in batches:
+            if feats is None:
+                yield smp.sample_blocks(None, seeds)
+            else:
+                yield smp.sample_blocks_and_index(None, seeds, feats)

@@ -201,6 +201,32 @@ def test_fused_plan_arithmetic_and_limits():
     assert lib.dgs_sample_blocks_workspace_bytes(1024, fan3, 3, 2) == 0
 
 
+def test_seed_loader_host_side():
+    # what SeedLoader does before any GPU work: batch counts, the options it takes from upstream's
+    # DataLoader call (single_node/chunktensor.py:123-132) and the ones it refuses
+    import torch
+    pkg = load_pkg()
+
+    class NoSampler:
+        fused = True
+
+    ids = torch.arange(1050)
+    loader = pkg.SeedLoader(None, ids, NoSampler(), device=None, batch_size=100, shuffle=True, drop_last=False,
+                            num_workers=0, use_ddp=True, use_uva=True)
+    assert len(loader) == 11 and sorted(b.numel() for b in loader._batches()) == [50] + [100] * 10
+    assert len(pkg.SeedLoader(None, ids, NoSampler(), batch_size=100, drop_last=True)) == 10
+    assert len(pkg.SeedLoader(None, ids[:0], NoSampler(), batch_size=100)) == 0
+    assert len(pkg.SeedLoader(None, ids[:100], NoSampler(), batch_size=100)) == 1
+    with pytest.raises(TypeError, match="collate"):
+        pkg.SeedLoader(None, ids, NoSampler(), collate_fn=None)
+    with pytest.raises(ValueError, match="num_workers"):
+        pkg.SeedLoader(None, ids, NoSampler(), num_workers=2)
+    with pytest.raises(ValueError):
+        pkg.SeedLoader(None, ids.float(), NoSampler())
+    with pytest.raises(ValueError):
+        pkg.SeedLoader(None, ids, NoSampler(), batch_size=0)
+
+
 def test_placement_host_arithmetic(oracle):
     # the parts of the placement helpers that need no GPU: degree order, capacity <-> rows, hit rate
     import numpy as np

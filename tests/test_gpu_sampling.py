@@ -1007,3 +1007,52 @@ def test_bucketed_last_hop_near_its_largest_worst_case(pkg, oracle, graph):
             set_last_hop_mode(pkg, LAST_HOP_MODES[0])
         assert np.array_equal(_np(frontier), want_f), mode
         _check_blocks(blocks, want_blocks)
+
+
+def test_seed_loader_stands_in_for_the_dataloader(pkg, oracle, graph):
+    # SeedLoader where upstream's loop has the DGL DataLoader (single_node/chunktensor.py:123-151): batches of
+    # the training ids in order or shuffled, the short last batch kept or dropped, every batch what the
+    # sampler returns for it (held against the oracle), with and without the feature gather, one batch at a
+    # time and in flight, and with a sampler that cannot run fused
+    indptr, indices = graph
+    big = 1 << 40
+    rng = np.random.default_rng(21)
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, big)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, big)
+    feats = rng.standard_normal((20000, 12)).astype(np.float32)
+    x_ct = pkg.create_chunktensor(torch.from_numpy(feats), 1, big, cache_rate=0.5)
+    train = rng.permutation(20000)[:1050].astype(np.int64)
+
+    def check(loader, fanouts, seed, want_batches, with_x):
+        got = list(loader)
+        assert len(got) == len(loader) == len(want_batches)
+        for i, (out, want_seeds) in enumerate(zip(got, want_batches)):
+            assert np.array_equal(_np(out[1]), want_seeds)
+            want_f, _, want_blocks = oracle.sample_blocks(want_seeds, indptr, indices, fanouts, False, seed,
+                                                          len(fanouts) * i)
+            assert np.array_equal(_np(out[0]), want_f)
+            for b, w in zip(out[2], want_blocks):
+                assert np.array_equal(_np(b.src_local), w[0]) and np.array_equal(_np(b.dst_local), w[1])
+            assert len(out) == (4 if with_x else 3)
+            if with_x:
+                assert np.array_equal(_np(out[3]), feats[want_f])
+
+    in_order = [train[i:i + 100] for i in range(0, 1050, 100)]
+    for inflight, fanouts, device in ((3, [5, 4], None), (1, [5, 4], "cuda"), (3, [70, 3], None)):
+        sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct, seed=77)
+        assert sampler.fused == (max(fanouts) <= 64)
+        check(pkg.SeedLoader(None, torch.from_numpy(train), sampler, device=device, batch_size=100, chunk_features=x_ct,
+                             inflight=inflight, use_ddp=True, use_uva=True), fanouts, 77, in_order, True)
+    sampler = pkg.ChunkTensorSampler([5, 4], ip_ct, ix_ct, seed=78)
+    check(pkg.SeedLoader(None, torch.from_numpy(train), sampler, batch_size=100, drop_last=True), [5, 4], 78, in_order[:10], False)
+    # shuffled: every id once per iteration (the tail of 50 dropped), a new order every iteration, the order
+    # that the generator gives
+    sampler = pkg.ChunkTensorSampler([3], ip_ct, ix_ct, seed=79)
+    loader = pkg.SeedLoader(None, torch.from_numpy(train), sampler, device="cuda", batch_size=100, shuffle=True,
+                            drop_last=True, generator=torch.Generator().manual_seed(5))
+    first = torch.cat([out[1] for out in loader]).cpu()
+    second = torch.cat([out[1] for out in loader]).cpu()
+    g = torch.Generator().manual_seed(5)
+    assert torch.equal(first, torch.from_numpy(train)[torch.randperm(1050, generator=g)][:1000])
+    assert torch.equal(second, torch.from_numpy(train)[torch.randperm(1050, generator=g)][:1000])
+    assert not torch.equal(first, second) and first.unique().numel() == 1000
