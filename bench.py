@@ -737,6 +737,21 @@ def main():
     # would see (its DataLoader passes host seeds, its model runs on the current stream)
     ms_handed_over_host_seeds = (1e3 * timed_steps(sampler, batches_cpu, handed_inflight, True)[0] / args.steps
                                  if inflight > 1 else None)
+    # the training loop's own shape: SeedLoader in the place of upstream's DataLoader (host ids in, as
+    # train_idx; batches cut by the loader, each handed to the calling stream with its feature rows)
+    loader_ids = torch.cat(batches_cpu[args.warmup:])
+    loader = dgs.SeedLoader(None, loader_ids, sampler, batch_size=cfg["batch"], chunk_features=ct_feats,
+                            inflight=handed_inflight)
+    ms_seed_loader = None
+    if len(loader) == args.steps:
+        for out in loader:  # untimed: the loader's first iteration
+            sizes(out)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for out in loader:
+            sizes(out)
+        torch.cuda.synchronize()
+        ms_seed_loader = 1e3 * (time.perf_counter() - t0) / len(loader)
     # what an unmodified upstream harness runs: per hop one sampling operator and one relabel
     # operator (each returns tensors of exact length, so each waits for its lengths), then _CAPI_index
     # -- called through torch.ops.dgs_ops with torch as it is, which is what such a harness does
@@ -828,6 +843,7 @@ def main():
         "ms_per_step_handed_over": ms_handed_over,
         "ms_per_step_host_seeds": ms_host_seeds,
         "ms_per_step_handed_over_host_seeds": ms_handed_over_host_seeds,
+        "ms_per_step_seed_loader": ms_seed_loader,
         "ms_per_step_per_hop_ops": ms_per_hop_ops,
         "ms_per_step_per_hop_ops_no_gather": ms_per_hop_ops_no_gather,
         "ms_per_step_per_hop_ops_light_dispatch": ms_per_hop_ops_light,
@@ -837,14 +853,20 @@ def main():
                                                "(at most three batches in flight: the calling stream is a stream too)",
                     "ms_per_step_host_seeds": "as the headline, seeds passed as pageable host tensors",
                     "ms_per_step_handed_over_host_seeds": "host seeds in, each batch handed to the calling stream",
+                    "ms_per_step_seed_loader": "the training loop's own shape: SeedLoader where upstream builds the DGL "
+                                               "DataLoader (host ids in, batches cut by the loader, each handed to the "
+                                               "calling stream with its feature rows)",
                     "ms_per_step_per_hop_ops": "upstream's own loop: _CAPI_sample_neighbors_with_chunk_tensor + "
                                                "_CAPI_tensor_relabel per hop, then _CAPI_index, one batch at a time",
                     "ms_per_step_per_hop_ops_no_gather": "that loop without _CAPI_index: the six operator calls alone",
                     "ms_per_step_per_hop_ops_light_dispatch": "that loop (with _CAPI_index) after "
                                                               "lighten_torch_dispatch(), operators called by their C++ entries",
                     "what_an_unmodified_harness_sees": "ms_per_step_per_hop_ops (one batch at a time through the "
-                                                       "upstream operator names); the headline needs the added "
-                                                       "fused operator and batches in flight"},
+                                                       "upstream operator names); with this package's ChunkTensorSampler "
+                                                       "in the place of upstream's class: ms_per_batch_alone; with "
+                                                       "SeedLoader in the place of the DataLoader as well: "
+                                                       "ms_per_step_seed_loader; the headline leaves each batch on "
+                                                       "its own stream"},
         "sample_edges_per_s": stage_edges / args.steps / (ms_sample * 1e-3),
         "gather_GBps": gather_gbps,
         "ms_sample_relabel": ms_sample,
