@@ -1056,3 +1056,50 @@ def test_seed_loader_stands_in_for_the_dataloader(pkg, oracle, graph):
     assert torch.equal(first, torch.from_numpy(train)[torch.randperm(1050, generator=g)][:1000])
     assert torch.equal(second, torch.from_numpy(train)[torch.randperm(1050, generator=g)][:1000])
     assert not torch.equal(first, second) and first.unique().numel() == 1000
+
+
+def test_hashed_pass_reports_a_bucket_its_table_cannot_hold(pkg, oracle):
+    # The hashed form of the bucketed pass tells a bucket's ids apart in an on-chip table and goes over a
+    # crowded bucket in parts; ids that share bucket AND part beyond the table's slots cannot happen by
+    # chance, but they can be made: 400 distinct neighbour ids whose hash (the library's, restated here)
+    # agrees in the bits that choose the bucket (256 of them for an input this small) and the part (4 for
+    # 400 units and tables of 256 slots).  Every kernel runs to its end, the hop's flag word says so, the
+    # operator raises, and the same call on the node table gives the oracle's answer.  (The pass serves the
+    # last of at least two hops: the first hop here has fanout 0 and leaves the seeds as they are.)
+    def hash_id(ids):
+        h = ids.astype(np.uint32)
+        h ^= h >> np.uint32(16); h *= np.uint32(0x85EBCA6B)
+        h ^= h >> np.uint32(13); h *= np.uint32(0xC2B2AE35)
+        h ^= h >> np.uint32(16)
+        return h
+
+    n = 1 << 21
+    h = hash_id(np.arange(n, dtype=np.int64))
+    crowd = np.flatnonzero(((h & 255) == 0) & ((h >> 23) % 4 == 0))[:400]
+    assert crowd.size == 400
+    seeds = np.flatnonzero((h & 255) != 0)[:40].astype(np.int64)
+    deg = np.zeros(n, dtype=np.int64)
+    deg[seeds] = 10
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    indices = crowd.astype(np.int64)  # row of seed j = crowd[10 j : 10 j + 10], copied whole at fanout 10
+    ip_ct = pkg.create_chunktensor(torch.from_numpy(indptr), 1, 1 << 40)
+    ix_ct = pkg.create_chunktensor(torch.from_numpy(indices), 1, 1 << 40)
+    fanouts = [10, 0]  # model order: hop order is 0, then 10
+    sampler = pkg.ChunkTensorSampler(fanouts, ip_ct, ix_ct)
+    try:
+        set_last_hop_mode(pkg, LAST_HOP_MODES[3])
+        with pytest.raises(RuntimeError, match="crowd"):
+            sampler.sample_blocks(None, _dev(seeds))
+        torch.cuda.synchronize()
+        # half of the crowd fits the tables: the same mode then answers, and answers right
+        want_f, _, want_b = oracle.sample_blocks(seeds[:20], indptr, indices, fanouts, False, 3, 0)
+        pkg.set_rng_state(3, 0)
+        f, _, blocks = sampler.sample_blocks(None, _dev(seeds[:20]))
+        assert np.array_equal(_np(f), want_f) and np.array_equal(_np(blocks[0].src_local), want_b[0][0])
+    finally:
+        set_last_hop_mode(pkg, LAST_HOP_MODES[0])
+    want_f, _, want_b = oracle.sample_blocks(seeds, indptr, indices, fanouts, False, 3, 0)
+    pkg.set_rng_state(3, 0)
+    f, _, blocks = sampler.sample_blocks(None, _dev(seeds))
+    assert np.array_equal(_np(f), want_f) and np.array_equal(_np(blocks[0].src_local), want_b[0][0])
+    assert np.array_equal(_np(blocks[0].dst_local), want_b[0][1])
