@@ -406,11 +406,7 @@ def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8
     if inflight > 1:  # the allocator's per-stream pools see every buffer size before anything is timed
         run_batches(sampler, (seeds * 4)[:4 * inflight + warmup], ct_x, inflight)
     torch.cuda.synchronize()
-    frontiers = []  # the first few, for the gather leg below; of the other batches only the lengths are kept
-
-    def keep(r):
-        if len(frontiers) < stage_batches:
-            frontiers.append(r[0])
+    def keep(r):  # of a timed batch only the lengths are kept: every buffer goes back to its stream's pool at once
         return {"frontier": r[0].numel(),
                 "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]}
     resident = torch.cuda.memory_allocated()
@@ -447,6 +443,7 @@ def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8
     n_stage = min(steps, stage_batches)
     sample_ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(n_stage)]
     stage_stats = []
+    frontiers = []
     sampler.sample_blocks(None, seeds[0])
     torch.cuda.synchronize()
     for i in range(n_stage):
@@ -455,6 +452,7 @@ def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8
         sample_ev[i][1].record()
         stage_stats.append({"frontier": r[0].numel(),
                             "hops": [(b.num_dst, b.src_local.numel(), b.num_src) for b in reversed(r[2])]})
+        frontiers.append(r[0].clone())  # for the gather leg below (a copy: the batch's own block goes back to the pool)
         del r
     torch.cuda.synchronize()
     ms_sample = float(np.mean([a.elapsed_time(b) for a, b in sample_ev]))
@@ -506,7 +504,7 @@ def measure_large(name, dgs, steps, warmup, inflight, scale=1.0, stage_batches=8
              "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes": (bs + bu + bg) / steps,
              "avg_us": 1e6 * elapsed / steps},
         ],
-        # torch allocations of the batches in flight at their peak (outputs, workspaces, kept frontiers),
+        # torch allocations of the batches in flight at their peak (outputs, workspaces),
         # beyond what was resident before the timed loop; the stores themselves are not torch memory
         "peak_batch_bytes": peak_batch_bytes,
         "gather_buffer_cap_bytes": int(torch.ops.dgs_ops._CAPI_get_gather_buffer_cap()),
