@@ -71,13 +71,20 @@ constexpr int64_t kInlineTiles = 2048;         // above this a separate scan lau
 // graph deduplicates heavily).  Grids are capped and blocks stride over the virtual block index,
 // so a mostly empty worst case costs a few loop trips instead of 10^5 empty blocks.
 constexpr int64_t kGridCap = 16384;
+// A launch that loops anyway is given fewer blocks than the cap: its worst case is far beyond the
+// work, and blocks that find none still take a slot each from whatever else shares the GPU
+// (measured with batches in flight, 1024 / 2048 / 4096 / 16384 blocks: 111 M-node graph 0.169-0.180 /
+// 0.167-0.178 / 0.165-0.169 / 0.183-0.187 ms per step, R-MAT [50,50] 0.342-0.352 / 0.345-0.356 /
+// 0.343-0.353 / 0.357-0.361; a batch alone is level or 2 % faster).
+constexpr int64_t kLoopGrid = 4096;
 inline int64_t grid_cap() {
   const int64_t forced = debug_option(DGS_DEBUG_SAMPLER_GRID_CAP);
   return forced > 0 ? forced : kGridCap;
 }
 inline uint32_t capped_grid(int64_t virtual_blocks) {
   const int64_t cap = grid_cap();
-  return uint32_t(virtual_blocks < 1 ? 1 : (virtual_blocks > cap ? cap : virtual_blocks));
+  if (virtual_blocks <= cap) return uint32_t(virtual_blocks < 1 ? 1 : virtual_blocks);
+  return uint32_t(cap < kLoopGrid ? cap : kLoopGrid);  // (a forced cap below kLoopGrid is the grid itself)
 }
 inline bool is_capped(int64_t virtual_blocks) { return virtual_blocks > grid_cap(); }
 // Kernels come in two flavours: STRIDE = false runs exactly one virtual block per block (the
