@@ -780,7 +780,7 @@ def main():
         events[i][0].record()
         r = sampler.sample_blocks(None, batches[args.warmup + i])
         events[i][1].record()
-        frontiers.append(r[0])
+        frontiers.append(r[0].clone())  # a copy, outside the events: the batch's own block goes back to the pool
         stage_stats.append(sizes(r))
         widest_hop_seeds = r[2][0].dst_ids
     del r
