@@ -57,6 +57,8 @@ SIGNATURES = {
     "dgs_current_allocated": (c_i64, []),
     "dgs_gather_rows": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i32, c_vp, c_vp]),
     "dgs_gather_rows_dyn": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i32, c_vp, c_vp]),
+    "dgs_gather_rows_dyn_shared": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i32, c_i32, c_vp,
+                                                  c_vp]),
     "dgs_split_index_workspace_bytes": (c_sz, [c_i64]),
     "dgs_split_index": (ctypes.c_int, [View, c_i64, c_vp, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "dgs_sample_workspace_bytes": (c_sz, [c_i64]),

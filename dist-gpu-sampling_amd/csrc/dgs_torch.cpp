@@ -805,10 +805,16 @@ class PendingBlocks : public torch::CustomClassHolder {
         // bytes, a launch of exactly the right size 113 us, of half the size 114, with a quarter
         // more blocks than needed 116, at the 32768-block cap 118)
         const int64_t last = indptr->frontier_hint();
-        p->gather_status_ = dgs_gather_rows_dyn(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
-                                                buffer_rows, sizes_dev.data_ptr<int64_t>() + hops,
-                                                last, p->x_.data_ptr(), DGS_TIER_ANY,
-                                                features->bad_index_word(), st);
+        // Weighted fills are bound by vector arithmetic and need wave slots beside other batches'
+        // gathers, which by themselves take every slot of a CU: such a batch's gather keeps half of
+        // them (measured with four weighted batches in flight, 8 / 5 / 4 / 3 blocks per CU: 0.2165 /
+        // 0.197 / 0.193 / 0.205 ms per step; the uniform sampler's kernels wait for memory, and its
+        // steps are 9 % slower at 5 and 4)
+        const int32_t gather_blocks_per_cu = probs ? 4 : 0;
+        p->gather_status_ = dgs_gather_rows_dyn_shared(features->view(), features->elem_stride(), p->all_.data_ptr(), w,
+                                                       buffer_rows, sizes_dev.data_ptr<int64_t>() + hops, last,
+                                                       p->x_.data_ptr(), DGS_TIER_ANY, gather_blocks_per_cu,
+                                                       features->bad_index_word(), st);
       }
     }
     // the batch's one ticket, behind its last launch: it bounds the wait for the lengths, tells the

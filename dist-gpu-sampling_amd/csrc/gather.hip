@@ -24,6 +24,20 @@ constexpr uint32_t kMaxFlatChunksPerRow = 32768;
 // A launch sized for a worst-case row count (dgs_gather_rows_dyn) is capped at this many blocks;
 // blocks stride over the tiles, so a mostly unused worst case does not cost 10^5 empty blocks.
 constexpr int64_t kMaxDynGrid = 32768;
+constexpr int kGatherBlocksPerCu = 8;  // what fits by registers and wave slots when nothing is reserved
+
+// LDS of one CU on the current device (160 KB on gfx950); asked once per process.
+inline int64_t lds_per_cu() {
+  static const int64_t bytes = [] {
+    int dev = 0, per_cu = 0, per_block = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return int64_t(65536);
+    if (hipDeviceGetAttribute(&per_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess) per_cu = 0;
+    if (hipDeviceGetAttribute(&per_block, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) per_block = 0;
+    const int64_t most = per_cu > per_block ? per_cu : per_block;
+    return most > 0 ? most : int64_t(65536);
+  }();
+  return bytes;
+}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -171,7 +185,7 @@ __global__ __launch_bounds__(kGatherThreads) void gather_wide_kernel(
 
 template <int VEC, int TIER, typename IndexT>
 dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index, int64_t n,
-                         const int64_t* n_dev, int64_t n_expected, int64_t* bad_index, void* out, hipStream_t st) {
+                         const int64_t* n_dev, int64_t n_expected, int32_t blocks_per_cu, int64_t* bad_index, void* out, hipStream_t st) {
   const int64_t cpr = row_bytes / VEC;
   const int64_t thr_bytes = v.threshold * v.elem_bytes;
   // rows the tier holds whole: the device tier the rows that end at or before the boundary, the
@@ -194,7 +208,10 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
     }
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;
     const uint32_t magic = cpr > 1 ? uint32_t((uint64_t(1) << 32) / uint64_t(cpr)) + 1u : 0u;
+    // LDS that the kernel does not use, reserved so that fewer of its blocks fit a CU: a caller's
+    // limit (dgs_gather_rows_dyn_shared), or the measurement hook's byte count
     int64_t lds = debug_option(DGS_DEBUG_GATHER_LDS_BYTES);
+    if (lds <= 0 && blocks_per_cu > 0 && blocks_per_cu < kGatherBlocksPerCu) lds = lds_per_cu() / blocks_per_cu / 256 * 256;
     lds = lds < 0 ? 0 : (lds > 65536 ? 65536 : lds);
     if (blocks < tiles)
       hipLaunchKernelGGL((gather_flat_kernel<VEC, TIER, IndexT, true>), dim3(uint32_t(blocks)),
@@ -221,22 +238,22 @@ dgs_status launch_gather(const dgs_view& v, int64_t row_bytes, const void* index
 
 template <int VEC, int TIER>
 dgs_status dispatch_index(const dgs_view& v, int64_t row_bytes, const void* index,
-                          int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t n_expected, int64_t* bad,
+                          int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t n_expected, int32_t blocks_per_cu, int64_t* bad,
                           void* out, hipStream_t st) {
-  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, n_expected, bad, out, st)
-                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, n_expected, bad, out, st);
+  return index_bytes == 8 ? launch_gather<VEC, TIER, int64_t>(v, row_bytes, index, n, n_dev, n_expected, blocks_per_cu, bad, out, st)
+                          : launch_gather<VEC, TIER, int32_t>(v, row_bytes, index, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
 }
 
 template <int TIER>
 dgs_status dispatch_vec(int vec, const dgs_view& v, int64_t row_bytes, const void* index,
-                        int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t n_expected, int64_t* bad,
+                        int32_t index_bytes, int64_t n, const int64_t* n_dev, int64_t n_expected, int32_t blocks_per_cu, int64_t* bad,
                         void* out, hipStream_t st) {
   switch (vec) {
-    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
-    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
-    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
-    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
-    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    case 16: return dispatch_index<16, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
+    case 8: return dispatch_index<8, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
+    case 4: return dispatch_index<4, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
+    case 2: return dispatch_index<2, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
+    default: return dispatch_index<1, TIER>(v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
   }
 }
 
@@ -337,7 +354,7 @@ __global__ __launch_bounds__(kSplitThreads) void split_scatter_kernel(
 
 namespace {
 dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_t index_bytes, int64_t n,
-                        const int64_t* n_dev, int64_t n_expected, void* out, int32_t tier, int64_t* bad,
+                        const int64_t* n_dev, int64_t n_expected, int32_t blocks_per_cu, void* out, int32_t tier, int64_t* bad,
                         void* stream) {
   using namespace dgs;
   DGS_REQUIRE(width_ok(index_bytes), DGS_ERR_INVALID, "gather: index width %d is not 4 or 8", index_bytes);
@@ -362,9 +379,9 @@ dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_
   const int vec = pick_vec(v, row_bytes, out, tier);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (tier) {
-    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
-    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
-    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, bad, out, st);
+    case DGS_TIER_DEVICE: return dispatch_vec<DGS_TIER_DEVICE>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
+    case DGS_TIER_HOST: return dispatch_vec<DGS_TIER_HOST>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
+    default: return dispatch_vec<DGS_TIER_ANY>(vec, v, row_bytes, index, index_bytes, n, n_dev, n_expected, blocks_per_cu, bad, out, st);
   }
 }
 }  // namespace
@@ -372,7 +389,7 @@ dgs_status gather_entry(dgs_view v, int64_t row_elems, const void* index, int32_
 DGS_API dgs_status dgs_gather_rows(dgs_view v, int64_t row_elems, const void* index,
                                    int32_t index_bytes, int64_t n, void* out, int32_t tier,
                                    int64_t* bad_index, void* stream) {
-  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, 0, out, tier, bad_index, stream);
+  return gather_entry(v, row_elems, index, index_bytes, n, nullptr, 0, 0, out, tier, bad_index, stream);
 }
 
 DGS_API dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
@@ -380,7 +397,17 @@ DGS_API dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void
                                        int64_t n_expected, void* out, int32_t tier, int64_t* bad_index,
                                        void* stream) {
   DGS_REQUIRE(n_rows_dev != nullptr, DGS_ERR_INVALID, "gather_dyn: null n_rows_dev");
-  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, n_expected, out, tier, bad_index, stream);
+  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, n_expected, 0, out, tier, bad_index, stream);
+}
+
+DGS_API dgs_status dgs_gather_rows_dyn_shared(dgs_view v, int64_t row_elems, const void* index,
+                                              int32_t index_bytes, int64_t n_max, const int64_t* n_rows_dev,
+                                              int64_t n_expected, void* out, int32_t tier, int32_t blocks_per_cu,
+                                              int64_t* bad_index, void* stream) {
+  DGS_REQUIRE(n_rows_dev != nullptr, DGS_ERR_INVALID, "gather_dyn_shared: null n_rows_dev");
+  DGS_REQUIRE(blocks_per_cu >= 0, DGS_ERR_INVALID, "gather_dyn_shared: blocks_per_cu %d", blocks_per_cu);
+  return gather_entry(v, row_elems, index, index_bytes, n_max, n_rows_dev, n_expected, blocks_per_cu, out, tier, bad_index,
+                      stream);
 }
 
 DGS_API size_t dgs_split_index_workspace_bytes(int64_t n) {

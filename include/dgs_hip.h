@@ -201,6 +201,21 @@ dgs_status dgs_gather_rows_dyn(dgs_view v, int64_t row_elems, const void* index,
                                int32_t tier, int64_t* bad_index, void* stream);
 
 /*
+ * dgs_gather_rows_dyn for a gather that shares the GPU with other streams' kernels which need
+ * wave slots more than memory bandwidth (the weighted sampler's fills are bound by vector
+ * arithmetic): at most `blocks_per_cu` of the gather's 256-thread blocks are resident on a CU at
+ * a time (3..7; 0, or 8 and more: all that fit, as dgs_gather_rows_dyn).  The kernel reserves
+ * on-chip memory it does not use, nothing else changes; results are those of dgs_gather_rows_dyn.
+ * By itself the gather loses about 1.5 % at 4 blocks per CU and 4 % at 3; a step of weighted
+ * batches in flight gains 11 % at 4.  No counterpart in the reference.
+ */
+dgs_status dgs_gather_rows_dyn_shared(dgs_view v, int64_t row_elems, const void* index,
+                                      int32_t index_bytes, int64_t n_max,
+                                      const int64_t* n_rows_dev, int64_t n_expected, void* out,
+                                      int32_t tier, int32_t blocks_per_cu, int64_t* bad_index,
+                                      void* stream);
+
+/*
  * Stable partition of an index list into (device-resident rows, host-resident
  * rows): row r is "host" iff r >= threshold / row_elems
  * (src/cuda/index_with_chunk_tensor.cu:55-108; the "remote" class is empty at

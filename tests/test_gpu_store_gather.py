@@ -323,6 +323,17 @@ def test_gather_dyn_with_more_rows_than_expected(pkg, dtype, dim):
                                                     out.data_ptr(), capi.TIER_ANY, bad.data_ptr(), capi.stream_ptr()))
             assert torch.equal(out[:count].cpu(), full[idx[:count].cpu().long()]), (count, expected)
             assert (out[count:] == -3.0).all().item() and bad.item() == 0, (count, expected)
+        # the same gather with fewer of its blocks on a CU at a time (for callers that share the GPU with
+        # compute-bound kernels): the same rows, whatever the limit
+        for blocks_per_cu in (0, 1, 3, 4, 7, 8, 1000):
+            out.fill_(-3.0)
+            capi.check(capi.lib.dgs_gather_rows_dyn_shared(view, dim, tail.data_ptr(), 4, n_max, n_dev.data_ptr(), count,
+                                                           out.data_ptr(), capi.TIER_ANY, blocks_per_cu, bad.data_ptr(),
+                                                           capi.stream_ptr()))
+            assert torch.equal(out[:count].cpu(), full[idx[:count].cpu().long()]), (count, blocks_per_cu)
+            assert (out[count:] == -3.0).all().item() and bad.item() == 0, (count, blocks_per_cu)
+    assert capi.lib.dgs_gather_rows_dyn_shared(view, dim, idx.data_ptr(), 4, n_max, n_dev.data_ptr(), 0, out.data_ptr(),
+                                               capi.TIER_ANY, -1, None, capi.stream_ptr()) == capi.DGS_ERR_INVALID
     tail = idx.clone()
     tail[17] = rows  # one past the last row, inside the count
     n_dev = torch.tensor([100], dtype=torch.int64, device="cuda")
