@@ -637,7 +637,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="with --workload c1: do not also run c1w, c2, c4 and c3 after the headline")
-    ap.add_argument("--other-steps", type=int, default=20, help="timed batches of each other workload")
+    ap.add_argument("--other-steps", type=int, default=40, help="timed batches of each other workload")
     ap.add_argument("--other-budget-s", type=float, default=300.0,
                     help="no further workload is started once this much time has gone into them")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0)
